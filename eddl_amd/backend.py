@@ -1,0 +1,223 @@
+"""ctypes binding of the C ABI: device tensors and one method per operator.
+
+Every method launches asynchronously on the device's stream; ``DeviceTensor.numpy()`` and
+``Backend.synchronize()`` wait.  Shapes follow the reference: NCHW activations, OIHW filters,
+[in, out] dense weights, all float32.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+
+
+class EddlHipError(RuntimeError):
+    """A C ABI call returned a negative code; the text is eddlhip_last_error()."""
+
+
+class DeviceTensor:
+    """A float32 tensor in HBM owned by this object (freed when collected)."""
+
+    def __init__(self, backend, shape):
+        self.backend = backend
+        self.shape = tuple(int(d) for d in shape)
+        self.size = int(np.prod(self.shape)) if len(self.shape) else 1
+        self.nbytes = self.size * 4
+        self.ptr = backend._malloc(self.nbytes)
+
+    def __del__(self):
+        try:
+            if getattr(self, "ptr", None):
+                self.backend._free(self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+    def numpy(self):
+        out = np.empty(self.shape, np.float32)
+        self.backend._check(self.backend.lib.eddlhip_memcpy_d2h(self.backend.dev, out.ctypes.data, self.ptr, self.nbytes))
+        return out
+
+    def copy_from(self, host):
+        host = np.ascontiguousarray(host, dtype=np.float32)
+        if host.size != self.size:
+            raise ValueError("size mismatch: %s vs %s" % (host.shape, self.shape))
+        self.backend._check(self.backend.lib.eddlhip_memcpy_h2d(self.backend.dev, self.ptr, host.ctypes.data, self.nbytes))
+        return self
+
+    def reshape(self, shape):
+        """A view with another shape sharing the storage (the reference's reshape_)."""
+        view = object.__new__(DeviceTensor)
+        view.backend, view.ptr, view.nbytes, view.size = self.backend, self.ptr, self.nbytes, self.size
+        view.shape = tuple(int(d) for d in shape)
+        if int(np.prod(view.shape)) != self.size:
+            raise ValueError("reshape changes the size")
+        view._base = self  # keeps the owner alive
+        view.__class__ = _View
+        return view
+
+
+class _View(DeviceTensor):
+    def __del__(self):  # storage belongs to the base tensor
+        pass
+
+
+class Event:
+    def __init__(self, backend):
+        self.backend = backend
+        h = ctypes.c_void_p()
+        backend._check(backend.lib.eddlhip_event_create(backend.dev, ctypes.byref(h)))
+        self.handle = h
+
+    def record(self):
+        self.backend._check(self.backend.lib.eddlhip_event_record(self.backend.dev, self.handle))
+        return self
+
+    def elapsed_ms(self, stop):
+        ms = ctypes.c_float()
+        self.backend._check(self.backend.lib.eddlhip_event_elapsed_ms(self.backend.dev, self.handle, stop.handle, ctypes.byref(ms)))
+        return ms.value
+
+    def __del__(self):
+        try:
+            self.backend.lib.eddlhip_event_destroy(self.backend.dev, self.handle)
+        except Exception:
+            pass
+
+
+def _ptr(t):
+    return None if t is None else t.ptr
+
+
+class Backend:
+    """One device of libeddlhip.so."""
+
+    def __init__(self, dev=0):
+        self.lib = _lib.load()
+        self.dev = int(dev)
+        self._check(self.lib.eddlhip_init(self.dev))
+
+    # ---- plumbing
+    def _check(self, rc):
+        if rc != 0:
+            raise EddlHipError("%s (code %d)" % (self.lib.eddlhip_last_error().decode(), rc))
+
+    def _malloc(self, nbytes):
+        p = ctypes.c_void_p()
+        self._check(self.lib.eddlhip_malloc(self.dev, max(nbytes, 4), ctypes.byref(p)))
+        return p.value
+
+    def _free(self, ptr):
+        self.lib.eddlhip_free(self.dev, ptr)
+
+    @property
+    def name(self):
+        buf = ctypes.create_string_buffer(256)
+        self._check(self.lib.eddlhip_device_name(self.dev, buf, 256))
+        return buf.value.decode()
+
+    def synchronize(self):
+        self._check(self.lib.eddlhip_synchronize(self.dev))
+
+    def event(self):
+        return Event(self)
+
+    def empty(self, shape):
+        return DeviceTensor(self, shape)
+
+    def array(self, host):
+        host = np.ascontiguousarray(host, dtype=np.float32)
+        return DeviceTensor(self, host.shape).copy_from(host)
+
+    def full(self, shape, v):
+        t = DeviceTensor(self, shape)
+        self.fill_(t, v)
+        return t
+
+    def set_conv_algo(self, algo):
+        self._check(self.lib.eddlhip_conv2d_set_algo({"auto": 0, "mfma": 1, "direct": 2}.get(algo, algo)))
+
+    # ---- operators (names follow the reference's gpu_* functions)
+    def fill_(self, A, v):
+        self._check(self.lib.eddlhip_fill(self.dev, A.ptr, A.size, v))
+
+    def conv2D(self, I, K, bias, O, sr, sc, padrt, padcl, bn=None, residual=None, relu=False):
+        """``bn`` = (g, b, mean, var, eps) device tensors (g, b may be None) or None."""
+        N, C, H, W = I.shape
+        Kf, C2, R, S = K.shape
+        if C2 != C:
+            raise ValueError("filter depth %d != input channels %d" % (C2, C))
+        if O.shape[0] != N or O.shape[1] != Kf:
+            raise ValueError("output shape %s does not match" % (O.shape,))
+        g = b = mean = var = None
+        eps = 0.0
+        if bn is not None:
+            g, b, mean, var, eps = bn
+        self._check(self.lib.eddlhip_conv2d_fwd(self.dev, I.ptr, K.ptr, _ptr(bias), O.ptr, N, C, H, W, Kf, R, S, sr, sc, padrt,
+                                                padcl, O.shape[2], O.shape[3], _ptr(g), _ptr(b), _ptr(mean), _ptr(var), eps,
+                                                _ptr(residual), int(relu)))
+
+    def batchnorm_inference(self, x, y, opa, gmean, gvar, g, b, variance, eps):
+        N, C = x.shape[0], x.shape[1]
+        rc = x.size // (N * C) if N * C else 1
+        self._check(self.lib.eddlhip_batchnorm_inference(self.dev, N, C, rc, x.ptr, y.ptr, _ptr(opa), gmean.ptr, gvar.ptr, _ptr(g),
+                                                         _ptr(b), variance.ptr, eps))
+
+    def relu(self, A, B):
+        self._check(self.lib.eddlhip_relu(self.dev, A.ptr, B.ptr, A.size))
+
+    def sigmoid(self, A, B):
+        self._check(self.lib.eddlhip_sigmoid(self.dev, A.ptr, B.ptr, A.size))
+
+    def full_softmax(self, A, B, axis, stable=True):
+        outer = int(np.prod(A.shape[:axis])) if axis > 0 else 1
+        inner = int(np.prod(A.shape[axis + 1:])) if axis + 1 < len(A.shape) else 1
+        self._check(self.lib.eddlhip_softmax(self.dev, A.ptr, B.ptr, outer, A.shape[axis], inner, int(stable)))
+
+    def pool_out_dims(self, H, W, k, stride, pads):
+        lp, lq = ctypes.c_int(), ctypes.c_int()
+        self._check(self.lib.eddlhip_pool2d_out_dims(H, W, k[0], k[1], stride[0], stride[1], *pads, ctypes.byref(lp), ctypes.byref(lq)))
+        return lp.value, lq.value
+
+    def mpool2D(self, I, O, indX, indY, k, stride, pads):
+        N, C, H, W = I.shape
+        self._check(self.lib.eddlhip_maxpool2d(self.dev, I.ptr, O.ptr, indX.ptr, indY.ptr, N, C, H, W, k[0], k[1], stride[0],
+                                               stride[1], *pads))
+
+    def avgpool2D(self, I, O, k, stride, pads):
+        N, C, H, W = I.shape
+        self._check(self.lib.eddlhip_avgpool2d(self.dev, I.ptr, O.ptr, N, C, H, W, k[0], k[1], stride[0], stride[1], *pads))
+
+    def scale(self, A, B, new_shape):
+        N, C, H, W = A.shape
+        self._check(self.lib.eddlhip_scale_nearest(self.dev, A.ptr, B.ptr, N, C, H, W, B.shape[2], B.shape[3], new_shape[0],
+                                                   new_shape[1]))
+
+    def concat(self, out, ts, axis):
+        outer = int(np.prod(out.shape[:axis])) if axis > 0 else 1
+        inner = int(np.prod(out.shape[axis + 1:])) if axis + 1 < len(out.shape) else 1
+        ptrs = (ctypes.c_void_p * len(ts))(*[t.ptr for t in ts])
+        ext = (ctypes.c_int * len(ts))(*[t.shape[axis] for t in ts])
+        if sum(t.shape[axis] for t in ts) != out.shape[axis]:
+            raise ValueError("The dimension of the output tensor is incorrect")
+        self._check(self.lib.eddlhip_concat(self.dev, out.ptr, ptrs, ext, len(ts), outer, inner))
+
+    def add(self, scA, A, scB, B, C, incC=0):
+        self._check(self.lib.eddlhip_add(self.dev, scA, A.ptr, scB, B.ptr, C.ptr, incC, A.size))
+
+    def inc(self, A, B):
+        self._check(self.lib.eddlhip_inc(self.dev, A.ptr, B.ptr, A.size))
+
+    def pad(self, A, B, pads):
+        N, C, H, W = A.shape
+        self._check(self.lib.eddlhip_pad(self.dev, A.ptr, B.ptr, N, C, H, W, *pads))
+
+    def mult2D(self, A, B, C, incC=0):
+        m, k = A.shape
+        k2, n = B.shape
+        if k != k2 or C.shape != (m, n):
+            raise ValueError("mult2D shapes %s x %s -> %s" % (A.shape, B.shape, C.shape))
+        self._check(self.lib.eddlhip_mult2d(self.dev, A.ptr, B.ptr, C.ptr, m, k, n, incC))
+
+    def sum2D_rowwise(self, A, B, C):
+        self._check(self.lib.eddlhip_sum2d_rowwise(self.dev, A.ptr, B.ptr, C.ptr, A.shape[0], A.shape[1]))

@@ -1,0 +1,59 @@
+// Shared state and helpers of libeddlhip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/eddlhip.h"
+
+#define EDDLHIP_MAX_DEVICES 16
+#define EDDLHIP_NUM_XCD 8  // MI355X: 256 CUs in 8 XCDs, workgroups are dealt to XCDs round-robin
+
+namespace eddlhip {
+
+struct DeviceState {
+    bool inited = false;
+    hipStream_t stream = nullptr;  // null stream unless the caller installed its own
+    int num_cu = 0;
+    void *workspace = nullptr;  // private, grow-only (repacked filters, split-K partials)
+    size_t workspace_bytes = 0;
+    void *flag = nullptr;  // one int of device memory for kernels that report a condition
+};
+
+DeviceState &state(int dev);
+int set_error(int code, const char *fmt, ...);
+// Makes `dev` current and initialises it on first use.
+int use_device(int dev);
+// Returns a workspace of at least `bytes` (contents undefined); waits for the stream before
+// replacing a smaller one so that kernels still reading it finish first.
+int get_workspace(int dev, size_t bytes, void **ptr);
+
+}  // namespace eddlhip
+
+#define EH_TRY_HIP(expr)                                                                          \
+    do {                                                                                          \
+        hipError_t _e = (expr);                                                                   \
+        if (_e != hipSuccess)                                                                     \
+            return eddlhip::set_error(EDDLHIP_EHIP, "%s: %s (%s:%d)", #expr, hipGetErrorString(_e), \
+                                      __FILE__, __LINE__);                                        \
+    } while (0)
+
+#define EH_TRY(expr)          \
+    do {                      \
+        int _r = (expr);      \
+        if (_r != 0) return _r; \
+    } while (0)
+
+#define EH_REQUIRE(cond, ...)                                            \
+    do {                                                                 \
+        if (!(cond)) return eddlhip::set_error(EDDLHIP_EINVAL, __VA_ARGS__); \
+    } while (0)
+
+#define EH_CHECK_LAUNCH() EH_TRY_HIP(hipGetLastError())
+
+static inline unsigned eh_blocks(size_t work, unsigned per_block, unsigned cap = 1u << 20) {
+    size_t b = (work + per_block - 1) / per_block;
+    if (b < 1) b = 1;
+    if (b > cap) b = cap;
+    return (unsigned)b;
+}

@@ -1,0 +1,254 @@
+// MaxPool2D (with argmax) and AvgPool2D forward.  Semantics of the reference's CPU loops
+// (src/hardware/cpu/nn/cpu_pool.cpp:74-121 and :226-274): window origins step from -pad,
+// taps scanned ky then kx, strict '>' so the first maximum wins, indices are absolute input
+// coordinates stored as floats, average divides by kr*kc whatever the padding.
+//
+// Two kernels per operator:
+//   * small windows: one thread per output, neighbouring lanes on neighbouring outputs so
+//     loads and the three stores are coalesced; a 2x2/stride-2 fast path reads two input
+//     rows as float4 and produces two outputs per thread;
+//   * large windows (>= 64 taps, e.g. global pooling): one wavefront per output, lanes
+//     stride over the taps in scan order and a wavefront (max, tap-index) reduction picks the
+//     winner; ties go to the lower tap index, which is the first maximum of the scan.
+#include "common.h"
+
+using namespace eddlhip;
+
+namespace {
+
+constexpr int TPB = 256;
+constexpr float LOWEST = -3.40282e+38f;  // the reference's running-maximum start value
+
+struct PoolShape {
+    int C, H, W, kr, kc, sr, sc, pt, pl, LP, LQ;
+};
+
+__global__ __launch_bounds__(TPB) void maxpool_kernel(const float *__restrict__ I, float *__restrict__ O,
+                                                      float *__restrict__ indX, float *__restrict__ indY, size_t total,
+                                                      PoolShape s) {
+    size_t t0 = (size_t)blockIdx.x * TPB + threadIdx.x, stride = (size_t)gridDim.x * TPB;
+    for (size_t p = t0; p < total; p += stride) {
+        int oj = (int)(p % s.LQ);
+        size_t r = p / s.LQ;
+        int oi = (int)(r % s.LP);
+        size_t plane = r / s.LP;  // b*C + k
+        const float *img = I + plane * s.H * s.W;
+        const int i = oi * s.sr - s.pt, j = oj * s.sc - s.pl;
+        float mx = LOWEST;
+        int bx = 0, by = 0;
+        bool found = false;
+        for (int ki = 0; ki < s.kr; ki++) {
+            int py = i + ki;
+            if (py < 0 || py >= s.H) continue;  // out-of-image taps read -FLT_MAX and never win
+            for (int kj = 0; kj < s.kc; kj++) {
+                int px = j + kj;
+                if (px < 0 || px >= s.W) continue;
+                float v = img[(size_t)py * s.W + px];
+                if (v > mx) {
+                    mx = v;
+                    bx = px;
+                    by = py;
+                    found = true;
+                }
+            }
+        }
+        O[p] = mx;
+        if (found) {
+            indX[p] = (float)bx;
+            indY[p] = (float)by;
+        }
+    }
+}
+
+// 2x2 window, stride 2, no padding, even W, 16-byte aligned rows: each thread reads a float4
+// from two consecutive input rows and writes two outputs (float2 stores).
+__global__ __launch_bounds__(TPB) void maxpool_2x2s2_kernel(const float *__restrict__ I, float *__restrict__ O,
+                                                            float *__restrict__ indX, float *__restrict__ indY,
+                                                            size_t total_pairs, int H, int W, int LP, int LQ) {
+    const int LQ2 = LQ / 2;
+    size_t t0 = (size_t)blockIdx.x * TPB + threadIdx.x, stride = (size_t)gridDim.x * TPB;
+    for (size_t t = t0; t < total_pairs; t += stride) {
+        int oj2 = (int)(t % LQ2);
+        size_t r = t / LQ2;
+        int oi = (int)(r % LP);
+        size_t plane = r / LP;
+        const float *row0 = I + (plane * H + 2 * oi) * W + 4 * oj2;
+        float4 a = *reinterpret_cast<const float4 *>(row0);
+        float4 b = *reinterpret_cast<const float4 *>(row0 + W);
+        float2 o, ix, iy;
+        const float x0 = (float)(4 * oj2), y0 = (float)(2 * oi);
+        {
+            float mx = LOWEST;
+            float fx = 0.f, fy = 0.f;
+            bool found = false;
+            if (a.x > mx) { mx = a.x; fx = x0; fy = y0; found = true; }
+            if (a.y > mx) { mx = a.y; fx = x0 + 1.f; fy = y0; found = true; }
+            if (b.x > mx) { mx = b.x; fx = x0; fy = y0 + 1.f; found = true; }
+            if (b.y > mx) { mx = b.y; fx = x0 + 1.f; fy = y0 + 1.f; found = true; }
+            o.x = mx;
+            size_t p = (plane * LP + oi) * LQ + 2 * oj2;
+            if (!found) { fx = indX[p]; fy = indY[p]; }
+            ix.x = fx; iy.x = fy;
+        }
+        {
+            float mx = LOWEST;
+            float fx = 0.f, fy = 0.f;
+            bool found = false;
+            if (a.z > mx) { mx = a.z; fx = x0 + 2.f; fy = y0; found = true; }
+            if (a.w > mx) { mx = a.w; fx = x0 + 3.f; fy = y0; found = true; }
+            if (b.z > mx) { mx = b.z; fx = x0 + 2.f; fy = y0 + 1.f; found = true; }
+            if (b.w > mx) { mx = b.w; fx = x0 + 3.f; fy = y0 + 1.f; found = true; }
+            o.y = mx;
+            size_t p = (plane * LP + oi) * LQ + 2 * oj2 + 1;
+            if (!found) { fx = indX[p]; fy = indY[p]; }
+            ix.y = fx; iy.y = fy;
+        }
+        size_t p = (plane * LP + oi) * LQ + 2 * oj2;
+        *reinterpret_cast<float2 *>(O + p) = o;
+        *reinterpret_cast<float2 *>(indX + p) = ix;
+        *reinterpret_cast<float2 *>(indY + p) = iy;
+    }
+}
+
+// One wavefront per output.  Lane l visits taps l, l+64, ... in scan order (tap = ki*kc + kj),
+// keeping its first maximum; the reduction keeps the larger value and, on equal values, the
+// lower tap index.
+__global__ __launch_bounds__(TPB) void maxpool_wave_kernel(const float *__restrict__ I, float *__restrict__ O,
+                                                           float *__restrict__ indX, float *__restrict__ indY, size_t total,
+                                                           PoolShape s) {
+    const int lane = threadIdx.x & 63;
+    const size_t wave = ((size_t)blockIdx.x * TPB + threadIdx.x) >> 6, nwaves = ((size_t)gridDim.x * TPB) >> 6;
+    const int taps = s.kr * s.kc;
+    for (size_t p = wave; p < total; p += nwaves) {
+        int oj = (int)(p % s.LQ);
+        size_t r = p / s.LQ;
+        int oi = (int)(r % s.LP);
+        size_t plane = r / s.LP;
+        const float *img = I + plane * s.H * s.W;
+        const int i = oi * s.sr - s.pt, j = oj * s.sc - s.pl;
+        float mx = LOWEST;
+        int best = 0x7fffffff;  // tap index of the winner; "none" sorts last
+        for (int t = lane; t < taps; t += 64) {
+            int ki = t / s.kc, kj = t - ki * s.kc;
+            int py = i + ki, px = j + kj;
+            if (py < 0 || py >= s.H || px < 0 || px >= s.W) continue;
+            float v = img[(size_t)py * s.W + px];
+            if (v > mx) {
+                mx = v;
+                best = t;
+            }
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            float omx = __shfl_xor(mx, off, 64);
+            int obest = __shfl_xor(best, off, 64);
+            if (omx > mx || (omx == mx && obest < best)) {
+                mx = omx;
+                best = obest;
+            }
+        }
+        if (lane == 0) {
+            O[p] = mx;
+            if (best != 0x7fffffff) {
+                int ki = best / s.kc, kj = best - ki * s.kc;
+                indX[p] = (float)(j + kj);
+                indY[p] = (float)(i + ki);
+            }
+        }
+    }
+}
+
+// Sequential (ky,kx) sum of the in-image taps, one thread per output: bit-exact with the
+// reference's accumulation order for every window size.
+__global__ __launch_bounds__(TPB) void avgpool_kernel(const float *__restrict__ I, float *__restrict__ O, size_t total,
+                                                      PoolShape s) {
+    size_t t0 = (size_t)blockIdx.x * TPB + threadIdx.x, stride = (size_t)gridDim.x * TPB;
+    const float ksize = (float)(s.kr * s.kc);
+    for (size_t p = t0; p < total; p += stride) {
+        int oj = (int)(p % s.LQ);
+        size_t r = p / s.LQ;
+        int oi = (int)(r % s.LP);
+        size_t plane = r / s.LP;
+        const float *img = I + plane * s.H * s.W;
+        const int i = oi * s.sr - s.pt, j = oj * s.sc - s.pl;
+        float sum = 0.0f;
+        for (int ki = 0; ki < s.kr; ki++) {
+            int py = i + ki;
+            if (py < 0 || py >= s.H) continue;
+            for (int kj = 0; kj < s.kc; kj++) {
+                int px = j + kj;
+                if (px < 0 || px >= s.W) continue;
+                sum = __fadd_rn(sum, img[(size_t)py * s.W + px]);
+            }
+        }
+        O[p] = __fdiv_rn(sum, ksize);
+    }
+}
+
+int loop_count(int in, int k, int stride, int pad_lo, int pad_hi) {
+    long long last = (long long)in + pad_hi - k, first = -(long long)pad_lo;
+    if (last < first) return 0;
+    return (int)((last - first) / stride) + 1;
+}
+
+int check_pool(const char *name, int N, int C, int H, int W, int kr, int kc, int sr, int sc, int pt, int pb, int pl, int pr,
+               PoolShape *s) {
+    EH_REQUIRE(N >= 0 && C > 0 && H > 0 && W > 0, "%s: bad input shape", name);
+    EH_REQUIRE(kr > 0 && kc > 0 && sr > 0 && sc > 0, "%s: bad window/stride", name);
+    EH_REQUIRE(pt >= 0 && pb >= 0 && pl >= 0 && pr >= 0, "%s: negative padding", name);
+    *s = PoolShape{C, H, W, kr, kc, sr, sc, pt, pl, loop_count(H, kr, sr, pt, pb), loop_count(W, kc, sc, pl, pr)};
+    EH_REQUIRE((long long)C * H * W <= 0x7fffffffLL, "%s: image too large", name);
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int eddlhip_pool2d_out_dims(int H, int W, int kr, int kc, int sr, int sc, int pad_top, int pad_bottom, int pad_left,
+                            int pad_right, int *LP, int *LQ) {
+    EH_REQUIRE(LP && LQ, "pool2d_out_dims: NULL output");
+    EH_REQUIRE(H > 0 && W > 0 && kr > 0 && kc > 0 && sr > 0 && sc > 0, "pool2d_out_dims: bad shape");
+    *LP = loop_count(H, kr, sr, pad_top, pad_bottom);
+    *LQ = loop_count(W, kc, sc, pad_left, pad_right);
+    return 0;
+}
+
+int eddlhip_maxpool2d(int dev, const float *I, float *O, float *indX, float *indY, int N, int C, int H, int W, int kr, int kc,
+                      int sr, int sc, int pad_top, int pad_bottom, int pad_left, int pad_right) {
+    PoolShape s;
+    EH_TRY(check_pool("maxpool2d", N, C, H, W, kr, kc, sr, sc, pad_top, pad_bottom, pad_left, pad_right, &s));
+    size_t total = (size_t)N * C * s.LP * s.LQ;
+    if (total == 0) return 0;
+    EH_REQUIRE(I && O && indX && indY, "maxpool2d: NULL tensor");
+    EH_TRY(use_device(dev));
+    hipStream_t st = state(dev).stream;
+    auto al = [](const void *p, unsigned a) { return ((uintptr_t)p & (a - 1)) == 0; };
+    if (kr == 2 && kc == 2 && sr == 2 && sc == 2 && !pad_top && !pad_left && !pad_bottom && !pad_right && W % 4 == 0 &&
+        al(I, 16) && al(O, 8) && al(indX, 8) && al(indY, 8)) {
+        size_t pairs = total / 2;
+        hipLaunchKernelGGL(maxpool_2x2s2_kernel, dim3(eh_blocks(pairs, TPB, 1u << 18)), dim3(TPB), 0, st, I, O, indX, indY, pairs, H,
+                           W, s.LP, s.LQ);
+    } else if (kr * kc >= 64) {
+        hipLaunchKernelGGL(maxpool_wave_kernel, dim3(eh_blocks(total, TPB / 64, 1u << 18)), dim3(TPB), 0, st, I, O, indX, indY, total,
+                           s);
+    } else {
+        hipLaunchKernelGGL(maxpool_kernel, dim3(eh_blocks(total, TPB, 1u << 18)), dim3(TPB), 0, st, I, O, indX, indY, total, s);
+    }
+    EH_CHECK_LAUNCH();
+    return 0;
+}
+
+int eddlhip_avgpool2d(int dev, const float *I, float *O, int N, int C, int H, int W, int kr, int kc, int sr, int sc, int pad_top,
+                      int pad_bottom, int pad_left, int pad_right) {
+    PoolShape s;
+    EH_TRY(check_pool("avgpool2d", N, C, H, W, kr, kc, sr, sc, pad_top, pad_bottom, pad_left, pad_right, &s));
+    size_t total = (size_t)N * C * s.LP * s.LQ;
+    if (total == 0) return 0;
+    EH_REQUIRE(I && O, "avgpool2d: NULL tensor");
+    EH_TRY(use_device(dev));
+    hipLaunchKernelGGL(avgpool_kernel, dim3(eh_blocks(total, TPB, 1u << 18)), dim3(TPB), 0, state(dev).stream, I, O, total, s);
+    EH_CHECK_LAUNCH();
+    return 0;
+}
+
+}  // extern "C"

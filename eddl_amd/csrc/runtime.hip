@@ -1,0 +1,199 @@
+// Device runtime of libeddlhip.so: initialisation, memory, copies, events, error text.
+// Stands where the reference's gpu_init / gpu_create_tensor / gpu_copy_* do
+// (src/hardware/gpu/gpu_tensor.cu:121-240, src/hardware/gpu/gpu_core.cu:49-67).
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "common.h"
+
+namespace eddlhip {
+
+static DeviceState g_state[EDDLHIP_MAX_DEVICES];
+static thread_local char g_error[512] = "";
+
+DeviceState &state(int dev) { return g_state[dev]; }
+
+int set_error(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int use_device(int dev) {
+    if (dev < 0 || dev >= EDDLHIP_MAX_DEVICES) return set_error(EDDLHIP_ENODEV, "device index %d out of range", dev);
+    DeviceState &s = g_state[dev];
+    if (!s.inited) {
+        int count = 0;
+        EH_TRY_HIP(hipGetDeviceCount(&count));
+        if (dev >= count) return set_error(EDDLHIP_ENODEV, "device %d requested, %d present", dev, count);
+        EH_TRY_HIP(hipSetDevice(dev));
+        hipDeviceProp_t prop;
+        EH_TRY_HIP(hipGetDeviceProperties(&prop, dev));
+        if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+            return set_error(EDDLHIP_ENODEV, "device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
+        s.num_cu = prop.multiProcessorCount;
+        EH_TRY_HIP(hipMalloc(&s.flag, 256));
+        EH_TRY_HIP(hipMemset(s.flag, 0, 256));
+        s.inited = true;
+        return 0;
+    }
+    EH_TRY_HIP(hipSetDevice(dev));
+    return 0;
+}
+
+int get_workspace(int dev, size_t bytes, void **ptr) {
+    DeviceState &s = g_state[dev];
+    if (bytes > s.workspace_bytes) {
+        if (s.workspace) {
+            EH_TRY_HIP(hipStreamSynchronize(s.stream));
+            EH_TRY_HIP(hipFree(s.workspace));
+            s.workspace = nullptr;
+            s.workspace_bytes = 0;
+        }
+        size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+        hipError_t e = hipMalloc(&s.workspace, want);
+        if (e != hipSuccess) {
+            s.workspace = nullptr;
+            return set_error(EDDLHIP_ENOMEM, "workspace of %zu bytes: %s", want, hipGetErrorString(e));
+        }
+        s.workspace_bytes = want;
+    }
+    *ptr = s.workspace;
+    return 0;
+}
+
+}  // namespace eddlhip
+
+using namespace eddlhip;
+
+extern "C" {
+
+const char *eddlhip_version(void) { return "eddlhip 0.1 (gfx950)"; }
+
+const char *eddlhip_last_error(void) { return g_error; }
+
+int eddlhip_device_count(int *count) {
+    EH_REQUIRE(count != nullptr, "count is NULL");
+    EH_TRY_HIP(hipGetDeviceCount(count));
+    return 0;
+}
+
+int eddlhip_init(int dev) { return use_device(dev); }
+
+int eddlhip_shutdown(int dev) {
+    if (dev < 0 || dev >= EDDLHIP_MAX_DEVICES) return set_error(EDDLHIP_ENODEV, "device index %d out of range", dev);
+    DeviceState &s = g_state[dev];
+    if (!s.inited) return 0;
+    EH_TRY_HIP(hipSetDevice(dev));
+    EH_TRY_HIP(hipDeviceSynchronize());
+    if (s.workspace) EH_TRY_HIP(hipFree(s.workspace));
+    if (s.flag) EH_TRY_HIP(hipFree(s.flag));
+    s = DeviceState();
+    return 0;
+}
+
+int eddlhip_device_name(int dev, char *buf, size_t buflen) {
+    EH_REQUIRE(buf != nullptr && buflen > 0, "buf is NULL");
+    EH_TRY(use_device(dev));
+    hipDeviceProp_t prop;
+    EH_TRY_HIP(hipGetDeviceProperties(&prop, dev));
+    snprintf(buf, buflen, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    return 0;
+}
+
+int eddlhip_set_stream(int dev, void *hip_stream) {
+    EH_TRY(use_device(dev));
+    state(dev).stream = (hipStream_t)hip_stream;
+    return 0;
+}
+
+int eddlhip_synchronize(int dev) {
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipStreamSynchronize(state(dev).stream));
+    return 0;
+}
+
+int eddlhip_malloc(int dev, size_t bytes, void **dev_ptr) {
+    EH_REQUIRE(dev_ptr != nullptr, "dev_ptr is NULL");
+    EH_TRY(use_device(dev));
+    *dev_ptr = nullptr;
+    if (bytes == 0) return 0;
+    hipError_t e = hipMalloc(dev_ptr, bytes);
+    if (e != hipSuccess) {
+        *dev_ptr = nullptr;
+        (void)hipGetLastError();
+        return set_error(EDDLHIP_ENOMEM, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+    }
+    return 0;
+}
+
+int eddlhip_free(int dev, void *dev_ptr) {
+    if (!dev_ptr) return 0;
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipFree(dev_ptr));
+    return 0;
+}
+
+// The three copies wait for earlier kernels on the device's stream and return when the data
+// has landed, like the reference's plain cudaMemcpy calls.
+int eddlhip_memcpy_h2d(int dev, void *dev_dst, const void *host_src, size_t bytes) {
+    if (bytes == 0) return 0;
+    EH_REQUIRE(dev_dst && host_src, "NULL pointer in h2d copy");
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice, state(dev).stream));
+    EH_TRY_HIP(hipStreamSynchronize(state(dev).stream));
+    return 0;
+}
+
+int eddlhip_memcpy_d2h(int dev, void *host_dst, const void *dev_src, size_t bytes) {
+    if (bytes == 0) return 0;
+    EH_REQUIRE(host_dst && dev_src, "NULL pointer in d2h copy");
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipMemcpyAsync(host_dst, dev_src, bytes, hipMemcpyDeviceToHost, state(dev).stream));
+    EH_TRY_HIP(hipStreamSynchronize(state(dev).stream));
+    return 0;
+}
+
+int eddlhip_memcpy_d2d(int dev, void *dev_dst, const void *dev_src, size_t bytes) {
+    if (bytes == 0) return 0;
+    EH_REQUIRE(dev_dst && dev_src, "NULL pointer in d2d copy");
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipMemcpyAsync(dev_dst, dev_src, bytes, hipMemcpyDeviceToDevice, state(dev).stream));
+    return 0;
+}
+
+int eddlhip_event_create(int dev, void **event) {
+    EH_REQUIRE(event != nullptr, "event is NULL");
+    EH_TRY(use_device(dev));
+    hipEvent_t ev;
+    EH_TRY_HIP(hipEventCreate(&ev));
+    *event = (void *)ev;
+    return 0;
+}
+
+int eddlhip_event_destroy(int dev, void *event) {
+    if (!event) return 0;
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipEventDestroy((hipEvent_t)event));
+    return 0;
+}
+
+int eddlhip_event_record(int dev, void *event) {
+    EH_REQUIRE(event != nullptr, "event is NULL");
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipEventRecord((hipEvent_t)event, state(dev).stream));
+    return 0;
+}
+
+int eddlhip_event_elapsed_ms(int dev, void *start, void *stop, float *ms) {
+    EH_REQUIRE(start && stop && ms, "NULL argument");
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipEventSynchronize((hipEvent_t)stop));
+    EH_TRY_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return 0;
+}
+
+}  // extern "C"

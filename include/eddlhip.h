@@ -1,0 +1,174 @@
+/*
+ * eddlhip.h - C ABI of libeddlhip.so, an MI355X (gfx950) backend for the CNN forward path
+ * of EDDL (deephealthproject/eddl v1.1).
+ *
+ * The library replaces, for forward/inference, the family of `gpu_*` free functions that
+ * EDDL's Tensor / tensorNN dispatchers call when a tensor lives on a GPU device
+ * (declared in the reference's include/eddl/hardware/gpu/gpu_tensor.h:45-53,
+ * include/eddl/hardware/gpu/gpu_hw.h:30-257 and include/eddl/hardware/gpu/nn/gpu_tensor_nn.h:26-147).
+ * Those functions take Tensor* / Descriptor* C++ objects; thin C++ shims unpack the
+ * objects into the flat calls below (plain pointers and sizes).
+ *
+ * Conventions
+ *  - All tensors are fp32, contiguous, row-major: activations NCHW, filters OIHW,
+ *    dense weights [in, out].  Pointers named `const float*`/`float*` are DEVICE pointers
+ *    unless the parameter name starts with `host`.
+ *  - Every function returns 0 on success or a negative EDDLHIP_E* code; a message for the
+ *    last failure on the calling thread is available from eddlhip_last_error().
+ *  - Kernels are launched asynchronously on one stream per device (the null stream unless
+ *    eddlhip_set_stream was called); eddlhip_synchronize() waits for them.  The reference's
+ *    wrappers synchronise after every launch (e.g. src/hardware/gpu/nn/gpu_pool.cu:27-33);
+ *    the C++ shims reproduce that by calling eddlhip_synchronize() before returning.
+ *  - The library never owns user-visible tensors.  It keeps one private, grow-only
+ *    workspace per device (repacked filters); eddlhip_shutdown() releases it.
+ *  - Calls on one device must not overlap from several threads (the reference drives one
+ *    device from one thread: src/net/net_api.cpp:146-171).
+ */
+#ifndef EDDLHIP_H
+#define EDDLHIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EDDLHIP_OK 0
+#define EDDLHIP_EINVAL (-1)  /* bad argument (shape, null pointer, unsupported mode) */
+#define EDDLHIP_EHIP (-2)    /* a HIP runtime call failed */
+#define EDDLHIP_ENODEV (-3)  /* no such device */
+#define EDDLHIP_ENOMEM (-4)  /* device allocation failed */
+
+/* ------------------------------------------------------------------ runtime
+ * Replaces gpu_devices / gpu_init / gpu_set_device / gpu_create_tensor / gpu_delete_tensor
+ * (src/hardware/gpu/gpu_tensor.cu:121-240) and gpu_copy_to_gpu / gpu_copy_from_gpu /
+ * gpu_copy_gpu / gpu_fill_ (src/hardware/gpu/gpu_core.cu:49-67,139-147). */
+const char *eddlhip_version(void);
+const char *eddlhip_last_error(void);
+int eddlhip_device_count(int *count);
+int eddlhip_init(int dev);
+int eddlhip_shutdown(int dev);
+int eddlhip_device_name(int dev, char *buf, size_t buflen);
+int eddlhip_set_stream(int dev, void *hip_stream);
+int eddlhip_synchronize(int dev);
+int eddlhip_malloc(int dev, size_t bytes, void **dev_ptr);
+int eddlhip_free(int dev, void *dev_ptr);
+int eddlhip_memcpy_h2d(int dev, void *dev_dst, const void *host_src, size_t bytes);
+int eddlhip_memcpy_d2h(int dev, void *host_dst, const void *dev_src, size_t bytes);
+int eddlhip_memcpy_d2d(int dev, void *dev_dst, const void *dev_src, size_t bytes);
+int eddlhip_fill(int dev, float *A, size_t n, float v);
+
+/* Events on the device's stream, for timing kernels where they run.  No counterpart in the
+ * reference (its profiling is host wall-clock, include/eddl/profiling.h:27-66). */
+int eddlhip_event_create(int dev, void **event);
+int eddlhip_event_destroy(int dev, void *event);
+int eddlhip_event_record(int dev, void *event);
+int eddlhip_event_elapsed_ms(int dev, void *start, void *stop, float *ms);
+
+/* ------------------------------------------------------------------ convolution
+ * Replaces gpu_conv2D(ConvolDescriptor*) (src/hardware/gpu/nn/gpu_conv.cu:159-233; CPU
+ * semantics src/hardware/cpu/nn/cpu_conv.cpp:55-112,114-226,316-346).
+ *
+ * Cross-correlation.  I[N,C,H,W], K[Kf,C,R,S], O[N,Kf,P,Q].  Output pixel (p,q) reads taps
+ * (p*sr - pad_top + ky, q*sc - pad_left + kx); taps outside the image read 0.  P and Q come
+ * from the descriptor (its geometry rules are not a closed form of the pads), so they are
+ * arguments; only the top/left pads enter the arithmetic, as in the reference's lowering.
+ * bias may be NULL (descriptor's use_bias == false).
+ *
+ * Fused epilogue (all optional; what a Conv -> BatchNorm(inference) -> Add -> ReLU chain of
+ * layers computes, applied per output element in this order, each step rounded to fp32
+ * with no fused multiply-add):
+ *     v = acc;  if bias: v = v + bias[k]
+ *     if bn_mean: v = ((v - bn_mean[k]) / sqrtf(bn_var[k] + bn_eps)) * bn_g[k] + bn_b[k]
+ *                 (bn_g/bn_b NULL => no affine step)
+ *     if residual: v = v + residual[same index as O]
+ *     if relu: v = v > 0 ? v : 0
+ * With the epilogue pointers NULL and relu 0 it is exactly the descriptor call. */
+int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bias, float *O,
+                       int N, int C, int H, int W, int Kf, int R, int S, int sr, int sc,
+                       int pad_top, int pad_left, int P, int Q,
+                       const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var,
+                       float bn_eps, const float *residual, int relu);
+
+/* Selects the convolution kernel: 0 = automatic, 1 = force the general implicit-GEMM MFMA
+ * kernel, 2 = force the scalar direct kernel (one thread per output; taps summed in the
+ * reference's ky,kx,c order - used to cross-check the MFMA kernels on the device). */
+int eddlhip_conv2d_set_algo(int algo);
+
+/* ------------------------------------------------------------------ batch normalisation (inference)
+ * Replaces gpu_batchnorm_forward(...) with trmode == false
+ * (include/eddl/hardware/gpu/nn/gpu_tensor_nn.h:138-143, src/hardware/gpu/nn/gpu_bn.cu:65-98;
+ * CPU semantics src/hardware/cpu/nn/cpu_bn.cpp:154-179).  b = batch, z = channels, rc = H*W.
+ * Writes sd[c] = sqrtf(global_variance[c] + eps) into `variance` (the layer's bn_var), then
+ * o = (x - global_mean[c]) / sd[c]; with affine (affine_g != NULL): opa = o (if opa != NULL)
+ * and y = o*g[c] + b[c]. */
+int eddlhip_batchnorm_inference(int dev, int b, int z, int rc, const float *input, float *output, float *opa,
+                                const float *global_mean, const float *global_variance,
+                                const float *affine_g, const float *affine_b, float *variance, float epsilon);
+
+/* ------------------------------------------------------------------ activations
+ * Replace gpu_relu / gpu_sigmoid / gpu_full_softmax
+ * (include/eddl/hardware/gpu/nn/gpu_tensor_nn.h:26,44,59; CPU semantics
+ * src/hardware/cpu/nn/cpu_activations.cpp:18-33,329-375, src/hardware/cpu/cpu_math.cpp:354-357).
+ * Softmax runs over an axis of length `len` whose stride is `inner`; `outer` is the product
+ * of the dimensions before it. */
+int eddlhip_relu(int dev, const float *A, float *B, size_t n);
+int eddlhip_sigmoid(int dev, const float *A, float *B, size_t n);
+int eddlhip_softmax(int dev, const float *A, float *B, int outer, int len, int inner, int stable);
+
+/* ------------------------------------------------------------------ pooling
+ * Replace gpu_mpool2D / gpu_avgpool2D(PoolDescriptor*)
+ * (src/hardware/gpu/nn/gpu_pool.cu:26-46,101-117; CPU semantics
+ * src/hardware/cpu/nn/cpu_pool.cpp:74-121,226-274).  Window origins run
+ * i = -pad_top; i <= H + pad_bottom - kr; i += sr (same for columns); outputs are written
+ * densely in that loop order.  eddlhip_pool2d_out_dims returns the two loop counts.
+ * Max: indX/indY receive the absolute column/row of the first maximum, as floats; a window
+ * with no tap above -3.40282e+38f leaves its two index slots untouched.
+ * Avg: in-image taps summed in (ky,kx) order, divided by kr*kc. */
+int eddlhip_pool2d_out_dims(int H, int W, int kr, int kc, int sr, int sc,
+                            int pad_top, int pad_bottom, int pad_left, int pad_right, int *LP, int *LQ);
+int eddlhip_maxpool2d(int dev, const float *I, float *O, float *indX, float *indY,
+                      int N, int C, int H, int W, int kr, int kc, int sr, int sc,
+                      int pad_top, int pad_bottom, int pad_left, int pad_right);
+int eddlhip_avgpool2d(int dev, const float *I, float *O,
+                      int N, int C, int H, int W, int kr, int kc, int sr, int sc,
+                      int pad_top, int pad_bottom, int pad_left, int pad_right);
+
+/* ------------------------------------------------------------------ resize / concat / add / pad
+ * eddlhip_scale_nearest replaces gpu_scale(A, B, new_shape, wrap, c, mode) for the only
+ * combination UpSampling2D uses: nearest wrapping, "asymmetric" coordinates
+ * (src/hardware/gpu/gpu_da.cu:61-76; CPU semantics src/hardware/cpu/cpu_da.cpp:88-137,407-436).
+ * A[N,C,H,W] -> B[N,C,OH,OW]; source index = (int)((float)(dst + off) / ((float)new / in)),
+ * off = (int)((new - out)/2.0f).  Destination elements whose source falls outside A are left
+ * untouched and make the call fail with EDDLHIP_EINVAL (the reference raises there).
+ *
+ * eddlhip_concat replaces gpu_concat(A, t, axis, false) with the CPU backend's semantics
+ * (src/hardware/cpu/cpu_core.cpp:368-396): n_in device pointers (host array), the axis extent
+ * of each, `outer` = product of dims before the axis, `inner` = stride of the axis.
+ *
+ * eddlhip_add replaces gpu_add(scA, A, scB, B, C, incC) (src/hardware/gpu/gpu_math.cu:446-455;
+ * CPU src/hardware/cpu/cpu_math.cpp:278-287); eddlhip_inc replaces gpu_inc.
+ *
+ * eddlhip_pad replaces gpu_pad(A, B, pads) (CPU src/hardware/cpu/cpu_da.cpp:502-517): interior
+ * copy, pads in the reference's (top, right, bottom, left) order; B's border is not written. */
+int eddlhip_scale_nearest(int dev, const float *A, float *B, int N, int C, int H, int W, int OH, int OW,
+                          int newH, int newW);
+int eddlhip_concat(int dev, float *dest, const float *const *host_srcs, const int *host_axis_extent, int n_in,
+                   int outer, int inner);
+int eddlhip_add(int dev, float scA, const float *A, float scB, const float *B, float *C, int incC, size_t n);
+int eddlhip_inc(int dev, const float *A, float *B, size_t n);
+int eddlhip_pad(int dev, const float *A, float *B, int N, int C, int H, int W,
+                int top, int right, int bottom, int left);
+
+/* ------------------------------------------------------------------ dense
+ * eddlhip_mult2d replaces gpu_mult2D(A, tA, B, tB, C, incC) for the forward case
+ * tA = tB = 0 used by LDense::forward (src/layers/core/layer_dense.cpp:65-73,
+ * src/hardware/gpu/gpu_math.cu:457-488): C[m,n] (+)= A[m,k] * B[k,n], row-major.
+ * eddlhip_sum2d_rowwise replaces gpu_sum2D_rowwise: C[i][j] = A[i][j] + B[j]. */
+int eddlhip_mult2d(int dev, const float *A, const float *B, float *C, int m, int k, int n, int incC);
+int eddlhip_sum2d_rowwise(int dev, const float *A, const float *B, float *C, int rows, int cols);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EDDLHIP_H */

@@ -1,0 +1,90 @@
+"""CPU-side checks of the C ABI and of the host-side descriptor mirrors (no GPU needed)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from conftest import ROOT
+
+
+def _declared_functions():
+    src = open(os.path.join(ROOT, "include", "eddlhip.h")).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(eddlhip_\w+)\s*\(", src)))
+
+
+def test_library_exports_every_declared_symbol():
+    from eddl_amd import _lib
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    names = _declared_functions()
+    assert len(names) >= 30
+    for n in names:
+        assert hasattr(lib, n), "libeddlhip.so lacks %s" % n
+    assert set(names) == set(_lib.PROTOTYPES), "ctypes prototypes out of step with include/eddlhip.h"
+
+
+def test_version_and_argument_errors_without_a_device():
+    from eddl_amd import _lib
+    lib = _lib.load()
+    assert b"gfx950" in lib.eddlhip_version()
+    assert lib.eddlhip_conv2d_set_algo(9) == -1
+    assert b"unknown algorithm" in lib.eddlhip_last_error()
+    assert lib.eddlhip_conv2d_set_algo(0) == 0
+    lp, lq = ctypes.c_int(), ctypes.c_int()
+    assert lib.eddlhip_pool2d_out_dims(5, 5, 3, 3, 2, 2, 0, 1, 0, 1, ctypes.byref(lp), ctypes.byref(lq)) == 0
+    assert (lp.value, lq.value) == (2, 2)
+    assert lib.eddlhip_pool2d_out_dims(5, 5, 0, 3, 2, 2, 0, 1, 0, 1, ctypes.byref(lp), ctypes.byref(lq)) == -1
+
+
+def test_descriptor_mirrors_match_the_oracle_geometry(oracle, golden):
+    from eddl_amd.descriptors import ConvolDescriptor, PoolDescriptor
+    t = golden["output_sizes"]
+    i = 0
+    for p in t["padding"]:
+        for isz in t["input_sizes"]:
+            for s in t["strides"]:
+                for k in t["kernels"]:
+                    assert ConvolDescriptor.compute_output(p, isz, k, s) == t["output_sizes"][i]
+                    i += 1
+    rng = np.random.default_rng(3)
+    for _ in range(300):
+        H, W = int(rng.integers(1, 70)), int(rng.integers(1, 70))
+        kr, kc = int(rng.integers(1, 8)), int(rng.integers(1, 8))
+        sr, sc = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        for padding in ("same", "valid"):
+            try:
+                cd = ConvolDescriptor(4, [kr, kc], [sr, sc], padding).build([2, 3, H, W])
+                got = (cd.r, cd.c, tuple(cd.pads))
+            except RuntimeError:
+                got = None
+            P, Q, pads = oracle.conv_geometry(H, W, kr, kc, sr, sc, padding)
+            exp = (P, Q, pads) if P > 0 and Q > 0 else None
+            assert got == exp
+            try:
+                pd = PoolDescriptor([kr, kc], [sr, sc], padding).build([2, 3, H, W])
+                got = (pd.r, pd.c, tuple(pd.pad), pd.loop_rows, pd.loop_cols)
+            except RuntimeError:
+                got = None
+            r, c, p4, lp, lq = oracle.pool_geometry(H, W, kr, kc, sr, sc, padding)
+            assert got == ((r, c, p4, lp, lq) if r > 0 and c > 0 else None)
+        pads = [int(v) for v in rng.integers(0, 4, 4)]
+        P, Q, _ = oracle.conv_geometry(H, W, kr, kc, sr, sc, "custom", pads)
+        if P > 0 and Q > 0:
+            cd = ConvolDescriptor(4, [kr, kc], [sr, sc], "custom", pads).build([2, 3, H, W])
+            assert (cd.r, cd.c) == (P, Q)
+
+
+def test_descriptor_errors_follow_the_reference():
+    from eddl_amd.descriptors import ConvolDescriptor, PoolDescriptor
+    with pytest.raises(RuntimeError, match="ConvolDescriptor::ConvolDescriptor"):
+        ConvolDescriptor(4, [3, 3], [1, 1], "bogus")
+    with pytest.raises(RuntimeError, match="Grouped"):
+        ConvolDescriptor(4, [3, 3], [1, 1], "same", groups=2)
+    with pytest.raises(RuntimeError, match="ConvolDescriptor::build"):
+        ConvolDescriptor(4, [3, 3], [1, 1], "same").build([1, 3, 8])
+    with pytest.raises(RuntimeError, match="Invalid output shape"):
+        ConvolDescriptor(4, [5, 5], [1, 1], "valid").build([1, 3, 4, 4])
+    with pytest.raises(RuntimeError, match="PoolDescriptor::PoolDescriptor"):
+        PoolDescriptor([2, 2], [2, 2], "bogus")

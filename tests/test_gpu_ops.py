@@ -1,0 +1,340 @@
+"""Parity of the HIP kernels, called through the C ABI, with the CPU oracle on the same
+seeded inputs, and with the vectors the reference's own tests hold.
+
+Bars: bit-exact for ReLU, Add, Concat, UpSampling, Pad, MaxPool (values and argmax indices),
+AvgPool, BatchNorm-inference and the scalar direct convolution; floating-point tolerance for
+the MFMA convolution (|a-b| <= atol + rtol*|b|, rtol 1e-4, atol 1e-5*max|ref|), dense,
+sigmoid and softmax (different summation order / exp implementation).
+"""
+import numpy as np
+import pytest
+
+from conftest import eddl_allclose, tensor_of
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-4
+
+
+def assert_conv_close(ref, out, what=""):
+    atol = 1e-5 * float(np.max(np.abs(ref)))
+    err = np.abs(ref - out) - (atol + RTOL * np.abs(ref))
+    assert np.all(err <= 0), "%s: worst excess %g at %s (ref %g out %g)" % (
+        what, err.max(), np.unravel_index(err.argmax(), err.shape), ref.flat[err.argmax()], out.flat[err.argmax()])
+
+
+def run_conv(hip, oracle, x, w, b, stride, padding, pads=None, algo="auto", bn=None, residual=None, relu=False):
+    from eddl_amd.descriptors import ConvolDescriptor
+    cd = ConvolDescriptor(w.shape[0], list(w.shape[2:]), list(stride), padding, pads or [], use_bias=b is not None).build(list(x.shape))
+    O = hip.empty(cd.out_shape)
+    dbn = None
+    if bn is not None:
+        g, bb, mean, var, eps = bn
+        dbn = (hip.array(g) if g is not None else None, hip.array(bb) if bb is not None else None, hip.array(mean), hip.array(var), eps)
+    hip.set_conv_algo(algo)
+    try:
+        hip.conv2D(hip.array(x), hip.array(w), hip.array(b) if b is not None else None, O, cd.sr, cd.sc, cd.padrt, cd.padcl,
+                   bn=dbn, residual=hip.array(residual) if residual is not None else None, relu=relu)
+    finally:
+        hip.set_conv_algo("auto")
+    ref = oracle.conv2d(x, w, b, stride, cd.padrt, cd.padcl, cd.r, cd.c)
+    if bn is not None:
+        g, bb, mean, var, eps = bn
+        ref, _, _ = oracle.batchnorm_inference(ref, mean, var, g, bb, eps)
+    if residual is not None:
+        ref = oracle.add(ref, residual)
+    if relu:
+        ref = oracle.relu(ref)
+    return ref, O.numpy()
+
+
+# ------------------------------------------------------------------ reference-held vectors
+def _conv_inputs(case):
+    x = tensor_of(case["image"])
+    kshape = (case["filters"], x.shape[1], case["kernel"][0], case["kernel"][1])
+    w = np.ones(kshape, np.float32) if case["filters_data"] == "ones" else tensor_of(case["filters_data"])
+    b = np.zeros(case["filters"], np.float32) if case["bias_data"] == "zeros" else tensor_of(case["bias_data"])
+    return x, w, (b if case["use_bias"] else None)
+
+
+@pytest.mark.parametrize("algo", ["mfma", "direct"])
+def test_conv2d_reference_vectors(hip, oracle, golden, algo):
+    for case in golden["conv2d"]:
+        x, w, b = _conv_inputs(case)
+        ref, out = run_conv(hip, oracle, x, w, b, case["strides"], case["padding"], algo=algo)
+        exp = tensor_of(case["forward"])
+        assert out.shape == exp.shape, case["name"]
+        assert eddl_allclose(exp, out, case["atol"], case["rtol"]), case["name"]
+        assert np.array_equal(exp, out), case["name"]  # small integers: exact in any order
+
+
+def test_pool_reference_vectors(hip, golden):
+    from eddl_amd.descriptors import PoolDescriptor
+    for case in golden["maxpool2d"]:
+        x = tensor_of(case["image"])
+        pd = PoolDescriptor(case["kernel"], case["strides"], case["padding"]).build(list(x.shape))
+        O, ix, iy = hip.empty(pd.out_shape), hip.full(pd.out_shape, -1.0), hip.full(pd.out_shape, -1.0)
+        hip.mpool2D(hip.array(x), O, ix, iy, pd.ksize, pd.stride, pd.pad)
+        assert np.array_equal(O.numpy(), tensor_of(case["forward"])), case["name"]
+        hist = np.zeros_like(x)
+        for yy, xx in zip(iy.numpy().ravel(), ix.numpy().ravel()):
+            hist[0, 0, int(yy), int(xx)] += 1
+        assert np.array_equal(hist, tensor_of(case["backward_of_ones"])), case["name"]
+    for case in golden["avgpool2d"]:
+        x = tensor_of(case["image"])
+        pd = PoolDescriptor(case["kernel"], case["strides"], case["padding"]).build(list(x.shape))
+        O = hip.empty(pd.out_shape)
+        hip.avgpool2D(hip.array(x), O, pd.ksize, pd.stride, pd.pad)
+        assert eddl_allclose(tensor_of(case["forward"]), O.numpy(), case["atol"], case["rtol"]), case["name"]
+
+
+def test_pad_and_softmax_reference_vectors(hip, golden):
+    case = golden["pad"]
+    x = tensor_of(case["input"])
+    exp = tensor_of(case["expected"])
+    B = hip.full(exp.shape, 0.0)
+    hip.pad(hip.array(x), B, case["pads"])
+    assert eddl_allclose(exp, B.numpy(), case["atol"])
+    case = golden["softmax"]
+    x = tensor_of(case["input"])
+    B = hip.empty(x.shape)
+    hip.full_softmax(hip.array(x), B, case["axis"])
+    assert eddl_allclose(tensor_of(case["expected"]), B.numpy(), case["atol"])
+
+
+# ------------------------------------------------------------------ convolution
+CONV_SHAPES = [
+    # N, C, H, W, Kf, R, S, sr, sc, padding, pads, bias
+    (8, 3, 32, 32, 32, 3, 3, 1, 1, "same", None, True),        # BASELINE config 1 shape
+    (2, 64, 28, 28, 64, 3, 3, 1, 1, "same", None, False),
+    (2, 16, 19, 23, 130, 3, 3, 1, 1, "same", None, True),      # ragged: channels and pixels not tile multiples
+    (3, 5, 17, 13, 7, 3, 3, 2, 2, "same", None, True),         # asymmetric same pads
+    (2, 3, 37, 41, 16, 7, 7, 2, 2, "custom", [3, 3, 3, 3], False),  # ResNet stem geometry
+    (2, 32, 14, 14, 96, 1, 1, 1, 1, "valid", None, False),     # 1x1
+    (2, 32, 15, 15, 48, 1, 1, 2, 2, "valid", None, True),      # 1x1 stride 2 (projection shortcut)
+    (2, 8, 12, 12, 4, 2, 2, 1, 1, "valid", None, True),        # 2x2 valid (U-Net up-conv after Pad)
+    (1, 64, 9, 9, 1, 1, 1, 1, 1, "valid", None, True),         # single output channel
+    (2, 6, 10, 12, 5, 3, 2, 1, 2, "same", None, True),         # rectangular filter, mixed strides
+    (1, 300, 8, 8, 33, 3, 3, 1, 1, "same", None, False),       # many taps (C*R*S = 2700)
+    (1, 1, 64, 64, 64, 3, 3, 1, 1, "same", None, True),        # single input channel (U-Net first layer)
+]
+
+
+@pytest.mark.parametrize("shape", CONV_SHAPES, ids=lambda s: "x".join(str(v) for v in s[:9]) + "-" + s[9])
+def test_conv2d_mfma_against_oracle(hip, oracle, shape):
+    N, C, H, W, Kf, R, S, sr, sc, padding, pads, use_bias = shape
+    rng = np.random.default_rng(100 + C * 7 + Kf)
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    w = (rng.standard_normal((Kf, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32)
+    b = rng.standard_normal(Kf, dtype=np.float32) if use_bias else None
+    ref, out = run_conv(hip, oracle, x, w, b, (sr, sc), padding, pads, algo="mfma")
+    assert out.shape == ref.shape
+    assert_conv_close(ref, out, str(shape))
+
+
+@pytest.mark.parametrize("shape", CONV_SHAPES[:6], ids=lambda s: "x".join(str(v) for v in s[:9]))
+def test_conv2d_direct_kernel_is_bit_exact(hip, oracle, shape):
+    N, C, H, W, Kf, R, S, sr, sc, padding, pads, use_bias = shape
+    rng = np.random.default_rng(200 + C)
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    w = rng.standard_normal((Kf, C, R, S), dtype=np.float32)
+    b = rng.standard_normal(Kf, dtype=np.float32) if use_bias else None
+    ref, out = run_conv(hip, oracle, x, w, b, (sr, sc), padding, pads, algo="direct")
+    assert np.array_equal(ref, out)
+
+
+def _bn_params(rng, C):
+    mean = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    var = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    g = rng.uniform(0.8, 1.2, C).astype(np.float32)
+    b = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    return g, b, mean, var, 1e-5
+
+
+def test_conv2d_fused_epilogue(hip, oracle):
+    rng = np.random.default_rng(300)
+    N, C, H, W, Kf = 2, 24, 14, 14, 40
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    w = (rng.standard_normal((Kf, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32)
+    bias = rng.standard_normal(Kf, dtype=np.float32)
+    res = rng.standard_normal((N, Kf, H, W), dtype=np.float32)
+    bn = _bn_params(rng, Kf)
+    # direct kernel + fused tail: every step has the oracle's rounding, so it is bit-exact
+    for kw in (dict(bn=bn, relu=True), dict(bn=bn, residual=res, relu=True), dict(b=bias, bn=(None, None) + bn[2:]),
+               dict(b=bias, residual=res), dict(relu=True)):
+        b = kw.pop("b", None)
+        ref, out = run_conv(hip, oracle, x, w, b, (1, 1), "same", algo="direct", **kw)
+        assert np.array_equal(ref, out), kw.keys()
+    for kw in (dict(bn=bn, relu=True), dict(bn=bn, residual=res, relu=True)):
+        ref, out = run_conv(hip, oracle, x, w, None, (1, 1), "same", algo="mfma", **kw)
+        assert_conv_close(ref, out, "fused mfma")
+        assert np.all(out >= 0)
+
+
+def test_conv2d_linearity_and_empty_batch(hip, oracle):
+    from eddl_amd.descriptors import ConvolDescriptor
+    rng = np.random.default_rng(301)
+    x1 = rng.standard_normal((2, 16, 20, 20), dtype=np.float32)
+    x2 = rng.standard_normal((2, 16, 20, 20), dtype=np.float32)
+    w = rng.standard_normal((32, 16, 3, 3), dtype=np.float32) / 12
+    _, o1 = run_conv(hip, oracle, x1, w, None, (1, 1), "same", algo="mfma")
+    _, o2 = run_conv(hip, oracle, x2, w, None, (1, 1), "same", algo="mfma")
+    _, o12 = run_conv(hip, oracle, x1 + x2, w, None, (1, 1), "same", algo="mfma")
+    np.testing.assert_allclose(o12, o1 + o2, rtol=1e-4, atol=1e-4)
+    # empty batch: nothing launched, no error
+    cd = ConvolDescriptor(32, [3, 3], [1, 1], "same").build([0, 16, 20, 20])
+    hip.conv2D(hip.empty((0, 16, 20, 20)), hip.array(w), None, hip.empty(cd.out_shape), 1, 1, 1, 1)
+    hip.synchronize()
+
+
+def test_conv2d_argument_errors(hip):
+    from eddl_amd import EddlHipError
+    x, w, o = hip.empty((1, 3, 8, 8)), hip.empty((4, 3, 3, 3)), hip.empty((1, 4, 8, 8))
+    g = hip.empty((4,))
+    with pytest.raises(EddlHipError, match="bn_mean and bn_var"):
+        hip.conv2D(x, w, None, o, 1, 1, 1, 1, bn=(None, None, g, None, 1e-5))
+    with pytest.raises(EddlHipError, match="strides"):
+        hip.conv2D(x, w, None, o, 0, 1, 1, 1)
+
+
+# ------------------------------------------------------------------ bandwidth-bound operators
+def test_batchnorm_inference_bit_exact(hip, oracle):
+    rng = np.random.default_rng(400)
+    for shape in [(4, 64, 28, 28), (3, 5, 7, 9), (2, 130, 1, 1), (2, 3, 6, 6), (1, 20000, 1, 2)]:
+        C = shape[1]
+        x = rng.standard_normal(shape, dtype=np.float32)
+        g, b, mean, var, eps = _bn_params(rng, C)
+        y_ref, opa_ref, sd_ref = oracle.batchnorm_inference(x, mean, var, g, b, eps)
+        y, opa, sd = hip.empty(shape), hip.empty(shape), hip.empty((C,))
+        hip.batchnorm_inference(hip.array(x), y, opa, hip.array(mean), hip.array(var), hip.array(g), hip.array(b), sd, eps)
+        assert np.array_equal(y.numpy(), y_ref) and np.array_equal(opa.numpy(), opa_ref) and np.array_equal(sd.numpy(), sd_ref)
+        y2_ref, _, _ = oracle.batchnorm_inference(x, mean, var, None, None, eps)
+        hip.batchnorm_inference(hip.array(x), y, None, hip.array(mean), hip.array(var), None, None, sd, eps)
+        assert np.array_equal(y.numpy(), y2_ref)
+
+
+def test_relu_add_inc_fill(hip, oracle):
+    rng = np.random.default_rng(401)
+    for n in (1, 3, 1023, 4096, 100003):
+        x = rng.standard_normal(n, dtype=np.float32)
+        y = rng.standard_normal(n, dtype=np.float32)
+        x[:: 7] = 0.0
+        if n > 8:
+            x[1], x[2], x[3], x[4] = -0.0, np.nan, np.inf, -np.inf
+        B = hip.empty((n,))
+        hip.relu(hip.array(x), B)
+        out = B.numpy()
+        assert np.array_equal(out, oracle.relu(x)) and not np.any(np.signbit(out))
+        C = hip.empty((n,))
+        x = np.nan_to_num(x, nan=1.0, posinf=2.0, neginf=-2.0)
+        hip.add(1.0, hip.array(x), 1.0, hip.array(y), C, 0)
+        assert np.array_equal(C.numpy(), oracle.add(x, y))
+        hip.add(0.5, hip.array(x), -3.0, hip.array(y), C, 1)
+        assert np.array_equal(C.numpy(), oracle.add(x, y, 0.5, -3.0, c=oracle.add(x, y)))
+        # the n-ary Add layer: fill_(0) then inc per parent
+        hip.fill_(C, 0.0)
+        hip.inc(hip.array(x), C)
+        hip.inc(hip.array(y), C)
+        assert np.array_equal(C.numpy(), (np.float32(0) + x) + y)
+        hip.fill_(C, 2.5)
+        assert np.all(C.numpy() == np.float32(2.5))
+
+
+def test_maxpool_bit_exact_with_indices(hip, oracle):
+    rng = np.random.default_rng(402)
+    cases = [
+        ((4, 16, 56, 56), (2, 2), (2, 2), (0, 0, 0, 0)),   # fast path
+        ((2, 3, 57, 55), (2, 2), (2, 2), (0, 0, 0, 0)),    # odd sizes: general path
+        ((2, 8, 28, 28), (3, 3), (2, 2), (1, 1, 1, 1)),    # ResNet stem pool geometry
+        ((2, 4, 13, 17), (3, 3), (1, 1), (1, 1, 1, 1)),
+        ((2, 4, 12, 12), (2, 2), (2, 2), (0, 1, 0, 1)),
+        ((3, 5, 7, 7), (7, 7), (1, 1), (0, 0, 0, 0)),      # 49 taps, one thread per output
+        ((3, 5, 9, 9), (9, 9), (1, 1), (0, 0, 0, 0)),      # 81 taps: one wavefront per output
+        ((2, 3, 20, 20), (8, 8), (4, 4), (2, 2, 2, 2)),    # wavefront path with padding
+    ]
+    for shape, k, s, pads in cases:
+        for ties in (False, True):
+            x = rng.integers(-3, 4, size=shape).astype(np.float32) if ties else rng.standard_normal(shape, dtype=np.float32)
+            O_ref, ix_ref, iy_ref = oracle.maxpool2d(x, k, s, pads, fill=-5.0)
+            O, ix, iy = hip.empty(O_ref.shape), hip.full(O_ref.shape, -5.0), hip.full(O_ref.shape, -5.0)
+            assert hip.pool_out_dims(shape[2], shape[3], k, s, pads) == O_ref.shape[2:]
+            hip.mpool2D(hip.array(x), O, ix, iy, k, s, pads)
+            assert np.array_equal(O.numpy(), O_ref), (shape, k)
+            assert np.array_equal(ix.numpy(), ix_ref) and np.array_equal(iy.numpy(), iy_ref), (shape, k, ties)
+    # windows with nothing above the start value keep their index slots
+    for shape, k in (((1, 2, 8, 8), (2, 2)), ((1, 2, 9, 9), (3, 3)), ((1, 1, 16, 16), (8, 8))):
+        x = np.full(shape, -np.inf, np.float32)
+        x[0, 0, :4, :4] = np.nan
+        O_ref, ix_ref, iy_ref = oracle.maxpool2d(x, k, k, (0, 0, 0, 0), fill=-5.0)
+        O, ix, iy = hip.empty(O_ref.shape), hip.full(O_ref.shape, -5.0), hip.full(O_ref.shape, -5.0)
+        hip.mpool2D(hip.array(x), O, ix, iy, k, k, (0, 0, 0, 0))
+        assert np.array_equal(O.numpy(), O_ref) and np.array_equal(ix.numpy(), ix_ref) and np.array_equal(iy.numpy(), iy_ref)
+
+
+def test_avgpool_bit_exact(hip, oracle):
+    rng = np.random.default_rng(403)
+    for shape, k, s, pads in [((4, 16, 56, 56), (2, 2), (2, 2), (0, 0, 0, 0)), ((2, 8, 28, 28), (3, 3), (2, 2), (1, 1, 1, 1)),
+                              ((2, 64, 7, 7), (7, 7), (1, 1), (0, 0, 0, 0)), ((2, 4, 13, 17), (3, 2), (1, 2), (1, 0, 0, 1))]:
+        x = rng.standard_normal(shape, dtype=np.float32)
+        ref = oracle.avgpool2d(x, k, s, pads)
+        O = hip.empty(ref.shape)
+        hip.avgpool2D(hip.array(x), O, k, s, pads)
+        assert np.array_equal(O.numpy(), ref), (shape, k)
+
+
+def test_upsample_concat_pad_bit_exact(hip, oracle):
+    from eddl_amd import EddlHipError
+    rng = np.random.default_rng(404)
+    x = rng.standard_normal((2, 5, 9, 7), dtype=np.float32)
+    for s in (2, 3):
+        ref = oracle.scale_nearest(x, (9 * s, 7 * s))
+        B = hip.empty(ref.shape)
+        hip.scale(hip.array(x), B, (9 * s, 7 * s))
+        assert np.array_equal(B.numpy(), ref)
+    ref = oracle.scale_nearest(x, (13, 10))  # non-integer factor, same float rule
+    B = hip.empty(ref.shape)
+    hip.scale(hip.array(x), B, (13, 10))
+    assert np.array_equal(B.numpy(), ref)
+    with pytest.raises(EddlHipError, match="outside the source"):
+        hip.scale(hip.array(x), hip.empty((2, 5, 18, 14)), (9, 7))  # zoom-out window: no nearest rule
+    parts = [rng.standard_normal((2, c, 8, 8), dtype=np.float32) for c in (4, 3, 9)]
+    for axis in (1, 0, 3):
+        ps = parts if axis == 1 else [parts[0], parts[0] * 2]
+        ref = oracle.concat(ps, axis)
+        out = hip.empty(ref.shape)
+        hip.concat(out, [hip.array(p) for p in ps], axis)
+        assert np.array_equal(out.numpy(), ref), axis
+    odd = [rng.standard_normal((2, c, 5, 3), dtype=np.float32) for c in (1, 2)]  # scalar path
+    out = hip.empty((2, 3, 5, 3))
+    hip.concat(out, [hip.array(p) for p in odd], 1)
+    assert np.array_equal(out.numpy(), np.concatenate(odd, 1))
+    ref = oracle.pad(x, (0, 1, 1, 0), cval=0.0)
+    B = hip.full(ref.shape, 0.0)
+    hip.pad(hip.array(x), B, (0, 1, 1, 0))
+    assert np.array_equal(B.numpy(), ref)
+    ref = oracle.pad(x, (1, 2, 3, 4), cval=7.0)
+    B = hip.full(ref.shape, 7.0)
+    hip.pad(hip.array(x), B, (1, 2, 3, 4))
+    assert np.array_equal(B.numpy(), ref)
+
+
+def test_dense_sigmoid_softmax_within_tolerance(hip, oracle):
+    rng = np.random.default_rng(405)
+    for m, k, n in [(32, 512, 1000), (5, 37, 300), (64, 2048, 10), (33, 100, 65)]:
+        a = rng.standard_normal((m, k), dtype=np.float32)
+        w = (rng.standard_normal((k, n)) * np.sqrt(2.0 / k)).astype(np.float32)
+        bias = rng.standard_normal(n, dtype=np.float32)
+        ref = oracle.dense(a, w, bias)
+        C = hip.empty((m, n))
+        hip.mult2D(hip.array(a), hip.array(w), C)
+        hip.sum2D_rowwise(C, hip.array(bias), C)
+        assert_conv_close(ref, C.numpy(), "dense %dx%dx%d" % (m, k, n))
+    x = rng.standard_normal((4, 1, 33, 31), dtype=np.float32) * 4
+    B = hip.empty(x.shape)
+    hip.sigmoid(hip.array(x), B)
+    np.testing.assert_allclose(B.numpy(), oracle.sigmoid(x), rtol=1e-6, atol=1e-7)
+    for shape, axis in [((32, 1000), 1), ((3, 7, 5, 4), 1), ((6, 1), 1)]:
+        x = rng.standard_normal(shape, dtype=np.float32) * 3
+        B = hip.empty(shape)
+        hip.full_softmax(hip.array(x), B, axis)
+        np.testing.assert_allclose(B.numpy(), oracle.softmax(x, axis), rtol=2e-6, atol=1e-8)
