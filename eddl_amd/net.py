@@ -1,0 +1,451 @@
+"""Forward-only model graphs over the HIP backend.
+
+The layer factories carry the names and arguments of the reference's API
+(src/apis/eddl.cpp:521-539,604-608,680-704,852-854,894-905,931-943,1067-1069,1150-1190,1264-1273)
+and each layer's unfused forward is the one call its reference counterpart makes
+(LConv::forward -> Conv2D, LBatchNorm::forward -> BatchNormForward in inference mode,
+LActivation -> ReLu/Sigmoid/FullSoftmax, LMaxPool -> MPool2D, LAveragePool -> AvgPool2D,
+LResize -> scale, LConcat -> concat, LAdd -> fill_+inc, LSum -> add, LPad -> pad,
+LDense -> mult2D + sum2D_rowwise, LReshape -> shared storage).
+
+``Net.build(backend, fuse=True)`` additionally runs a fusion pass in the spirit of the
+reference's FPGA model transformation (src/apis/fpga.cpp:173-331,656+): chains
+Pad(0) -> Conv -> BatchNorm -> Add -> ReLU whose intermediate results have one consumer become
+ONE convolution launch with a fused epilogue.  The arithmetic per element is unchanged
+(same operations, same order, each rounded to fp32).
+"""
+import numpy as np
+
+from .descriptors import ConvolDescriptor, PoolDescriptor, msg
+
+
+class Layer:
+    """A node of the graph: ``kind``, parents, output shape (batch first) and host parameters."""
+    _count = {}
+
+    def __init__(self, kind, parents, out_shape, name="", **attrs):
+        Layer._count[kind] = Layer._count.get(kind, 0) + 1
+        self.kind = kind
+        self.name = name or "%s%d" % (kind, Layer._count[kind])
+        self.parents = list(parents)
+        self.children = []
+        for p in self.parents:
+            p.children.append(self)
+        self.out_shape = [int(d) for d in out_shape]
+        self.attrs = attrs
+        self.params = {}  # name -> float32 numpy array (host copy; pushed to the device by Net.build)
+
+    def __repr__(self):
+        return "<%s %s %s>" % (self.kind, self.name, self.out_shape)
+
+
+class AsymmetricPaddingException(RuntimeError):
+    """Raised like the reference's (src/layers/conv/layer_conv2D.cpp:57-61)."""
+
+    def __init__(self, text, pads):
+        super().__init__(text)
+        self.pads = list(pads)
+
+
+# ---------------------------------------------------------------------------- layer factories
+def Input(shape, batch=1, name=""):
+    """``shape`` excludes the batch dimension, as in eddl::Input."""
+    return Layer("input", [], [batch] + list(shape), name)
+
+
+def Conv2D(parent, filters, kernel_size, strides=(1, 1), padding="same", use_bias=True, groups=1, dilation_rate=(1, 1), name="",
+           pads=()):
+    """eddl::Conv2D; ``padding="custom"`` with ``pads=[top, bottom, left, right]`` is the LConv constructor form."""
+    if len(parent.out_shape) != 4:
+        msg("LConv only works over 4D tensors", "LConv::LConv")
+    cd = ConvolDescriptor(filters, kernel_size, strides, padding, pads, groups, dilation_rate, use_bias).build(parent.out_shape)
+    l = Layer("conv2d", [parent], cd.out_shape, name, cd=cd)
+    if cd.pads[0] != cd.pads[1] or cd.pads[2] != cd.pads[3]:
+        raise AsymmetricPaddingException(
+            "In layer %s: Padding asymmetry detected (top=%d, bottom=%d, left=%d, right=%d). The padding asymmetry is not "
+            "allowed in a Conv layer, we suggest you to use an explicit padding layer before this layer to fix the asymmetry."
+            % (l.name, cd.pads[0], cd.pads[1], cd.pads[2], cd.pads[3]), cd.pads)
+    l.params["K"] = np.zeros(cd.K_shape, np.float32)
+    l.params["bias"] = np.zeros(cd.nk, np.float32)
+    return l
+
+
+def BatchNormalization(parent, affine=True, momentum=0.99, epsilon=1e-3, name=""):
+    C = parent.out_shape[1]
+    l = Layer("batchnorm", [parent], parent.out_shape, name, affine=affine, momentum=momentum, epsilon=float(epsilon))
+    # parameter order of the reference layer: bn_g, bn_b, mean, variance (layer_batchnorm.cpp:70-71)
+    if affine:
+        l.params["bn_g"] = np.ones(C, np.float32)
+        l.params["bn_b"] = np.zeros(C, np.float32)
+    l.params["mean"] = np.zeros(C, np.float32)
+    l.params["variance"] = np.ones(C, np.float32)
+    return l
+
+
+def ReLu(parent, name=""):
+    return Layer("relu", [parent], parent.out_shape, name)
+
+
+def Sigmoid(parent, name=""):
+    return Layer("sigmoid", [parent], parent.out_shape, name)
+
+
+def Softmax(parent, axis=-1, name=""):
+    nd = len(parent.out_shape)
+    if axis < 0:
+        axis += nd
+    if axis <= 0 or axis >= nd:
+        msg("The axis of a softmax must not be the batch", "LActivation::LActivation")
+    return Layer("softmax", [parent], parent.out_shape, name, axis=axis)
+
+
+def _pool(kind, parent, pool_size, strides, padding, name):
+    pd = PoolDescriptor(pool_size, strides, padding).build(parent.out_shape)
+    if pd.loop_rows != pd.r or pd.loop_cols != pd.c:
+        msg("pooling window walk (%dx%d) disagrees with the descriptor's output shape (%dx%d)"
+            % (pd.loop_rows, pd.loop_cols, pd.r, pd.c), "LPool::LPool")
+    return Layer(kind, [parent], pd.out_shape, name, pd=pd)
+
+
+def MaxPool2D(parent, pool_size=(2, 2), strides=(2, 2), padding="none", name=""):
+    """``padding`` may also be a 4-list [top, bottom, left, right] (the LMaxPool vector<int> constructor)."""
+    return _pool("maxpool2d", parent, pool_size, strides, padding, name)
+
+
+def AveragePool2D(parent, pool_size=(2, 2), strides=(2, 2), padding="none", name=""):
+    return _pool("avgpool2d", parent, pool_size, strides, padding, name)
+
+
+def GlobalAveragePool2D(parent, name=""):
+    if len(parent.out_shape) != 4:
+        msg("GlobalAveragePool only works over 4D tensors", "GlobalAveragePool2D")
+    return AveragePool2D(parent, [parent.out_shape[2], parent.out_shape[3]], [1, 1], "none", name or "GlobalAveragePool2D")
+
+
+def UpSampling2D(parent, size, interpolation="nearest", name=""):
+    if len(parent.out_shape) != 4:
+        msg("The number of dimensions of the input tensor must be 4", "EDDL::UpSampling2D")
+    if len(size) != 2:
+        msg('The number of dimensions of the "size" parameter must be 2', "EDDL::UpSampling2D")
+    if min(size) < 1:
+        msg('The scale factors in "size" parameter must be greater or equal to 1', "EDDL::UpSampling2D")
+    s = parent.out_shape
+    target = [s[2] * size[0], s[3] * size[1]]
+    return Layer("resize", [parent], [s[0], s[1]] + target, name, new_shape=target)
+
+
+def Concat(layers, axis=0, name=""):
+    """``axis`` excludes the batch dimension (0 = channels), as in eddl::Concat."""
+    if len(layers) < 2:
+        msg("Concat requires a minimum of two tensors", "Tensor::concat")
+    ax = axis + 1
+    shape = list(layers[0].out_shape)
+    for l in layers[1:]:
+        if len(l.out_shape) != len(shape):
+            msg("The number of dimensions of all tensors must match", "Tensor::concat")
+        for j, (a, b) in enumerate(zip(shape, l.out_shape)):
+            if j != ax and a != b:
+                msg("The dimensions across of all tensors must match (%d!=%d)" % (a, b), "Tensor::concat")
+        shape[ax] += l.out_shape[ax]
+    return Layer("concat", layers, shape, name, axis=ax)
+
+
+def Add(l1, l2=None, name=""):
+    """eddl::Add(l1, l2) (an LSum: one add) or eddl::Add({l1, l2, ...}) (an LAdd: fill_(0) then inc per parent)."""
+    if l2 is None:
+        layers = list(l1)
+        for l in layers[1:]:
+            if l.out_shape != layers[0].out_shape:
+                msg("Error adding layers with different tensor shape", "LAdd::LAdd")
+        return Layer("add_n", layers, layers[0].out_shape, name)
+    if l1.out_shape != l2.out_shape:
+        msg("Error adding layers with different tensor shape", "LSum::LSum")
+    return Layer("sum", [l1, l2], l1.out_shape, name)
+
+
+def Pad(parent, pads, constant=0.0, name=""):
+    """``pads`` = [top, right, bottom, left], or [rows, cols]."""
+    if len(pads) == 2:
+        pads = [pads[0], pads[1], pads[0], pads[1]]
+    elif len(pads) != 4:
+        msg("The padding on each border must follow this format (top-bottom, left-right) or (top, right, bottom, left)", "LPad::LPad")
+    if min(pads) < 0:
+        msg("Pad margin must be greater or equal than zero", "Tensor::pad")
+    s = parent.out_shape
+    return Layer("pad", [parent], [s[0], s[1], s[2] + pads[0] + pads[2], s[3] + pads[1] + pads[3]], name, pads=list(pads),
+                 constant=float(constant))
+
+
+def Reshape(parent, shape, name=""):
+    """``shape`` excludes the batch; one entry may be -1."""
+    per_image = int(np.prod(parent.out_shape[1:]))
+    shape = list(shape)
+    if shape.count(-1) > 1:
+        msg("Ambiguous reshape, more than one -1", "Reshape")
+    if -1 in shape:
+        known = int(np.prod([d for d in shape if d != -1])) if len(shape) > 1 else 1
+        shape[shape.index(-1)] = per_image // known
+    if int(np.prod(shape)) != per_image:
+        msg("Incompatible shapes", "Reshape")
+    return Layer("reshape", [parent], [parent.out_shape[0]] + shape, name)
+
+
+def Flatten(parent, name=""):
+    return Reshape(parent, [-1], name)
+
+
+def Dense(parent, ndim, use_bias=True, name=""):
+    in_dim = parent.out_shape[-1]
+    l = Layer("dense", [parent], parent.out_shape[:-1] + [ndim], name, use_bias=use_bias)
+    l.params["W"] = np.zeros((in_dim, ndim), np.float32)  # [in, out], as the reference stores it
+    l.params["bias"] = np.zeros(ndim, np.float32)
+    return l
+
+
+# ---------------------------------------------------------------------------- the net
+class Op:
+    """One launch group of the built plan.  ``flops``/``bytes`` are the algorithmic figures
+    (convolution: 2*N*K*C*R*S*P*Q and 4*(in + filters + out); bandwidth operators: bytes moved once)."""
+
+    def __init__(self, kind, name, run, flops=0, nbytes=0, layers=()):
+        self.kind, self.name, self.run, self.flops, self.bytes, self.layers = kind, name, run, flops, nbytes, list(layers)
+
+
+class Net:
+    def __init__(self, inputs, outputs):
+        self.lin, self.lout = list(inputs), list(outputs)
+        self.layers = self._topological()
+        self.backend = None
+
+    def _topological(self):
+        order, seen = [], set()
+
+        def visit(l):
+            if id(l) in seen:
+                return
+            seen.add(id(l))
+            for p in l.parents:
+                visit(p)
+            order.append(l)
+
+        for o in self.lout:
+            visit(o)
+        for i in self.lin:
+            if id(i) not in seen:
+                msg("input layer %s does not reach an output" % i.name, "Net::build")
+        return order
+
+    # ---- parameters (host side), in the reference's per-layer order
+    def get_parameters(self):
+        return [[p.copy() for p in l.params.values()] for l in self.layers]
+
+    def set_parameters(self, params):
+        for l, ps in zip(self.layers, params):
+            for key, v in zip(list(l.params), ps):
+                if tuple(v.shape) != l.params[key].shape:
+                    msg("parameter %s of %s has shape %s, expected %s" % (key, l.name, v.shape, l.params[key].shape), "Net::set_parameters")
+                l.params[key] = np.ascontiguousarray(v, np.float32)
+        if self.backend is not None:
+            self._push_parameters()
+
+    def _push_parameters(self):
+        for l in self.layers:
+            for key, v in l.params.items():
+                self.dparams[id(l)][key].copy_from(v)
+
+    # ---- build
+    def build(self, backend, fuse=True):
+        self.backend = hip = backend
+        self.fused = fuse
+        self.dparams = {id(l): {k: hip.empty(v.shape) for k, v in l.params.items()} for l in self.layers}
+        self._push_parameters()
+        self.out = {}   # id(layer) -> DeviceTensor holding its output (absent for layers folded into a fused op)
+        self.aux = {}   # id(layer) -> extra tensors (pool indices, bn side outputs)
+        self.ops = []
+        absorbed = set()
+        sole_child = lambda l: l.children[0] if len(l.children) == 1 and l not in self.lout else None
+
+        for l in self.layers:
+            if id(l) in absorbed:
+                continue
+            if l.kind == "input":
+                self.out[id(l)] = hip.empty(l.out_shape)
+                continue
+            if fuse and l.kind == "pad" and l.attrs["constant"] == 0.0:
+                c = sole_child(l)
+                if c is not None and c.kind == "conv2d":
+                    continue  # folded into the convolution below (its op is emitted when the conv is reached)
+            if l.kind == "conv2d":
+                self._emit_conv(l, fuse, absorbed, sole_child)
+                continue
+            self._emit_plain(l)
+        for o in self.lout:
+            if id(o) not in self.out:
+                msg("output layer %s was fused away" % o.name, "Net::build")
+        return self
+
+    def _emit_conv(self, l, fuse, absorbed, sole_child):
+        hip, cd = self.backend, l.attrs["cd"]
+        src = l.parents[0]
+        pt, pl = cd.padrt, cd.padcl
+        if fuse and src.kind == "pad" and id(src) not in self.out:
+            t, r, b, le = src.attrs["pads"]  # (top, right, bottom, left) -> added to the conv's top/left
+            pt, pl = pt + t, pl + le
+            src = src.parents[0]
+        bn = res = None
+        relu = False
+        last = l
+        if fuse:
+            c = sole_child(last)
+            if c is not None and c.kind == "batchnorm":
+                bn, last = c, c
+                c = sole_child(last)
+            if c is not None and c.kind == "sum":
+                other = c.parents[1] if c.parents[0] is last else c.parents[0]
+                if id(other) in self.out and other is not last:
+                    res, last = other, c
+                    c = sole_child(last)
+            if c is not None and c.kind == "relu":
+                relu, last = True, c
+        # collect absorbed layers (everything between l and last)
+        chain = []
+        cur = l
+        while cur is not last:
+            cur = cur.children[0]
+            chain.append(cur)
+        for m in chain:
+            absorbed.add(id(m))
+        O = hip.empty(last.out_shape)
+        self.out[id(last)] = O
+        I = self.out[id(src)]
+        dp = self.dparams[id(l)]
+        bias = dp["bias"] if cd.use_bias else None
+        dbn = None
+        if bn is not None:
+            bp = self.dparams[id(bn)]
+            dbn = (bp.get("bn_g"), bp.get("bn_b"), bp["mean"], bp["variance"], bn.attrs["epsilon"])
+        R = self.out[id(res)] if res is not None else None
+        N, Kf, P, Q = cd.out_shape
+        _, C, H, W = src.out_shape
+        flops = 2 * N * Kf * cd.kz * cd.kr * cd.kc * P * Q
+        nbytes = 4 * (N * C * H * W + Kf * cd.kz * cd.kr * cd.kc + N * Kf * P * Q)
+        name = "+".join(m.name for m in ([l] if not chain else [l] + chain))
+        if src is not l.parents[0]:
+            name = l.parents[0].name + "+" + name
+        self.ops.append(Op("conv2d", name, lambda: hip.conv2D(I, dp["K"], bias, O, cd.sr, cd.sc, pt, pl, bn=dbn, residual=R, relu=relu),
+                           flops, nbytes, [l] + chain))
+
+    def _emit_plain(self, l):
+        hip = self.backend
+        k = l.kind
+        ins = [self.out[id(p)] for p in l.parents]
+        n_out = int(np.prod(l.out_shape))
+        if k == "reshape":
+            self.out[id(l)] = ins[0].reshape(l.out_shape)  # shares storage; forward does nothing
+            return
+        O = hip.empty(l.out_shape)
+        self.out[id(l)] = O
+        if k == "batchnorm":
+            dp = self.dparams[id(l)]
+            C = l.out_shape[1]
+            opa = hip.empty(l.out_shape) if l.attrs["affine"] else None
+            bn_var = hip.empty((C,))
+            self.aux[id(l)] = {"opa": opa, "bn_var": bn_var}
+            run = lambda: hip.batchnorm_inference(ins[0], O, opa, dp["mean"], dp["variance"], dp.get("bn_g"), dp.get("bn_b"), bn_var,
+                                                  l.attrs["epsilon"])
+            nbytes = 8 * n_out + 16 * C
+        elif k == "relu":
+            run, nbytes = (lambda: hip.relu(ins[0], O)), 8 * n_out
+        elif k == "sigmoid":
+            run, nbytes = (lambda: hip.sigmoid(ins[0], O)), 8 * n_out
+        elif k == "softmax":
+            run, nbytes = (lambda: hip.full_softmax(ins[0], O, l.attrs["axis"])), 8 * n_out
+        elif k in ("maxpool2d", "avgpool2d"):
+            pd = l.attrs["pd"]
+            n_in = int(np.prod(l.parents[0].out_shape))
+            if k == "maxpool2d":
+                ix, iy = hip.full(l.out_shape, 0.0), hip.full(l.out_shape, 0.0)
+                self.aux[id(l)] = {"indX": ix, "indY": iy}
+                run, nbytes = (lambda: hip.mpool2D(ins[0], O, ix, iy, pd.ksize, pd.stride, pd.pad)), 4 * n_in + 12 * n_out
+            else:
+                run, nbytes = (lambda: hip.avgpool2D(ins[0], O, pd.ksize, pd.stride, pd.pad)), 4 * (n_in + n_out)
+        elif k == "resize":
+            n_in = int(np.prod(l.parents[0].out_shape))
+            run, nbytes = (lambda: hip.scale(ins[0], O, l.attrs["new_shape"])), 4 * (n_in + n_out)
+        elif k == "concat":
+            run, nbytes = (lambda: hip.concat(O, ins, l.attrs["axis"])), 8 * n_out
+        elif k == "sum":
+            run, nbytes = (lambda: hip.add(1.0, ins[0], 1.0, ins[1], O, 0)), 12 * n_out
+        elif k == "add_n":
+            def run():
+                hip.fill_(O, 0.0)
+                for t in ins:
+                    hip.inc(t, O)
+            nbytes = 4 * n_out * (1 + 3 * len(ins))
+        elif k == "pad":
+            hip.fill_(O, l.attrs["constant"])  # the border is written once, here; forward copies the interior
+            n_in = int(np.prod(l.parents[0].out_shape))
+            run, nbytes = (lambda: hip.pad(ins[0], O, l.attrs["pads"])), 8 * n_in
+        elif k == "dense":
+            dp = self.dparams[id(l)]
+            in_dim, ndim = dp["W"].shape
+            rows = n_out // ndim
+            A2, C2 = ins[0].reshape((rows, in_dim)), O.reshape((rows, ndim))
+            use_bias = l.attrs["use_bias"]
+
+            def run():
+                hip.mult2D(A2, dp["W"], C2, 0)
+                if use_bias:
+                    hip.sum2D_rowwise(C2, dp["bias"], C2)
+            self.ops.append(Op("dense", l.name, run, 2 * rows * in_dim * ndim, 4 * (rows * in_dim + in_dim * ndim + rows * ndim), [l]))
+            return
+        else:
+            msg("layer kind %s has no forward on this backend" % k, "Net::build")
+        self.ops.append(Op(k, l.name, run, 0, nbytes, [l]))
+
+    # ---- run
+    def resize(self, batch):
+        """Change the batch size: every output and scratch tensor is re-created (pointers change)."""
+        for l in self.layers:
+            l.out_shape[0] = batch
+            for key in ("cd", "pd"):
+                if key in l.attrs:
+                    l.attrs[key].resize(batch)
+        return self.build(self.backend, self.fused)
+
+    def forward(self, xs):
+        """``xs``: one array (or DeviceTensor) per input layer.  Returns the output DeviceTensors;
+        the launches are queued, not awaited."""
+        if not isinstance(xs, (list, tuple)):
+            xs = [xs]
+        if len(xs) != len(self.lin):
+            msg("Number of input tensors does not match the number of input layers", "Net::forward")
+        batch = xs[0].shape[0]
+        if batch != self.lin[0].out_shape[0]:
+            self.resize(batch)
+        for l, x in zip(self.lin, xs):
+            dst = self.out[id(l)]
+            if tuple(x.shape) != dst.shape:
+                msg("input shape %s does not match %s" % (tuple(x.shape), dst.shape), "Net::forward")
+            if isinstance(x, np.ndarray):
+                dst.copy_from(x)
+            elif x is not dst:
+                self.backend._check(self.backend.lib.eddlhip_memcpy_d2d(self.backend.dev, dst.ptr, x.ptr, dst.nbytes))
+        self.run()
+        return [self.out[id(o)] for o in self.lout]
+
+    def run(self):
+        """Queue every op of the plan on the device's stream (inputs already resident)."""
+        for op in self.ops:
+            op.run()
+
+    def predict(self, xs):
+        """Inference forward; returns host arrays (the reference's predict collects outputs to the CPU)."""
+        outs = self.forward(xs)
+        return [o.numpy() for o in outs]
+
+    def input_tensor(self, i=0):
+        return self.out[id(self.lin[i])]
+
+    def output_of(self, layer):
+        return self.out.get(id(layer))

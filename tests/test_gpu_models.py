@@ -1,0 +1,128 @@
+"""Model-level parity: every layer of the benchmark graphs (at reduced sizes) against the CPU
+oracle GIVEN THE DEVICE'S OWN INPUT to that layer, then fused plan == unfused plan bit for bit.
+
+Checking each layer on the device's own input separates kernel parity (the 1e-4 bar, or
+bit-exactness) from the growth of rounding differences through a deep net."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+EXACT = {"batchnorm", "relu", "maxpool2d", "avgpool2d", "resize", "concat", "sum", "add_n", "pad", "reshape"}
+
+
+def layer_oracle(ora, l, ins):
+    k = l.kind
+    if k == "conv2d":
+        cd = l.attrs["cd"]
+        return ora.conv2d(ins[0], l.params["K"], l.params["bias"] if cd.use_bias else None, (cd.sr, cd.sc), cd.padrt, cd.padcl,
+                          cd.r, cd.c, algo="im2col")
+    if k == "batchnorm":
+        return ora.batchnorm_inference(ins[0], l.params["mean"], l.params["variance"], l.params.get("bn_g"), l.params.get("bn_b"),
+                                       l.attrs["epsilon"])[0]
+    if k == "relu":
+        return ora.relu(ins[0])
+    if k == "sigmoid":
+        return ora.sigmoid(ins[0])
+    if k == "softmax":
+        return ora.softmax(ins[0], l.attrs["axis"])
+    if k == "maxpool2d":
+        pd = l.attrs["pd"]
+        return ora.maxpool2d(ins[0], pd.ksize, pd.stride, pd.pad, fill=0.0)
+    if k == "avgpool2d":
+        pd = l.attrs["pd"]
+        return ora.avgpool2d(ins[0], pd.ksize, pd.stride, pd.pad)
+    if k == "resize":
+        return ora.scale_nearest(ins[0], l.attrs["new_shape"])
+    if k == "concat":
+        return ora.concat(ins, l.attrs["axis"])
+    if k == "sum":
+        return ora.add(ins[0], ins[1])
+    if k == "pad":
+        return ora.pad(ins[0], l.attrs["pads"], l.attrs["constant"])
+    if k == "reshape":
+        return ins[0].reshape(l.out_shape)
+    if k == "dense":
+        return ora.dense(ins[0].reshape(-1, ins[0].shape[-1]), l.params["W"], l.params["bias"] if l.attrs["use_bias"] else None)
+    raise AssertionError(k)
+
+
+def check_model(hip, ora, model, x, seed):
+    from eddl_amd import models
+    models.init_he_normal(model, seed)
+    model.build(hip, fuse=False)
+    outs_unfused = [o.copy() for o in model.predict([x])]
+    dev = {id(l): model.output_of(l).numpy() for l in model.layers}
+    for l in model.layers:
+        if l.kind == "input":
+            continue
+        ins = [dev[id(p)] for p in l.parents]
+        ref = layer_oracle(ora, l, ins)
+        got = dev[id(l)]
+        if l.kind == "maxpool2d":
+            ref, ix, iy = ref
+            aux = model.aux[id(l)]
+            assert np.array_equal(aux["indX"].numpy(), ix) and np.array_equal(aux["indY"].numpy(), iy), l.name
+        ref = ref.reshape(got.shape)
+        if l.kind in EXACT:
+            assert np.array_equal(ref, got), l.name
+        else:
+            atol = 1e-5 * float(np.abs(ref).max())
+            assert np.all(np.abs(ref - got) <= atol + 1e-4 * np.abs(ref)), "%s: max err %g" % (l.name, np.abs(ref - got).max())
+    n_unfused = len(model.ops)
+    model.build(hip, fuse=True)
+    outs_fused = model.predict([x])
+    assert len(model.ops) < n_unfused
+    for a, b in zip(outs_unfused, outs_fused):
+        assert np.array_equal(a, b), "fused plan differs from the layer-by-layer plan"
+    return outs_fused
+
+
+def test_block(hip, oracle):
+    from eddl_amd import models
+    m = models.conv_bn_relu_pool_block(batch=4, channels=64, size=56, filters=64)
+    x = np.random.default_rng(2).standard_normal((4, 64, 56, 56), dtype=np.float32)
+    check_model(hip, oracle, m, x, 2)
+    assert [op.kind for op in m.ops] == ["conv2d", "maxpool2d"]
+
+
+def test_vgg16_small(hip, oracle):
+    from eddl_amd import models
+    m = models.vgg16(batch=2, size=32, num_classes=10, dense=128)
+    x = np.random.default_rng(3).uniform(0, 1, (2, 3, 32, 32)).astype(np.float32)
+    out = check_model(hip, oracle, m, x, 3)[0]
+    np.testing.assert_allclose(out.sum(1), 1.0, rtol=1e-5)
+    assert sum(op.kind == "conv2d" for op in m.ops) == 13 and not any(op.kind == "relu" and "conv" in op.name for op in m.ops)
+
+
+def test_resnet50_small(hip, oracle):
+    from eddl_amd import models
+    m = models.resnet50(batch=2, size=64, num_classes=10, base=16)
+    x = np.random.default_rng(4).standard_normal((2, 3, 64, 64), dtype=np.float32)
+    check_model(hip, oracle, m, x, 4)
+    kinds = [op.kind for op in m.ops]
+    assert kinds.count("conv2d") == 53 and "sum" not in kinds and "batchnorm" not in kinds and "relu" not in kinds
+
+
+def test_unet_small(hip, oracle):
+    from eddl_amd import models
+    m = models.unet(batch=1, size=64, widths=(8, 16, 32, 64), bottleneck=128)
+    x = np.random.default_rng(5).uniform(0, 1, (1, 1, 64, 64)).astype(np.float32)
+    check_model(hip, oracle, m, x, 5)
+    kinds = [op.kind for op in m.ops]
+    assert "pad" not in kinds and "batchnorm" not in kinds and kinds.count("conv2d") == 23
+
+
+def test_batch_resize_and_asymmetric_padding_exception(hip, oracle):
+    from eddl_amd import models, net as L
+    m = models.conv_bn_relu_pool_block(batch=2, channels=8, size=12, filters=8)
+    models.init_he_normal(m, 9)
+    m.build(hip)
+    x = np.random.default_rng(9).standard_normal((5, 8, 12, 12), dtype=np.float32)
+    y5 = m.predict([x])[0]          # batch 2 -> 5: every tensor re-created
+    y3 = m.predict([x[:3]])[0]
+    assert y5.shape == (5, 8, 6, 6) and np.array_equal(y5[:3], y3)
+    with pytest.raises(L.AsymmetricPaddingException):
+        L.Conv2D(L.Input([3, 224, 224], 1), 64, [7, 7], [2, 2], "same")
+    with pytest.raises(L.AsymmetricPaddingException):
+        L.Conv2D(L.Input([3, 8, 8], 1), 4, [2, 2], [1, 1], "same")
