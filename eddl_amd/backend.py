@@ -137,6 +137,10 @@ class Backend:
     def set_conv_algo(self, algo):
         self._check(self.lib.eddlhip_conv2d_set_algo({"auto": 0, "mfma": 1, "direct": 2}.get(algo, algo)))
 
+    def set_conv_profile_events(self, start=None, stop=None):
+        """Bracket the matrix-core kernel of the following conv2D calls with two events (None, None removes them)."""
+        self._check(self.lib.eddlhip_conv2d_set_profile_events(start.handle if start else None, stop.handle if stop else None))
+
     # ---- operators (names follow the reference's gpu_* functions)
     def fill_(self, A, v):
         self._check(self.lib.eddlhip_fill(self.dev, A.ptr, A.size, v))

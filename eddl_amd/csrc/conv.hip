@@ -293,6 +293,7 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvParams p) {
 }
 
 int g_algo = 0;
+hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;  // optional: bracket the main kernel of the next calls
 
 template <int WM, int WN, int TM, int TN>
 int launch_igemm(hipStream_t st, ConvParams &p) {
@@ -302,10 +303,12 @@ int launch_igemm(hipStream_t st, ConvParams &p) {
     EH_REQUIRE(gn * p.gm <= 0x7fffffffLL, "conv2d: too many tiles");
     p.gn = (int)gn;
     dim3 grid((unsigned)(gn * p.gm)), block(256);
+    if (g_prof_start) EH_TRY_HIP(hipEventRecord(g_prof_start, st));
     if (p.R == 3 && p.S == 3) hipLaunchKernelGGL((conv_igemm_kernel<WM, WN, TM, TN, 3, 3>), grid, block, 0, st, p);
     else if (p.R == 1 && p.S == 1) hipLaunchKernelGGL((conv_igemm_kernel<WM, WN, TM, TN, 1, 1>), grid, block, 0, st, p);
     else hipLaunchKernelGGL((conv_igemm_kernel<WM, WN, TM, TN, 0, 0>), grid, block, 0, st, p);
     EH_CHECK_LAUNCH();
+    if (g_prof_stop) EH_TRY_HIP(hipEventRecord(g_prof_stop, st));
     return 0;
 }
 
@@ -316,6 +319,13 @@ extern "C" {
 int eddlhip_conv2d_set_algo(int algo) {
     EH_REQUIRE(algo >= 0 && algo <= 2, "conv2d_set_algo: unknown algorithm %d", algo);
     g_algo = algo;
+    return 0;
+}
+
+int eddlhip_conv2d_set_profile_events(void *start, void *stop) {
+    EH_REQUIRE((start == nullptr) == (stop == nullptr), "conv2d_set_profile_events: give both events or neither");
+    g_prof_start = (hipEvent_t)start;
+    g_prof_stop = (hipEvent_t)stop;
     return 0;
 }
 

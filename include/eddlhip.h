@@ -95,6 +95,12 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
  * reference's ky,kx,c order - used to cross-check the MFMA kernels on the device). */
 int eddlhip_conv2d_set_algo(int algo);
 
+/* Measurement hook (no counterpart in the reference): while two events are installed, every
+ * eddlhip_conv2d_fwd records `start` on the device's stream immediately before its main
+ * (matrix-core) kernel and `stop` immediately after it, leaving the filter repack outside the
+ * bracket.  Pass NULL, NULL to remove them. */
+int eddlhip_conv2d_set_profile_events(void *start, void *stop);
+
 /* ------------------------------------------------------------------ batch normalisation (inference)
  * Replaces gpu_batchnorm_forward(...) with trmode == false
  * (include/eddl/hardware/gpu/nn/gpu_tensor_nn.h:138-143, src/hardware/gpu/nn/gpu_bn.cu:65-98;
