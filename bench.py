@@ -49,6 +49,7 @@ def time_ops(hip, model, reps):
     Convolutions are bracketed inside the library around the matrix-core kernel only."""
     n = len(model.ops)
     ev = [[(hip.event(), hip.event()) for _ in range(n)] for _ in range(reps)]
+    kernels = [None] * n
     for r in range(reps):
         for i, op in enumerate(model.ops):
             s, e = ev[r][i]
@@ -56,12 +57,13 @@ def time_ops(hip, model, reps):
                 hip.set_conv_profile_events(s, e)
                 op.run()
                 hip.set_conv_profile_events(None, None)
+                kernels[i] = hip.last_conv_kernel()
             else:
                 s.record()
                 op.run()
                 e.record()
     hip.synchronize()
-    return [float(np.mean([ev[r][i][0].elapsed_ms(ev[r][i][1]) for r in range(reps)])) for i in range(n)]
+    return [float(np.mean([ev[r][i][0].elapsed_ms(ev[r][i][1]) for r in range(reps)])) for i in range(n)], kernels
 
 
 def cpu_baseline(workload, want_seconds=20.0):
@@ -119,12 +121,14 @@ def main():
     ap.add_argument("--workload", default="vgg16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-op table to stderr")
+    ap.add_argument("--conv-algo", default="auto", choices=["auto", "mfma_staged", "mfma_lds"], help="input gather of the convolution kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on ONE GPU (the forward path has no collectives); --gpus %d is not supported" % args.gpus)
 
     import eddl_amd
     hip = eddl_amd.Backend(0)
+    hip.set_conv_algo(args.conv_algo)
     model, x, desc = build_workload(args.workload)
     model.build(hip, fuse=True)
     batch = x.shape[0]
@@ -146,10 +150,12 @@ def main():
 
     # ---- per-op device times (events on the kernels' stream), same resident input
     reps = max(3, min(args.steps, 10))
-    op_ms = time_ops(hip, model, reps)
+    op_ms, op_kernels = time_ops(hip, model, reps)
     rows = []
-    for op, ms in zip(model.ops, op_ms):
+    for op, ms, kern in zip(model.ops, op_ms, op_kernels):
         row = {"op": op.kind, "name": op.name, "ms": ms, "flops": op.flops, "bytes": op.bytes}
+        if kern:
+            row["kernel"] = kern
         if op.kind in ("conv2d", "dense") and ms > 0:
             row["tflops"] = op.flops / ms / 1e9
             row["frac_fp32_mfma_peak"] = row["tflops"] / PEAK_FP32_MFMA_TFLOPS
@@ -158,11 +164,13 @@ def main():
             row["frac_hbm_peak"] = row["gbs"] / PEAK_HBM_GBS
         rows.append(row)
 
-    # ---- dominant kernel: the matrix-core convolution launches that are compute-bound
-    # (arithmetic intensity above the fp32 ridge 157.3 TFLOP/s / 8 TB/s = 19.7 flop/byte)
+    # ---- dominant kernel: the convolution kernel (one template instance = one symbol in a
+    # rocprofv3 kernel trace) that accounts for the most device time in a step
     conv_rows = [r for r in rows if r["op"] == "conv2d"]
-    mfma_rows = [r for r in conv_rows if r["flops"] / max(r["bytes"], 1) > PEAK_FP32_MFMA_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)]
-    dom = mfma_rows or conv_rows
+    by_kernel = {}
+    for r in conv_rows:
+        by_kernel.setdefault(r.get("kernel", "?"), []).append(r)
+    dom_name, dom = max(by_kernel.items(), key=lambda kv: sum(r["ms"] for r in kv[1]))
     dom_flops, dom_ms = sum(r["flops"] for r in dom), sum(r["ms"] for r in dom)
     achieved = dom_flops / dom_ms / 1e9 if dom_ms > 0 else 0.0
     traffic = None
@@ -172,7 +180,7 @@ def main():
             traffic = json.load(fh).get("hbm_bytes_per_launch")
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": traffic,
-                "kernel": "conv_igemm_kernel (fp32 MFMA implicit GEMM)", "launches": len(dom),
+                "kernel": dom_name, "launches_per_step": len(dom),
                 "flops_per_launch": dom_flops / max(len(dom), 1), "avg_launch_ms": dom_ms / max(len(dom), 1)}
 
     conv_ms = sum(r["ms"] for r in conv_rows)
@@ -193,9 +201,10 @@ def main():
 
     table = ["%-44s %9s %9s %8s %9s %7s" % ("op", "ms", "TFLOP/s", "%mfma", "GB/s", "%hbm")]
     for r in rows:
-        table.append("%-44s %9.4f %9s %8s %9.1f %7.2f" % (
+        table.append("%-44s %9.4f %9s %8s %9.1f %7.2f  %s" % (
             r["name"][:44], r["ms"], "%.2f" % r["tflops"] if "tflops" in r else "-",
-            "%.1f" % (100 * r["frac_fp32_mfma_peak"]) if "tflops" in r else "-", r.get("gbs", 0.0), 100 * r.get("frac_hbm_peak", 0.0)))
+            "%.1f" % (100 * r["frac_fp32_mfma_peak"]) if "tflops" in r else "-", r.get("gbs", 0.0), 100 * r.get("frac_hbm_peak", 0.0),
+            r.get("kernel", "")))
     if args.layers:
         print("\n".join(table), file=sys.stderr)
     out_dir = os.path.join(ROOT, "gpurun_out")

@@ -35,6 +35,7 @@ PROTOTYPES = {
     "eddlhip_event_elapsed_ms": [c_int, c_void_p, c_void_p, ctypes.POINTER(c_float)],
     "eddlhip_conv2d_fwd": [c_int, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_set_algo": [c_int],
+    "eddlhip_conv2d_last_kernel": [],
     "eddlhip_conv2d_set_profile_events": [c_void_p, c_void_p],
     "eddlhip_batchnorm_inference": [c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, c_float],
     "eddlhip_relu": [c_int, P, P, c_size_t],
@@ -51,7 +52,8 @@ PROTOTYPES = {
     "eddlhip_mult2d": [c_int, P, P, P, c_int, c_int, c_int, c_int],
     "eddlhip_sum2d_rowwise": [c_int, P, P, P, c_int, c_int],
 }
-_RESTYPE = {"eddlhip_version": ctypes.c_char_p, "eddlhip_last_error": ctypes.c_char_p}
+_RESTYPE = {"eddlhip_version": ctypes.c_char_p, "eddlhip_last_error": ctypes.c_char_p,
+            "eddlhip_conv2d_last_kernel": ctypes.c_char_p}
 
 
 def load():

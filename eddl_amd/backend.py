@@ -135,7 +135,10 @@ class Backend:
         return t
 
     def set_conv_algo(self, algo):
-        self._check(self.lib.eddlhip_conv2d_set_algo({"auto": 0, "mfma": 1, "direct": 2}.get(algo, algo)))
+        self._check(self.lib.eddlhip_conv2d_set_algo({"auto": 0, "mfma": 1, "direct": 2, "mfma_staged": 3, "mfma_lds": 4}.get(algo, algo)))
+
+    def last_conv_kernel(self):
+        return self.lib.eddlhip_conv2d_last_kernel().decode()
 
     def set_conv_profile_events(self, start=None, stop=None):
         """Bracket the matrix-core kernel of the following conv2D calls with two events (None, None removes them)."""

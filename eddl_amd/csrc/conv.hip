@@ -6,26 +6,37 @@
 //     O[m][n] = sum_i  Wt[i][m] * Col[i][n]
 //     m = output channel, n = flattened (image, p, q) output pixel,
 //     i = (c, ky, kx) tap, c slowest  - the order of OIHW filter memory.
-// Col is never stored: each workgroup gathers the 16 x BN slice it needs straight from the
-// NCHW input into LDS (out-of-image taps become 0).  Filters are repacked once per call into
-// a tap-major, zero-padded matrix Wp[i][m] (private workspace) so that the filter slice of a
-// tile is 16 rows of contiguous floats: 16-byte global loads, 16-byte LDS stores.
+// Col is never stored: each workgroup gathers the BK x BN slice it needs straight from the
+// NCHW input into LDS.  The gather uses buffer loads: a tap that falls outside the image gets
+// an out-of-range offset and the hardware returns 0 for it - no branch, no select.  Filters are
+// repacked once per call into a tap-major, zero-padded matrix Wp[i][m] (private workspace) so
+// that the filter slice of a tile is BK rows of contiguous floats (16-byte loads).
 //
-// Tile: BM x BN outputs per 256-thread workgroup (4 wavefronts), K-step 16 taps, LDS
-// double-buffered (one barrier per step), global loads of step t+1 issued before the MFMAs of
-// step t.  Each wavefront owns TM x TN blocks of 32x32 outputs and advances them with
-// v_mfma_f32_32x32x2_f32 (A = 32 channels x 2 taps, B = 2 taps x 32 pixels).
+// Tile: BM x BN outputs per 256-thread workgroup (4 wavefronts), LDS double-buffered (one
+// barrier per K-step), loads of step t+1 issued before the MFMAs of step t.  Each wavefront
+// owns TM x TN blocks of 32x32 outputs and advances them with v_mfma_f32_32x32x2_f32
+// (A = 32 channels x 2 taps, B = 2 taps x 32 pixels).
+//
+// Two kernels:
+//   conv_tap_kernel  filter shape known at compile time (3x3, 1x1, 2x2): a K-step is CPB whole
+//                    input channels; every thread gathers ONE fixed output pixel, so the R*S
+//                    tap offsets (and their validity) are computed once, before the loop, and
+//                    the per-step address work is one scalar offset per channel.  Optionally
+//                    the gather goes global -> LDS directly (buffer_load ... lds), skipping
+//                    the register file.
+//   conv_gen_kernel  any filter shape, K-step 16 taps, tap validity computed per element.
 //
 // Accumulation order per output: taps in increasing i, two per MFMA (the instruction adds
-// both products of a pair into the fp32 accumulator), all in one accumulator from the first
-// tap to the last; no split over taps.  The reference CPU order is ky,kx,c per output in its
-// direct form and Eigen-internal in its GEMM form, so agreement is to a tolerance, not
-// bit-for-bit; the scalar kernel at the end of this file follows the direct form's order and
-// rounding exactly.
+// both products of a pair into the fp32 accumulator), one accumulator from the first tap to
+// the last; no split over taps.  The reference CPU order is ky,kx,c per output in its direct
+// form and Eigen-internal in its GEMM form, so agreement is to a tolerance, not bit-for-bit;
+// the scalar kernel at the end of this file follows the direct form's order and rounding.
 //
 // Workgroups are numbered so that those running on one XCD (workgroup id mod 8) cover
 // neighbouring pixel tiles for all channel tiles: the input slice they share stays in that
 // XCD's L2.
+#include <stdio.h>
+
 #include "common.h"
 
 using namespace eddlhip;
@@ -33,13 +44,15 @@ using namespace eddlhip;
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void lds_void;
 
-constexpr int BK = 16;       // taps per pipeline step
-constexpr int M_ALIGN = 128; // packed filter rows are padded to this many channels
+constexpr int M_ALIGN = 128;                  // packed filter rows are padded to this many channels
+constexpr int OOB = (int)0x80000000u;         // byte offset no buffer of <= 2 GiB contains
+constexpr unsigned RSRC_WORD3 = 0x00020000u;  // raw buffer, 32-bit data format
 
 struct ConvParams {
     const float *I;
-    const float *Wp;  // packed filters [CRSp][Mp]
+    const float *Wp;  // packed filters [rows][Mp]
     const float *K;   // original OIHW filters (scalar kernel only)
     float *O;
     const float *bias, *bn_g, *bn_b, *bn_mean, *bn_var, *residual;
@@ -49,6 +62,7 @@ struct ConvParams {
     int CRS, Mp, nsteps, PQ;
     long long npix;
     int gm, gn;
+    unsigned in_bytes;  // size the input's buffer descriptor covers
 };
 
 // The fused tail of a Conv -> BatchNorm(inference) -> Add -> ReLU chain; every step rounded
@@ -86,11 +100,60 @@ __device__ __forceinline__ float apply_epilogue(const ConvParams &p, const Chann
     return v;
 }
 
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, int voffset, int soffset) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voffset, soffset, 0));
+}
+
+// workgroup id -> (channel tile, pixel tile); ids that share an XCD get consecutive tiles
+__device__ __forceinline__ void tile_of_block(const ConvParams &p, int &m_tile, int &n_tile) {
+    const unsigned total = gridDim.x, bid = blockIdx.x;
+    const unsigned q = total / EDDLHIP_NUM_XCD, r = total % EDDLHIP_NUM_XCD;
+    const unsigned xcd = bid % EDDLHIP_NUM_XCD, slot = bid / EDDLHIP_NUM_XCD;
+    const int vid = (int)((xcd < r ? xcd * (q + 1) : r * (q + 1) + (xcd - r) * q) + slot);
+    m_tile = vid % p.gm;
+    n_tile = vid / p.gm;
+}
+
+// Writes a wavefront's TM x TN blocks.  A lane holds column (pixel) lane%32 and rows
+// 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 block: for a fixed v the 32 lanes of a half
+// wavefront store 32 consecutive pixels of one channel plane (128 contiguous bytes).
+template <int TM, int TN>
+__device__ __forceinline__ void store_tile(const ConvParams &p, floatx16 (&acc)[TM][TN], int m_base, long long n_base, int lane) {
+    size_t obase[TN];
+    bool nok[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+        const long long n = n_base + tn * 32 + (lane & 31);
+        nok[tn] = n < p.npix;
+        const long long nc = nok[tn] ? n : 0;
+        const int img = (int)(nc / p.PQ);
+        const int pq = (int)(nc - (long long)img * p.PQ);
+        obase[tn] = (size_t)img * p.Kf * p.PQ + pq;
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int m = m_base + tm * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+            if (m < p.Kf) {
+                const ChannelEpilogue e = load_channel(p, m);
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) {
+                    if (nok[tn]) {
+                        const size_t oidx = obase[tn] + (size_t)m * p.PQ;
+                        p.O[oidx] = apply_epilogue(p, e, acc[tm][tn][v], oidx);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------- filter repack
-// K[Kf][CRS] (OIHW memory) -> Wp[CRSp][Mp], zero-padded; 32x32 tiles through LDS so that
+// K[Kf][CRS] (OIHW memory) -> Wp[rows][Mp], zero-padded; 32x32 tiles through LDS so that
 // both the read and the write are coalesced.
 __global__ __launch_bounds__(256) void pack_filters_kernel(const float *__restrict__ K, float *__restrict__ Wp, int Kf, int CRS,
-                                                           int Mp, int CRSp) {
+                                                           int Mp, int rows) {
     __shared__ float tile[32][33];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
     const int i0 = blockIdx.x * 32, m0 = blockIdx.y * 32;
@@ -103,80 +166,252 @@ __global__ __launch_bounds__(256) void pack_filters_kernel(const float *__restri
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         int i = i0 + ty + 8 * j, m = m0 + tx;
-        if (i < CRSp && m < Mp) Wp[(size_t)i * Mp + m] = tile[tx][ty + 8 * j];
+        if (i < rows && m < Mp) Wp[(size_t)i * Mp + m] = tile[tx][ty + 8 * j];
     }
 }
 
-// ---------------------------------------------------------------- implicit GEMM, fp32 MFMA
-template <int WM, int WN, int TM, int TN, int R_, int S_>
-__global__ __launch_bounds__(256) void conv_igemm_kernel(const ConvParams p) {
+// ---------------------------------------------------------------- MFMA kernel, compile-time filter shape
+// K-step = CPB input channels x (R*S) taps.  Gather work is split by wavefront: a wavefront
+// serves one 64-pixel segment of the tile (its lanes = 64 consecutive output pixels) and CPW of
+// the step's channels; each of its loads is one (channel, tap) row segment of 64 floats.
+template <int WM, int WN, int TM, int TN, int R, int S, int CPB, bool DIRECT>
+__global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
+    constexpr int RS = R * S, BK = CPB * RS;
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    constexpr int LDA = BM + 32, LDB = BN + 32;  // +32 floats: the two half-wavefronts of an operand read hit different banks
-    constexpr int AV = BM >= 64 ? BM / 64 : 1;   // float4 filter loads per thread per step
-    constexpr int A_VECS = BK * BM / 4;          // float4 in one filter slice (fewer than 256 when BM = 32)
-    constexpr int EPT = BN / 16;                 // gathered input elements per thread per step
-    static_assert(BN >= 64, "a wavefront gathers one tap row slice");
+    constexpr int NS = BN / 64;     // 64-pixel segments in a tile row
+    constexpr int WPS = 4 / NS;     // wavefronts that share a segment
+    constexpr int CPW = CPB / WPS;  // channels a wavefront gathers per step
+    static_assert(BK % 2 == 0, "an MFMA consumes two taps");
+    static_assert(NS == 1 || NS == 2 || NS == 4, "BN is 64, 128 or 256");
+    static_assert(CPB % WPS == 0, "channels of a step divide over the wavefronts of a segment");
+    constexpr int LDA = BM + 32, LDB = BN + 32;  // +32 floats: the two halves of an operand read use different banks
+    constexpr int A_VECS = BK * BM / 4;          // float4 in one filter slice
+    constexpr int AV = (A_VECS + 255) / 256;     // float4 filter loads per thread per step (last one partial)
 
     __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
-    const int R = R_ ? R_ : p.R, S = S_ ? S_ : p.S, RS = R * S;
-
-    // workgroup id -> tile, XCD-contiguous
-    int vid;
-    {
-        const unsigned total = gridDim.x, bid = blockIdx.x;
-        const unsigned q = total / EDDLHIP_NUM_XCD, r = total % EDDLHIP_NUM_XCD;
-        const unsigned xcd = bid % EDDLHIP_NUM_XCD, slot = bid / EDDLHIP_NUM_XCD;
-        vid = (int)((xcd < r ? xcd * (q + 1) : r * (q + 1) + (xcd - r) * q) + slot);
-    }
-    const int m_tile = vid % p.gm, n_tile = vid / p.gm;
+    int m_tile, n_tile;
+    tile_of_block(p, m_tile, n_tile);
     const int m0 = m_tile * BM;
     const long long n0 = (long long)n_tile * BN;
 
-    // ---- this thread's gathered pixel (fixed for the whole kernel)
-    const int bn_l = tid % BN;
-    const int bg = __builtin_amdgcn_readfirstlane(tid / BN);  // tap group, uniform in a wavefront
-    const long long ng = n0 + bn_l;
-    const bool pvalid = ng < p.npix;
-    int ih0, iw0;
-    const float *in_img;
+    const __amdgpu_buffer_rsrc_t rsrc_in = __builtin_amdgcn_make_buffer_rsrc((void *)p.I, 0, p.in_bytes, RSRC_WORD3);
+
+    // ---- this thread's gathered pixel and its R*S tap offsets (bytes; OOB where the tap leaves the image)
+    const int seg = wave % NS, cg = wave / NS;
+    int voff[RS];
     {
+        const long long ng = n0 + seg * 64 + lane;
+        const bool pvalid = ng < p.npix;
+        const long long ngc = pvalid ? ng : 0;
+        const int img = (int)(ngc / p.PQ);
+        const int pq = (int)(ngc - (long long)img * p.PQ);
+        const int op = pq / p.Q, oq = pq - op * p.Q;
+        const int ih0 = op * p.sr - p.pt, iw0 = oq * p.sc - p.pl;
+        const int pix = img * (p.C * p.H * p.W) + ih0 * p.W + iw0;
+#pragma unroll
+        for (int t = 0; t < RS; t++) {
+            const int ky = t / S, kx = t % S;
+            const bool ok = pvalid && (unsigned)(ih0 + ky) < (unsigned)p.H && (unsigned)(iw0 + kx) < (unsigned)p.W;
+            voff[t] = ok ? (pix + ky * p.W + kx) * 4 : OOB;
+        }
+    }
+    const int HW4 = p.H * p.W * 4;
+
+    // ---- filter slice: float4 f of the slice is row f / (BM/4), channels 4*(f % (BM/4))
+    // (plain 16-byte loads: the packed matrix is padded to whole steps and whole tiles, so every address exists)
+    const float *a_ptr[AV];
+    int a_lds[AV];
+#pragma unroll
+    for (int j = 0; j < AV; j++) {
+        const int f = tid + j * 256;
+        const int kk = f / (BM / 4), m4 = (f % (BM / 4)) * 4;
+        a_ptr[j] = p.Wp + (size_t)kk * p.Mp + m0 + m4;
+        a_lds[j] = kk * LDA + m4;
+    }
+    const int a_step = BK * p.Mp;
+
+    float4 areg[AV];
+    float breg[DIRECT ? 1 : CPW * RS];
+
+    auto a_active = [&](int j) -> bool {  // only the last, partial round of a slice tests anything
+        return (A_VECS % 256 == 0 || j < AV - 1) ? true : (tid + j * 256 < A_VECS);
+    };
+    auto load_a = [&](int step) {
+#pragma unroll
+        for (int j = 0; j < AV; j++)
+            if (a_active(j)) areg[j] = *reinterpret_cast<const float4 *>(a_ptr[j] + (size_t)step * a_step);
+    };
+    auto store_a = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < AV; j++)
+            if (a_active(j)) *reinterpret_cast<float4 *>(&As[buf][a_lds[j]]) = areg[j];
+    };
+    // gather of one step; `checked` adds the test for channels past C (last step of an odd channel count)
+    auto load_b = [&](int step, int buf, bool checked) {
+#pragma unroll
+        for (int jc = 0; jc < CPW; jc++) {
+            const int cl = cg * CPW + jc;
+            const int c = step * CPB + cl;
+            const bool cok = !checked || c < p.C;
+            const int soff = (cok ? c : 0) * HW4;
+#pragma unroll
+            for (int t = 0; t < RS; t++) {
+                const int vo = cok ? voff[t] : OOB;
+                if constexpr (DIRECT) {
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_void *)&Bs[buf][(cl * RS + t) * LDB + seg * 64], 4, vo, soff, 0, 0);
+                } else {
+                    breg[jc * RS + t] = buf_load(rsrc_in, vo, soff);
+                }
+            }
+        }
+    };
+    auto store_b = [&](int buf) {
+        if constexpr (!DIRECT) {
+#pragma unroll
+            for (int jc = 0; jc < CPW; jc++)
+#pragma unroll
+                for (int t = 0; t < RS; t++) Bs[buf][((cg * CPW + jc) * RS + t) * LDB + seg * 64 + lane] = breg[jc * RS + t];
+        }
+    };
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.0f;
+
+    const int full_steps = p.C / CPB;  // steps whose channels all exist
+    load_a(0);
+    load_b(0, 0, full_steps == 0);
+    store_a(0);
+    store_b(0);
+    __syncthreads();
+
+    const int a_off = (lane >> 5) * LDA + wm * TM * 32 + (lane & 31);
+    const int b_off = (lane >> 5) * LDB + wn * TN * 32 + (lane & 31);
+
+    for (int step = 0; step < p.nsteps; step++) {
+        const int buf = step & 1;
+        const bool more = step + 1 < p.nsteps;
+        if (more) {
+            load_a(step + 1);
+            if (step + 1 < full_steps) load_b(step + 1, buf ^ 1, false);
+            else load_b(step + 1, buf ^ 1, true);
+        }
+        // operands of tap pair ks+1 are read from LDS while the MFMAs of pair ks run
+        float a[2][TM], b[2][TN];
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++) a[0][tm] = As[buf][a_off + tm * 32];
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++) b[0][tn] = Bs[buf][b_off + tn * 32];
+#pragma unroll
+        for (int ks = 0; ks < BK / 2; ks++) {
+            const int cur = ks & 1, nxt = cur ^ 1;
+            if (ks + 1 < BK / 2) {
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++) a[nxt][tm] = As[buf][(ks + 1) * 2 * LDA + a_off + tm * 32];
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) b[nxt][tn] = Bs[buf][(ks + 1) * 2 * LDB + b_off + tn * 32];
+            }
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++)
+                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
+        }
+        if (more) {
+            store_a(buf ^ 1);
+            store_b(buf ^ 1);
+        }
+        __syncthreads();
+    }
+
+    store_tile<TM, TN>(p, acc, m0 + wm * TM * 32, n0 + wn * TN * 32, lane);
+}
+
+// ---------------------------------------------------------------- MFMA kernel, any filter shape
+// K-step = 16 taps.  Thread t gathers pixel t % BN for EPT consecutive taps of the step; the tap
+// walk (c, ky, kx) is uniform in a wavefront and advances with scalar arithmetic.
+template <int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(256) void conv_gen_kernel(const ConvParams p) {
+    static_assert(WM * WN == 4, "four wavefronts per workgroup");
+    constexpr int BK = 16;
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    constexpr int LDA = BM + 32, LDB = BN + 32;
+    constexpr int A_VECS = BK * BM / 4;
+    constexpr int AV = (A_VECS + 255) / 256;
+    constexpr int EPT = BN / 16;  // gathered elements per thread per step
+    static_assert(BN >= 64 && BN <= 256, "a wavefront gathers whole tap rows");
+
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int R = p.R, S = p.S, RS = R * S;
+    int m_tile, n_tile;
+    tile_of_block(p, m_tile, n_tile);
+    const int m0 = m_tile * BM;
+    const long long n0 = (long long)n_tile * BN;
+
+    const __amdgpu_buffer_rsrc_t rsrc_in = __builtin_amdgcn_make_buffer_rsrc((void *)p.I, 0, p.in_bytes, RSRC_WORD3);
+
+    const int bn_l = tid % BN;
+    const int bg = __builtin_amdgcn_readfirstlane(tid / BN);  // tap group (BN >= 64: uniform in a wavefront)
+    int ih0, iw0, pix;
+    bool pvalid;
+    {
+        const long long ng = n0 + bn_l;
+        pvalid = ng < p.npix;
         const long long ngc = pvalid ? ng : 0;
         const int img = (int)(ngc / p.PQ);
         const int pq = (int)(ngc - (long long)img * p.PQ);
         const int op = pq / p.Q, oq = pq - op * p.Q;
         ih0 = op * p.sr - p.pt;
         iw0 = oq * p.sc - p.pl;
-        in_img = p.I + (size_t)img * p.C * p.H * p.W;
+        pix = img * (p.C * p.H * p.W) + ih0 * p.W + iw0;
     }
+    const int HW4 = p.H * p.W * 4;
 
+    // (plain 16-byte loads: the packed matrix is padded to whole steps and whole tiles, so every address exists)
+    const float *a_ptr[AV];
+    int a_lds[AV];
+#pragma unroll
+    for (int j = 0; j < AV; j++) {
+        const int f = tid + j * 256;
+        const int kk = f / (BM / 4), m4 = (f % (BM / 4)) * 4;
+        a_ptr[j] = p.Wp + (size_t)kk * p.Mp + m0 + m4;
+        a_lds[j] = kk * LDA + m4;
+    }
+    const int a_step = BK * p.Mp;
     float4 areg[AV];
     float breg[EPT];
 
+    auto a_active = [&](int j) -> bool { return (A_VECS % 256 == 0 || j < AV - 1) ? true : (tid + j * 256 < A_VECS); };
     auto load_a = [&](int step) {
 #pragma unroll
-        for (int j = 0; j < AV; j++) {
-            const int f = tid + j * 256;
-            const int kk = f / (BM / 4), m4 = (f % (BM / 4)) * 4;
-            if (f < A_VECS) areg[j] = *reinterpret_cast<const float4 *>(p.Wp + (size_t)(step * BK + kk) * p.Mp + m0 + m4);
-        }
+        for (int j = 0; j < AV; j++)
+            if (a_active(j)) areg[j] = *reinterpret_cast<const float4 *>(a_ptr[j] + (size_t)step * a_step);
     };
     auto load_b = [&](int step) {
-        int i = step * BK + bg * EPT;
+        const int i = step * BK + bg * EPT;  // uniform
         int c = i / RS;
-        int rem = i - c * RS;
+        const int rem = i - c * RS;
         int ky = rem / S, kx = rem - ky * S;
 #pragma unroll
         for (int e = 0; e < EPT; e++) {
-            const int ih = ih0 + ky, iw = iw0 + kx;
-            const bool ok = pvalid && c < p.C && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
-            float v = 0.0f;
-            if (ok) v = in_img[((size_t)c * p.H + ih) * p.W + iw];
-            breg[e] = v;
+            const bool ok = pvalid && c < p.C && (unsigned)(ih0 + ky) < (unsigned)p.H && (unsigned)(iw0 + kx) < (unsigned)p.W;
+            const int vo = ok ? (pix + ky * p.W + kx) * 4 : OOB;
+            breg[e] = buf_load(rsrc_in, vo, (c < p.C ? c : 0) * HW4);
             if (++kx == S) {
                 kx = 0;
                 if (++ky == R) {
@@ -188,11 +423,8 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(const ConvParams p) {
     };
     auto store_ab = [&](int buf) {
 #pragma unroll
-        for (int j = 0; j < AV; j++) {
-            const int f = tid + j * 256;
-            const int kk = f / (BM / 4), m4 = (f % (BM / 4)) * 4;
-            if (f < A_VECS) *reinterpret_cast<float4 *>(&As[buf][kk * LDA + m4]) = areg[j];
-        }
+        for (int j = 0; j < AV; j++)
+            if (a_active(j)) *reinterpret_cast<float4 *>(&As[buf][a_lds[j]]) = areg[j];
 #pragma unroll
         for (int e = 0; e < EPT; e++) Bs[buf][(bg * EPT + e) * LDB + bn_l] = breg[e];
     };
@@ -220,44 +452,32 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(const ConvParams p) {
             load_a(step + 1);
             load_b(step + 1);
         }
+        // operands of tap pair ks+1 are read from LDS while the MFMAs of pair ks run
+        float a[2][TM], b[2][TN];
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++) a[0][tm] = As[buf][a_off + tm * 32];
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++) b[0][tn] = Bs[buf][b_off + tn * 32];
 #pragma unroll
         for (int ks = 0; ks < BK / 2; ks++) {
-            float a[TM], b[TN];
+            const int cur = ks & 1, nxt = cur ^ 1;
+            if (ks + 1 < BK / 2) {
 #pragma unroll
-            for (int tm = 0; tm < TM; tm++) a[tm] = As[buf][ks * 2 * LDA + a_off + tm * 32];
+                for (int tm = 0; tm < TM; tm++) a[nxt][tm] = As[buf][(ks + 1) * 2 * LDA + a_off + tm * 32];
 #pragma unroll
-            for (int tn = 0; tn < TN; tn++) b[tn] = Bs[buf][ks * 2 * LDB + b_off + tn * 32];
+                for (int tn = 0; tn < TN; tn++) b[nxt][tn] = Bs[buf][(ks + 1) * 2 * LDB + b_off + tn * 32];
+            }
 #pragma unroll
             for (int tm = 0; tm < TM; tm++)
 #pragma unroll
                 for (int tn = 0; tn < TN; tn++)
-                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tm], b[tn], acc[tm][tn], 0, 0, 0);
+                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
         }
         if (more) store_ab(buf ^ 1);
         __syncthreads();
     }
 
-    // ---- store: lane holds column (pixel) lane%32 and rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 block
-#pragma unroll
-    for (int tn = 0; tn < TN; tn++) {
-        const long long n = n0 + wn * TN * 32 + tn * 32 + (lane & 31);
-        if (n >= p.npix) continue;
-        const int img = (int)(n / p.PQ);
-        const int pq = (int)(n - (long long)img * p.PQ);
-        const size_t obase = (size_t)img * p.Kf * p.PQ + pq;
-#pragma unroll
-        for (int tm = 0; tm < TM; tm++) {
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int m = m0 + wm * TM * 32 + tm * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                if (m < p.Kf) {
-                    const ChannelEpilogue e = load_channel(p, m);
-                    const size_t oidx = obase + (size_t)m * p.PQ;
-                    p.O[oidx] = apply_epilogue(p, e, acc[tm][tn][v], oidx);
-                }
-            }
-        }
-    }
+    store_tile<TM, TN>(p, acc, m0 + wm * TM * 32, n0 + wn * TN * 32, lane);
 }
 
 // ---------------------------------------------------------------- scalar direct kernel
@@ -292,24 +512,46 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvParams p) {
     }
 }
 
+// ---------------------------------------------------------------- host side
 int g_algo = 0;
 hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;  // optional: bracket the main kernel of the next calls
+thread_local char g_last_kernel[96] = "";
 
-template <int WM, int WN, int TM, int TN>
-int launch_igemm(hipStream_t st, ConvParams &p) {
-    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    p.gm = (p.Kf + BM - 1) / BM;
-    long long gn = (p.npix + BN - 1) / BN;
-    EH_REQUIRE(gn * p.gm <= 0x7fffffffLL, "conv2d: too many tiles");
-    p.gn = (int)gn;
-    dim3 grid((unsigned)(gn * p.gm)), block(256);
-    if (g_prof_start) EH_TRY_HIP(hipEventRecord(g_prof_start, st));
-    if (p.R == 3 && p.S == 3) hipLaunchKernelGGL((conv_igemm_kernel<WM, WN, TM, TN, 3, 3>), grid, block, 0, st, p);
-    else if (p.R == 1 && p.S == 1) hipLaunchKernelGGL((conv_igemm_kernel<WM, WN, TM, TN, 1, 1>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((conv_igemm_kernel<WM, WN, TM, TN, 0, 0>), grid, block, 0, st, p);
-    EH_CHECK_LAUNCH();
-    if (g_prof_stop) EH_TRY_HIP(hipEventRecord(g_prof_stop, st));
-    return 0;
+struct Variant {
+    const char *name;
+    int bm, bn, cpb;  // cpb = channels per K-step (0: the 16-tap kernel for any filter shape)
+    void (*kernel)(const ConvParams);
+};
+
+#define TAP(WM, WN, TM, TN, R, S, CPB, D)                                                                                     \
+    {                                                                                                                         \
+        "conv_tap_kernel<" #WM "," #WN "," #TM "," #TN "," #R "," #S "," #CPB "," #D ">", WM *TM * 32, WN *TN * 32, CPB,       \
+            conv_tap_kernel<WM, WN, TM, TN, R, S, CPB, D>                                                                     \
+    }
+#define GEN(WM, WN, TM, TN) \
+    { "conv_gen_kernel<" #WM "," #WN "," #TM "," #TN ">", WM *TM * 32, WN *TN * 32, 0, conv_gen_kernel<WM, WN, TM, TN> }
+
+// Per filter shape: [gather kind: register-staged, LDS-direct][tile: 128x128, 64x128, 64x64, 32x128]
+const Variant k3x3[2][4] = {
+    {TAP(2, 2, 2, 2, 3, 3, 2, false), TAP(1, 4, 2, 1, 3, 3, 2, false), TAP(2, 2, 1, 1, 3, 3, 4, false), TAP(1, 4, 1, 1, 3, 3, 2, false)},
+    {TAP(2, 2, 2, 2, 3, 3, 2, true), TAP(1, 4, 2, 1, 3, 3, 2, true), TAP(2, 2, 1, 1, 3, 3, 4, true), TAP(1, 4, 1, 1, 3, 3, 2, true)}};
+const Variant k1x1[2][4] = {
+    {TAP(2, 2, 2, 2, 1, 1, 16, false), TAP(1, 4, 2, 1, 1, 1, 16, false), TAP(2, 2, 1, 1, 1, 1, 16, false), TAP(1, 4, 1, 1, 1, 1, 16, false)},
+    {TAP(2, 2, 2, 2, 1, 1, 16, true), TAP(1, 4, 2, 1, 1, 1, 16, true), TAP(2, 2, 1, 1, 1, 1, 16, true), TAP(1, 4, 1, 1, 1, 1, 16, true)}};
+const Variant k2x2[2][4] = {
+    {TAP(2, 2, 2, 2, 2, 2, 4, false), TAP(1, 4, 2, 1, 2, 2, 4, false), TAP(2, 2, 1, 1, 2, 2, 4, false), TAP(1, 4, 1, 1, 2, 2, 4, false)},
+    {TAP(2, 2, 2, 2, 2, 2, 4, true), TAP(1, 4, 2, 1, 2, 2, 4, true), TAP(2, 2, 1, 1, 2, 2, 4, true), TAP(1, 4, 1, 1, 2, 2, 4, true)}};
+const Variant kgen[4] = {GEN(2, 2, 2, 2), GEN(1, 4, 2, 1), GEN(2, 2, 1, 1), GEN(1, 4, 1, 1)};
+
+// The largest tile that still gives every CU about two workgroups; small channel counts take
+// the narrow tiles (index: 0 = 128x128, 1 = 64x128, 2 = 64x64, 3 = 32x128).
+int pick_tile(int Kf, long long npix, int num_cu) {
+    const long long want = 2LL * num_cu;
+    auto tiles = [&](int bm, int bn) { return (long long)((Kf + bm - 1) / bm) * ((npix + bn - 1) / bn); };
+    if (Kf > 64 && tiles(128, 128) >= want) return 0;
+    if (Kf > 32 && tiles(64, 128) >= want) return 1;
+    if (Kf > 32) return 2;
+    return 3;
 }
 
 }  // namespace
@@ -317,7 +559,7 @@ int launch_igemm(hipStream_t st, ConvParams &p) {
 extern "C" {
 
 int eddlhip_conv2d_set_algo(int algo) {
-    EH_REQUIRE(algo >= 0 && algo <= 2, "conv2d_set_algo: unknown algorithm %d", algo);
+    EH_REQUIRE(algo >= 0 && algo <= 4, "conv2d_set_algo: unknown algorithm %d", algo);
     g_algo = algo;
     return 0;
 }
@@ -328,6 +570,8 @@ int eddlhip_conv2d_set_profile_events(void *start, void *stop) {
     g_prof_stop = (hipEvent_t)stop;
     return 0;
 }
+
+const char *eddlhip_conv2d_last_kernel(void) { return g_last_kernel; }
 
 int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bias, float *O, int N, int C, int H, int W, int Kf,
                        int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b,
@@ -340,7 +584,9 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     EH_REQUIRE((bn_mean == nullptr) == (bn_var == nullptr), "conv2d: bn_mean and bn_var must come together");
     EH_REQUIRE((bn_g == nullptr) == (bn_b == nullptr), "conv2d: bn_g and bn_b must come together");
     EH_REQUIRE(bn_g == nullptr || bn_mean != nullptr, "conv2d: affine parameters without statistics");
-    EH_REQUIRE((long long)C * H * W <= 0x7fffffffLL && (long long)C * R * S <= 0x7fffff00LL, "conv2d: image or filter too large");
+    const long long img_elems = (long long)C * H * W;
+    EH_REQUIRE(img_elems <= (1LL << 28), "conv2d: one image of %lld elements exceeds the 1 GiB a buffer descriptor may cover", img_elems);
+    EH_REQUIRE((long long)C * R * S <= (1LL << 24), "conv2d: filter too large");
     EH_REQUIRE((long long)P * Q <= 0x7fffffffLL, "conv2d: output plane too large");
     if (N == 0) return 0;
     EH_REQUIRE(I && K && O, "conv2d: NULL tensor");
@@ -357,31 +603,64 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     p.PQ = P * Q;
     p.npix = (long long)N * P * Q;
     p.gm = p.gn = 0;
-    p.nsteps = (p.CRS + BK - 1) / BK;
+    p.nsteps = 0;
     p.Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
+    p.in_bytes = 0;
 
     if (g_algo == 2) {
         size_t total = (size_t)p.npix * Kf;
+        snprintf(g_last_kernel, sizeof(g_last_kernel), "conv_direct_kernel");
+        if (g_prof_start) EH_TRY_HIP(hipEventRecord(g_prof_start, st));
         hipLaunchKernelGGL(conv_direct_kernel, dim3(eh_blocks(total, 256, 1u << 20)), dim3(256), 0, st, p);
         EH_CHECK_LAUNCH();
+        if (g_prof_stop) EH_TRY_HIP(hipEventRecord(g_prof_stop, st));
         return 0;
     }
 
-    // repack the filters (tap-major, zero-padded) into the private workspace
-    const int CRSp = p.nsteps * BK;
+    // ---- kernel variant
+    const int direct = (g_algo == 4) ? 1 : 0;
+    const int tile = pick_tile(Kf, p.npix, state(dev).num_cu);
+    const Variant *v;
+    if (R == 3 && S == 3) v = &k3x3[direct][tile];
+    else if (R == 1 && S == 1) v = &k1x1[direct][tile];
+    else if (R == 2 && S == 2) v = &k2x2[direct][tile];
+    else v = &kgen[tile];
+    const int bk = v->cpb ? v->cpb * R * S : 16;
+    p.nsteps = v->cpb ? (C + v->cpb - 1) / v->cpb : (p.CRS + 15) / 16;
+    snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", v->name);
+
+    // ---- repack the filters (tap-major, zero-padded) into the private workspace
+    const int rows = p.nsteps * bk;
+    const size_t wp_bytes = (size_t)rows * p.Mp * sizeof(float);
+    EH_REQUIRE(wp_bytes <= 0x7fffffffu, "conv2d: packed filters exceed 2 GiB");
     void *ws = nullptr;
-    EH_TRY(get_workspace(dev, (size_t)CRSp * p.Mp * sizeof(float), &ws));
+    EH_TRY(get_workspace(dev, wp_bytes, &ws));
     p.Wp = (const float *)ws;
-    hipLaunchKernelGGL(pack_filters_kernel, dim3((CRSp + 31) / 32, p.Mp / 32), dim3(256), 0, st, K, (float *)ws, Kf, p.CRS, p.Mp, CRSp);
+    hipLaunchKernelGGL(pack_filters_kernel, dim3((rows + 31) / 32, p.Mp / 32), dim3(256), 0, st, K, (float *)ws, Kf, p.CRS, p.Mp, rows);
     EH_CHECK_LAUNCH();
 
-    // tile choice: the largest tile that still gives every CU about two workgroups
-    const long long want = 2LL * state(dev).num_cu;
-    auto tiles = [&](int bm, int bn) { return (long long)((Kf + bm - 1) / bm) * ((p.npix + bn - 1) / bn); };
-    if (Kf > 64 && tiles(128, 128) >= want) return launch_igemm<2, 2, 2, 2>(st, p);
-    if (Kf > 32 && tiles(64, 128) >= want) return launch_igemm<1, 4, 2, 1>(st, p);
-    if (Kf > 32) return launch_igemm<2, 2, 1, 1>(st, p);
-    return launch_igemm<1, 4, 1, 1>(st, p);
+    // ---- launch, in batch chunks whose input stays below the 2 GiB a buffer descriptor addresses
+    // with 32-bit offsets (one chunk for every shape of the CNN configurations)
+    const long long max_imgs = (1LL << 29) / img_elems;  // 2 GiB / 4 bytes
+    if (g_prof_start) EH_TRY_HIP(hipEventRecord(g_prof_start, st));
+    for (long long b0 = 0; b0 < N; b0 += max_imgs) {
+        const int nb = (int)((N - b0 < max_imgs) ? N - b0 : max_imgs);
+        ConvParams q = p;
+        q.N = nb;
+        q.I = I + (size_t)b0 * img_elems;
+        q.O = O + (size_t)b0 * Kf * p.PQ;
+        if (residual) q.residual = residual + (size_t)b0 * Kf * p.PQ;
+        q.npix = (long long)nb * p.PQ;
+        q.in_bytes = (unsigned)((size_t)nb * img_elems * sizeof(float));
+        q.gm = (Kf + v->bm - 1) / v->bm;
+        const long long gn = (q.npix + v->bn - 1) / v->bn;
+        EH_REQUIRE(gn * q.gm <= 0x7fffffffLL, "conv2d: too many tiles");
+        q.gn = (int)gn;
+        hipLaunchKernelGGL(v->kernel, dim3((unsigned)(gn * q.gm)), dim3(256), 0, st, q);
+        EH_CHECK_LAUNCH();
+    }
+    if (g_prof_stop) EH_TRY_HIP(hipEventRecord(g_prof_stop, st));
+    return 0;
 }
 
 }  // extern "C"

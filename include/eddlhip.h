@@ -90,10 +90,14 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
                        const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var,
                        float bn_eps, const float *residual, int relu);
 
-/* Selects the convolution kernel: 0 = automatic, 1 = force the general implicit-GEMM MFMA
- * kernel, 2 = force the scalar direct kernel (one thread per output; taps summed in the
- * reference's ky,kx,c order - used to cross-check the MFMA kernels on the device). */
+/* Selects the convolution kernel: 0 = automatic; 1 = matrix-core (MFMA) implicit GEMM;
+ * 2 = the scalar direct kernel (one thread per output; taps summed in the reference's ky,kx,c
+ * order with its rounding - used to cross-check the MFMA kernels on the device);
+ * 3 = MFMA with the input gather staged through registers; 4 = MFMA with the input gather
+ * written by the load unit straight into LDS.  eddlhip_conv2d_last_kernel() names the kernel
+ * the calling thread's last eddlhip_conv2d_fwd launched. */
 int eddlhip_conv2d_set_algo(int algo);
+const char *eddlhip_conv2d_last_kernel(void);
 
 /* Measurement hook (no counterpart in the reference): while two events are installed, every
  * eddlhip_conv2d_fwd records `start` on the device's stream immediately before its main

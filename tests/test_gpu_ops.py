@@ -57,7 +57,7 @@ def _conv_inputs(case):
     return x, w, (b if case["use_bias"] else None)
 
 
-@pytest.mark.parametrize("algo", ["mfma", "direct"])
+@pytest.mark.parametrize("algo", ["mfma_staged", "mfma_lds", "direct"])
 def test_conv2d_reference_vectors(hip, oracle, golden, algo):
     for case in golden["conv2d"]:
         x, w, b = _conv_inputs(case)
@@ -117,19 +117,26 @@ CONV_SHAPES = [
     (2, 6, 10, 12, 5, 3, 2, 1, 2, "same", None, True),         # rectangular filter, mixed strides
     (1, 300, 8, 8, 33, 3, 3, 1, 1, "same", None, False),       # many taps (C*R*S = 2700)
     (1, 1, 64, 64, 64, 3, 3, 1, 1, "same", None, True),        # single input channel (U-Net first layer)
+    (8, 32, 56, 56, 128, 3, 3, 1, 1, "same", None, True),      # enough tiles for the 128x128 kernel
+    (8, 31, 56, 56, 130, 3, 3, 1, 1, "same", None, False),     # 128x128 kernel, odd channels, ragged filters
+    (8, 24, 56, 56, 64, 3, 3, 1, 1, "same", None, True),       # 64x128 kernel
+    (8, 40, 56, 56, 256, 1, 1, 1, 1, "valid", None, True),     # 1x1 on the 128x128 kernel, channels not a multiple of 16
+    (8, 16, 57, 57, 128, 2, 2, 1, 1, "valid", None, True),     # 2x2 on the 128x128 kernel
+    (6, 10, 64, 64, 16, 3, 3, 2, 2, "custom", [1, 1, 1, 1], True),  # 32x128 kernel, stride 2
 ]
 
 
+@pytest.mark.parametrize("algo", ["mfma_staged", "mfma_lds"])
 @pytest.mark.parametrize("shape", CONV_SHAPES, ids=lambda s: "x".join(str(v) for v in s[:9]) + "-" + s[9])
-def test_conv2d_mfma_against_oracle(hip, oracle, shape):
+def test_conv2d_mfma_against_oracle(hip, oracle, shape, algo):
     N, C, H, W, Kf, R, S, sr, sc, padding, pads, use_bias = shape
     rng = np.random.default_rng(100 + C * 7 + Kf)
     x = rng.standard_normal((N, C, H, W), dtype=np.float32)
     w = (rng.standard_normal((Kf, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32)
     b = rng.standard_normal(Kf, dtype=np.float32) if use_bias else None
-    ref, out = run_conv(hip, oracle, x, w, b, (sr, sc), padding, pads, algo="mfma")
+    ref, out = run_conv(hip, oracle, x, w, b, (sr, sc), padding, pads, algo=algo)
     assert out.shape == ref.shape
-    assert_conv_close(ref, out, str(shape))
+    assert_conv_close(ref, out, str(shape) + " " + hip.last_conv_kernel())
 
 
 @pytest.mark.parametrize("shape", CONV_SHAPES[:6], ids=lambda s: "x".join(str(v) for v in s[:9]))
@@ -165,10 +172,11 @@ def test_conv2d_fused_epilogue(hip, oracle):
         b = kw.pop("b", None)
         ref, out = run_conv(hip, oracle, x, w, b, (1, 1), "same", algo="direct", **kw)
         assert np.array_equal(ref, out), kw.keys()
-    for kw in (dict(bn=bn, relu=True), dict(bn=bn, residual=res, relu=True)):
-        ref, out = run_conv(hip, oracle, x, w, None, (1, 1), "same", algo="mfma", **kw)
-        assert_conv_close(ref, out, "fused mfma")
-        assert np.all(out >= 0)
+    for algo in ("mfma_staged", "mfma_lds"):
+        for kw in (dict(bn=bn, relu=True), dict(bn=bn, residual=res, relu=True)):
+            ref, out = run_conv(hip, oracle, x, w, None, (1, 1), "same", algo=algo, **kw)
+            assert_conv_close(ref, out, "fused " + algo)
+            assert np.all(out >= 0)
 
 
 def test_conv2d_linearity_and_empty_batch(hip, oracle):
