@@ -44,6 +44,7 @@ using namespace eddlhip;
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lds_void;
 
 constexpr int M_ALIGN = 128;                  // packed filter rows are padded to this many channels
@@ -189,7 +190,8 @@ __global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
     constexpr int A_VECS = BK * BM / 4;          // float4 in one filter slice
     constexpr int AV = (A_VECS + 255) / 256;     // float4 filter loads per thread per step (last one partial)
 
-    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
+    // (+256 floats after each filter slice: where the lanes past the end of a partial last load round park their float4)
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA + 256];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -225,32 +227,31 @@ __global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
 
     // ---- filter slice: float4 f of the slice is row f / (BM/4), channels 4*(f % (BM/4))
     // (plain 16-byte loads: the packed matrix is padded to whole steps and whole tiles, so every address exists)
+    // Every thread loads in every round, without a condition: in a partial last round the lanes past
+    // the end of the slice re-read their first element and park it behind the slice in LDS.
     const float *a_ptr[AV];
     int a_lds[AV];
 #pragma unroll
     for (int j = 0; j < AV; j++) {
         const int f = tid + j * 256;
-        const int kk = f / (BM / 4), m4 = (f % (BM / 4)) * 4;
+        const bool in_slice = f < A_VECS;
+        const int fc = in_slice ? f : tid % A_VECS;
+        const int kk = fc / (BM / 4), m4 = (fc % (BM / 4)) * 4;
         a_ptr[j] = p.Wp + (size_t)kk * p.Mp + m0 + m4;
-        a_lds[j] = kk * LDA + m4;
+        a_lds[j] = in_slice ? kk * LDA + m4 : BK * LDA + lane * 4;
     }
     const int a_step = BK * p.Mp;
 
-    float4 areg[AV];
+    floatx4 areg[AV];
     float breg[DIRECT ? 1 : CPW * RS];
 
-    auto a_active = [&](int j) -> bool {  // only the last, partial round of a slice tests anything
-        return (A_VECS % 256 == 0 || j < AV - 1) ? true : (tid + j * 256 < A_VECS);
-    };
     auto load_a = [&](int step) {
 #pragma unroll
-        for (int j = 0; j < AV; j++)
-            if (a_active(j)) areg[j] = *reinterpret_cast<const float4 *>(a_ptr[j] + (size_t)step * a_step);
+        for (int j = 0; j < AV; j++) areg[j] = *reinterpret_cast<const floatx4 *>(a_ptr[j] + (size_t)step * a_step);
     };
     auto store_a = [&](int buf) {
 #pragma unroll
-        for (int j = 0; j < AV; j++)
-            if (a_active(j)) *reinterpret_cast<float4 *>(&As[buf][a_lds[j]]) = areg[j];
+        for (int j = 0; j < AV; j++) *reinterpret_cast<floatx4 *>(&As[buf][a_lds[j]]) = areg[j];
     };
     // gather of one step; `checked` adds the test for channels past C (last step of an odd channel count)
     auto load_b = [&](int step, int buf, bool checked) {
@@ -301,11 +302,35 @@ __global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
     for (int step = 0; step < p.nsteps; step++) {
         const int buf = step & 1;
         const bool more = step + 1 < p.nsteps;
-        if (more) {
+#ifndef LAB_MODE
+#define LAB_MODE 0
+#endif
+        if (more && !(LAB_MODE & 1)) {
             load_a(step + 1);
             if (step + 1 < full_steps) load_b(step + 1, buf ^ 1, false);
             else load_b(step + 1, buf ^ 1, true);
         }
+#if LAB_MODE & 4
+        {
+            float a[BK / 2][TM], b[BK / 2][TN];
+#pragma unroll
+            for (int ks = 0; ks < BK / 2; ks++) {
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++) a[ks][tm] = As[buf][ks * 2 * LDA + a_off + tm * 32];
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) b[ks][tn] = Bs[buf][ks * 2 * LDB + b_off + tn * 32];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < BK / 2; ks++)
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++)
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ks][tm], b[ks][tn], acc[tm][tn], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#else
         // operands of tap pair ks+1 are read from LDS while the MFMAs of pair ks run
         float a[2][TM], b[2][TN];
 #pragma unroll
@@ -327,11 +352,14 @@ __global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
                 for (int tn = 0; tn < TN; tn++)
                     acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
         }
-        if (more) {
+#endif
+        if (more && !(LAB_MODE & 1)) {
             store_a(buf ^ 1);
             store_b(buf ^ 1);
         }
+#if !(LAB_MODE & 2)
         __syncthreads();
+#endif
     }
 
     store_tile<TM, TN>(p, acc, m0 + wm * TM * 32, n0 + wn * TN * 32, lane);
@@ -351,7 +379,8 @@ __global__ __launch_bounds__(256) void conv_gen_kernel(const ConvParams p) {
     constexpr int EPT = BN / 16;  // gathered elements per thread per step
     static_assert(BN >= 64 && BN <= 256, "a wavefront gathers whole tap rows");
 
-    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
+    // (+256 floats after each filter slice: where the lanes past the end of a partial last load round park their float4)
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA + 256];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -383,24 +412,27 @@ __global__ __launch_bounds__(256) void conv_gen_kernel(const ConvParams p) {
     const int HW4 = p.H * p.W * 4;
 
     // (plain 16-byte loads: the packed matrix is padded to whole steps and whole tiles, so every address exists)
+    // Every thread loads in every round, without a condition: in a partial last round the lanes past
+    // the end of the slice re-read their first element and park it behind the slice in LDS.
     const float *a_ptr[AV];
     int a_lds[AV];
 #pragma unroll
     for (int j = 0; j < AV; j++) {
         const int f = tid + j * 256;
-        const int kk = f / (BM / 4), m4 = (f % (BM / 4)) * 4;
+        const bool in_slice = f < A_VECS;
+        const int fc = in_slice ? f : tid % A_VECS;
+        const int kk = fc / (BM / 4), m4 = (fc % (BM / 4)) * 4;
         a_ptr[j] = p.Wp + (size_t)kk * p.Mp + m0 + m4;
-        a_lds[j] = kk * LDA + m4;
+        a_lds[j] = in_slice ? kk * LDA + m4 : BK * LDA + lane * 4;
     }
     const int a_step = BK * p.Mp;
-    float4 areg[AV];
+    floatx4 areg[AV];
     float breg[EPT];
 
-    auto a_active = [&](int j) -> bool { return (A_VECS % 256 == 0 || j < AV - 1) ? true : (tid + j * 256 < A_VECS); };
     auto load_a = [&](int step) {
 #pragma unroll
         for (int j = 0; j < AV; j++)
-            if (a_active(j)) areg[j] = *reinterpret_cast<const float4 *>(a_ptr[j] + (size_t)step * a_step);
+            areg[j] = *reinterpret_cast<const floatx4 *>(a_ptr[j] + (size_t)step * a_step);
     };
     auto load_b = [&](int step) {
         const int i = step * BK + bg * EPT;  // uniform
@@ -424,7 +456,7 @@ __global__ __launch_bounds__(256) void conv_gen_kernel(const ConvParams p) {
     auto store_ab = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < AV; j++)
-            if (a_active(j)) *reinterpret_cast<float4 *>(&As[buf][a_lds[j]]) = areg[j];
+            *reinterpret_cast<floatx4 *>(&As[buf][a_lds[j]]) = areg[j];
 #pragma unroll
         for (int e = 0; e < EPT; e++) Bs[buf][(bg * EPT + e) * LDB + bn_l] = breg[e];
     };
