@@ -57,7 +57,7 @@ def time_ops(hip, model, reps):
                 hip.set_conv_profile_events(s, e)
                 op.run()
                 hip.set_conv_profile_events(None, None)
-                kernels[i] = hip.last_conv_kernel()
+                kernels[i] = hip.last_conv_kernel().split(" +ksplit")[0]
             else:
                 s.record()
                 op.run()

@@ -135,7 +135,7 @@ class Backend:
         return t
 
     def set_conv_algo(self, algo):
-        self._check(self.lib.eddlhip_conv2d_set_algo({"auto": 0, "mfma": 1, "direct": 2, "mfma_staged": 3, "mfma_lds": 4}.get(algo, algo)))
+        self._check(self.lib.eddlhip_conv2d_set_algo({"auto": 0, "mfma": 1, "direct": 2, "mfma_staged": 3, "mfma_lds": 4, "ksplit_off": 5, "ksplit_on": 6}.get(algo, algo)))
 
     def last_conv_kernel(self):
         return self.lib.eddlhip_conv2d_last_kernel().decode()

@@ -64,6 +64,11 @@ struct ConvParams {
     long long npix;
     int gm, gn;
     unsigned in_bytes;  // size the input's buffer descriptor covers
+    // Tiles [tile0, tile0 + gridDim.x / nslices) are computed by this launch.  With nslices > 1 a
+    // tile's K-steps are divided over nslices workgroups of slice_steps steps each, which write
+    // their raw accumulators to `partial`; conv_reduce_kernel adds the slices and finishes the tile.
+    int tile0, nslices, slice_steps;
+    float *partial;
 };
 
 // The fused tail of a Conv -> BatchNorm(inference) -> Add -> ReLU chain; every step rounded
@@ -105,14 +110,32 @@ __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, int voffset,
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voffset, soffset, 0));
 }
 
-// workgroup id -> (channel tile, pixel tile); ids that share an XCD get consecutive tiles
-__device__ __forceinline__ void tile_of_block(const ConvParams &p, int &m_tile, int &n_tile) {
+// workgroup id -> (channel tile, pixel tile, K slice); ids that share an XCD get consecutive tiles
+__device__ __forceinline__ void tile_of_block(const ConvParams &p, int &m_tile, int &n_tile, int &local_tile, int &slice) {
     const unsigned total = gridDim.x, bid = blockIdx.x;
     const unsigned q = total / EDDLHIP_NUM_XCD, r = total % EDDLHIP_NUM_XCD;
     const unsigned xcd = bid % EDDLHIP_NUM_XCD, slot = bid / EDDLHIP_NUM_XCD;
     const int vid = (int)((xcd < r ? xcd * (q + 1) : r * (q + 1) + (xcd - r) * q) + slot);
-    m_tile = vid % p.gm;
-    n_tile = vid / p.gm;
+    slice = vid % p.nslices;
+    local_tile = vid / p.nslices;
+    const int tile = p.tile0 + local_tile;
+    m_tile = tile % p.gm;
+    n_tile = tile / p.gm;
+}
+
+// Raw accumulators of one K slice of one tile, laid out [slice][tile][wave][block][v][lane] so
+// that every store instruction of a wavefront writes 256 contiguous bytes.
+template <int TM, int TN>
+__device__ __forceinline__ void store_partial(const ConvParams &p, floatx16 (&acc)[TM][TN], int local_tile, int slice, int wave,
+                                              int lane) {
+    const size_t tiles = gridDim.x / p.nslices;
+    float *dst = p.partial + (((size_t)slice * tiles + local_tile) * 4 + wave) * (TM * TN * 16 * 64) + lane;
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) dst[((tm * TN + tn) * 16 + v) * 64] = acc[tm][tn][v];
 }
 
 // Writes a wavefront's TM x TN blocks.  A lane holds column (pixel) lane%32 and rows
@@ -197,8 +220,10 @@ __global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
-    int m_tile, n_tile;
-    tile_of_block(p, m_tile, n_tile);
+    int m_tile, n_tile, local_tile, slice;
+    tile_of_block(p, m_tile, n_tile, local_tile, slice);
+    const int step_lo = slice * p.slice_steps;
+    const int step_hi = min(step_lo + p.slice_steps, p.nsteps);
     const int m0 = m_tile * BM;
     const long long n0 = (long long)n_tile * BN;
 
@@ -290,8 +315,8 @@ __global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
             for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.0f;
 
     const int full_steps = p.C / CPB;  // steps whose channels all exist
-    load_a(0);
-    load_b(0, 0, full_steps == 0);
+    load_a(step_lo);
+    load_b(step_lo, 0, step_lo >= full_steps);
     store_a(0);
     store_b(0);
     __syncthreads();
@@ -299,38 +324,14 @@ __global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
     const int a_off = (lane >> 5) * LDA + wm * TM * 32 + (lane & 31);
     const int b_off = (lane >> 5) * LDB + wn * TN * 32 + (lane & 31);
 
-    for (int step = 0; step < p.nsteps; step++) {
-        const int buf = step & 1;
-        const bool more = step + 1 < p.nsteps;
-#ifndef LAB_MODE
-#define LAB_MODE 0
-#endif
-        if (more && !(LAB_MODE & 1)) {
+    for (int step = step_lo; step < step_hi; step++) {
+        const int buf = (step - step_lo) & 1;
+        const bool more = step + 1 < step_hi;
+        if (more) {
             load_a(step + 1);
             if (step + 1 < full_steps) load_b(step + 1, buf ^ 1, false);
             else load_b(step + 1, buf ^ 1, true);
         }
-#if LAB_MODE & 4
-        {
-            float a[BK / 2][TM], b[BK / 2][TN];
-#pragma unroll
-            for (int ks = 0; ks < BK / 2; ks++) {
-#pragma unroll
-                for (int tm = 0; tm < TM; tm++) a[ks][tm] = As[buf][ks * 2 * LDA + a_off + tm * 32];
-#pragma unroll
-                for (int tn = 0; tn < TN; tn++) b[ks][tn] = Bs[buf][ks * 2 * LDB + b_off + tn * 32];
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int ks = 0; ks < BK / 2; ks++)
-#pragma unroll
-                for (int tm = 0; tm < TM; tm++)
-#pragma unroll
-                    for (int tn = 0; tn < TN; tn++)
-                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ks][tm], b[ks][tn], acc[tm][tn], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-#else
         // operands of tap pair ks+1 are read from LDS while the MFMAs of pair ks run
         float a[2][TM], b[2][TN];
 #pragma unroll
@@ -352,17 +353,15 @@ __global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
                 for (int tn = 0; tn < TN; tn++)
                     acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
         }
-#endif
-        if (more && !(LAB_MODE & 1)) {
+        if (more) {
             store_a(buf ^ 1);
             store_b(buf ^ 1);
         }
-#if !(LAB_MODE & 2)
         __syncthreads();
-#endif
     }
 
-    store_tile<TM, TN>(p, acc, m0 + wm * TM * 32, n0 + wn * TN * 32, lane);
+    if (p.nslices > 1) store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
+    else store_tile<TM, TN>(p, acc, m0 + wm * TM * 32, n0 + wn * TN * 32, lane);
 }
 
 // ---------------------------------------------------------------- MFMA kernel, any filter shape
@@ -387,8 +386,10 @@ __global__ __launch_bounds__(256) void conv_gen_kernel(const ConvParams p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int R = p.R, S = p.S, RS = R * S;
-    int m_tile, n_tile;
-    tile_of_block(p, m_tile, n_tile);
+    int m_tile, n_tile, local_tile, slice;
+    tile_of_block(p, m_tile, n_tile, local_tile, slice);
+    const int step_lo = slice * p.slice_steps;
+    const int step_hi = min(step_lo + p.slice_steps, p.nsteps);
     const int m0 = m_tile * BM;
     const long long n0 = (long long)n_tile * BN;
 
@@ -469,17 +470,17 @@ __global__ __launch_bounds__(256) void conv_gen_kernel(const ConvParams p) {
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.0f;
 
-    load_a(0);
-    load_b(0);
+    load_a(step_lo);
+    load_b(step_lo);
     store_ab(0);
     __syncthreads();
 
     const int a_off = (lane >> 5) * LDA + wm * TM * 32 + (lane & 31);
     const int b_off = (lane >> 5) * LDB + wn * TN * 32 + (lane & 31);
 
-    for (int step = 0; step < p.nsteps; step++) {
-        const int buf = step & 1;
-        const bool more = step + 1 < p.nsteps;
+    for (int step = step_lo; step < step_hi; step++) {
+        const int buf = (step - step_lo) & 1;
+        const bool more = step + 1 < step_hi;
         if (more) {
             load_a(step + 1);
             load_b(step + 1);
@@ -509,6 +510,43 @@ __global__ __launch_bounds__(256) void conv_gen_kernel(const ConvParams p) {
         __syncthreads();
     }
 
+    if (p.nslices > 1) store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
+    else store_tile<TM, TN>(p, acc, m0 + wm * TM * 32, n0 + wn * TN * 32, lane);
+}
+
+// ---------------------------------------------------------------- finishing kernel of K-split tiles
+// One workgroup per tile, same thread -> output mapping as the MFMA kernels: adds the slices
+// in increasing K order (a fixed order: results do not depend on scheduling), then applies the
+// fused tail and stores.
+template <int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(256) void conv_reduce_kernel(const ConvParams p) {
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int local_tile = blockIdx.x;
+    const int tile = p.tile0 + local_tile;
+    const int m0 = (tile % p.gm) * BM;
+    const long long n0 = (long long)(tile / p.gm) * BN;
+    const size_t tiles = gridDim.x;
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.0f;
+    for (int sl = 0; sl < p.nslices; sl++) {
+        const float *src = p.partial + (((size_t)sl * tiles + local_tile) * 4 + wave) * (TM * TN * 16 * 64) + lane;
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const float x = src[((tm * TN + tn) * 16 + v) * 64];
+                    acc[tm][tn][v] = sl == 0 ? x : __fadd_rn(acc[tm][tn][v], x);
+                }
+    }
     store_tile<TM, TN>(p, acc, m0 + wm * TM * 32, n0 + wn * TN * 32, lane);
 }
 
@@ -547,21 +585,25 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvParams p) {
 // ---------------------------------------------------------------- host side
 int g_algo = 0;
 hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;  // optional: bracket the main kernel of the next calls
-thread_local char g_last_kernel[96] = "";
+thread_local char g_last_kernel[128] = "";
+int g_split = 1;  // divide the tiles of a mostly idle last round along K (set_algo 5 turns it off)
 
 struct Variant {
     const char *name;
     int bm, bn, cpb;  // cpb = channels per K-step (0: the 16-tap kernel for any filter shape)
     void (*kernel)(const ConvParams);
+    void (*reduce)(const ConvParams);
+    mutable int occupancy;  // resident workgroups per CU, asked of the runtime on first use
 };
 
 #define TAP(WM, WN, TM, TN, R, S, CPB, D)                                                                                     \
     {                                                                                                                         \
         "conv_tap_kernel<" #WM "," #WN "," #TM "," #TN "," #R "," #S "," #CPB "," #D ">", WM *TM * 32, WN *TN * 32, CPB,       \
-            conv_tap_kernel<WM, WN, TM, TN, R, S, CPB, D>                                                                     \
+            conv_tap_kernel<WM, WN, TM, TN, R, S, CPB, D>, conv_reduce_kernel<WM, WN, TM, TN>, 0                              \
     }
 #define GEN(WM, WN, TM, TN) \
-    { "conv_gen_kernel<" #WM "," #WN "," #TM "," #TN ">", WM *TM * 32, WN *TN * 32, 0, conv_gen_kernel<WM, WN, TM, TN> }
+    { "conv_gen_kernel<" #WM "," #WN "," #TM "," #TN ">", WM *TM * 32, WN *TN * 32, 0, conv_gen_kernel<WM, WN, TM, TN>, \
+      conv_reduce_kernel<WM, WN, TM, TN>, 0 }
 
 // Per filter shape: [gather kind: register-staged, LDS-direct][tile: 128x128, 64x128, 64x64, 32x128]
 const Variant k3x3[2][4] = {
@@ -575,15 +617,67 @@ const Variant k2x2[2][4] = {
     {TAP(2, 2, 2, 2, 2, 2, 4, true), TAP(1, 4, 2, 1, 2, 2, 4, true), TAP(2, 2, 1, 1, 2, 2, 4, true), TAP(1, 4, 1, 1, 2, 2, 4, true)}};
 const Variant kgen[4] = {GEN(2, 2, 2, 2), GEN(1, 4, 2, 1), GEN(2, 2, 1, 1), GEN(1, 4, 1, 1)};
 
-// The largest tile that still gives every CU about two workgroups; small channel counts take
-// the narrow tiles (index: 0 = 128x128, 1 = 64x128, 2 = 64x64, 3 = 32x128).
-int pick_tile(int Kf, long long npix, int num_cu) {
-    const long long want = 2LL * num_cu;
-    auto tiles = [&](int bm, int bn) { return (long long)((Kf + bm - 1) / bm) * ((npix + bn - 1) / bn); };
-    if (Kf > 64 && tiles(128, 128) >= want) return 0;
-    if (Kf > 32 && tiles(64, 128) >= want) return 1;
-    if (Kf > 32) return 2;
-    return 3;
+// Launch plan: tile shape and, for the tiles of the last (partial) round of workgroups, the
+// number of K slices.  A grid that is not a whole number of device-filling rounds leaves its
+// last round mostly idle (28x28x512 at batch 32: 784 tiles of 128x128 for 768 resident
+// workgroups).  Those "leftover" tiles can be divided along K over several workgroups each so
+// that they, too, occupy the whole device; conv_reduce_kernel then adds the slices in a fixed
+// order.  The plan minimises a simple time estimate over the four tile shapes and 1..16 slices:
+//   a K-step of a tile costs its flops over (CU peak x tile efficiency); a workgroup costs its
+//   K-steps plus a fixed prologue/epilogue; a full round keeps `occupancy` workgroups on every
+//   CU; the last round costs ceil(workgroups / CUs) workgroup times; divided tiles add the
+//   traffic of their partial sums and two more launches.
+struct Plan {
+    int tile, nsteps, nslices, slice_steps;
+    long long tiles, leftover;
+    double cost_us;
+};
+
+Plan plan_conv(const Variant *family, int Kf, int C, int RS, long long npix, int num_cu, bool allow_split) {
+    static const double kEff[4] = {0.80, 0.66, 0.52, 0.40};      // fraction of the MFMA peak a long K loop sustains, per tile shape
+    static const double kOverheadUs[4] = {5.0, 3.5, 2.5, 2.5};   // prologue + epilogue of one workgroup (CU time)
+    const double cu_flops_per_us = 157.3e6 / 256.0;
+    const double bytes_per_us = 3.0e6;  // partial-sum traffic
+    // a CU with fewer resident workgroups than it can hold hides less latency
+    auto crowd = [](long long resident) { return resident >= 3 ? 1.0 : (resident == 2 ? 0.9 : 0.73); };
+    Plan best;
+    best.cost_us = -1.0;
+    for (int t = 0; t < 4; t++) {
+        const Variant &v = family[t];
+        // wide tiles only pay off when the filters fill them
+        if ((v.bm == 128 && Kf <= 64) || (v.bm == 64 && Kf <= 32)) continue;
+        const int bk = v.cpb ? v.cpb * RS : 16;
+        const int nsteps = v.cpb ? (C + v.cpb - 1) / v.cpb : (C * RS + 15) / 16;
+        const long long tiles = (long long)((Kf + v.bm - 1) / v.bm) * ((npix + v.bn - 1) / v.bn);
+        const long long slots = (long long)num_cu * v.occupancy;
+        const long long full = tiles / slots, left = tiles % slots;
+        const double step_us = 2.0 * v.bm * v.bn * bk / (cu_flops_per_us * kEff[t]);
+        const double base = (double)full * v.occupancy * (nsteps * step_us + kOverheadUs[t]) / crowd(v.occupancy);
+        const int smax = allow_split ? (nsteps / 4 < 16 ? nsteps / 4 : 16) : 1;
+        for (int want = 1; want <= (smax < 1 ? 1 : smax); want++) {
+            const int ss = (nsteps + want - 1) / want;
+            const int sl = (nsteps + ss - 1) / ss;
+            if (sl != want && want != 1) continue;  // same plan as a smaller `want`
+            double last = 0.0;
+            if (left > 0) {
+                const long long wgs = left * sl;
+                const long long per_cu = (wgs + num_cu - 1) / num_cu;
+                last = (double)per_cu * (ss * step_us + kOverheadUs[t]) / crowd(per_cu < v.occupancy ? per_cu : v.occupancy);
+                if (sl > 1) last += (double)wgs * v.bm * v.bn * 8.0 / bytes_per_us + 6.0;
+            }
+            const double cost = base + last;
+            if (best.cost_us < 0 || cost < best.cost_us) {
+                best.tile = t;
+                best.nsteps = nsteps;
+                best.nslices = sl;
+                best.slice_steps = ss;
+                best.tiles = tiles;
+                best.leftover = left;
+                best.cost_us = cost;
+            }
+        }
+    }
+    return best;
 }
 
 }  // namespace
@@ -591,7 +685,11 @@ int pick_tile(int Kf, long long npix, int num_cu) {
 extern "C" {
 
 int eddlhip_conv2d_set_algo(int algo) {
-    EH_REQUIRE(algo >= 0 && algo <= 4, "conv2d_set_algo: unknown algorithm %d", algo);
+    EH_REQUIRE(algo >= 0 && algo <= 6, "conv2d_set_algo: unknown algorithm %d", algo);
+    if (algo == 5 || algo == 6) {
+        g_split = (algo == 6);
+        return 0;
+    }
     g_algo = algo;
     return 0;
 }
@@ -638,6 +736,7 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     p.nsteps = 0;
     p.Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
     p.in_bytes = 0;
+    p.tile0 = 0; p.nslices = 1; p.slice_steps = 0; p.partial = nullptr;
 
     if (g_algo == 2) {
         size_t total = (size_t)p.npix * Kf;
@@ -649,34 +748,46 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
         return 0;
     }
 
-    // ---- kernel variant
+    // ---- kernel variant and launch plan
     const int direct = (g_algo == 4) ? 1 : 0;
-    const int tile = pick_tile(Kf, p.npix, state(dev).num_cu);
-    const Variant *v;
-    if (R == 3 && S == 3) v = &k3x3[direct][tile];
-    else if (R == 1 && S == 1) v = &k1x1[direct][tile];
-    else if (R == 2 && S == 2) v = &k2x2[direct][tile];
-    else v = &kgen[tile];
+    const Variant *family;
+    if (R == 3 && S == 3) family = k3x3[direct];
+    else if (R == 1 && S == 1) family = k1x1[direct];
+    else if (R == 2 && S == 2) family = k2x2[direct];
+    else family = kgen;
+    for (int t = 0; t < 4; t++) {
+        if (family[t].occupancy == 0) {
+            int occ = 0;
+            EH_TRY_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, family[t].kernel, 256, 0));
+            family[t].occupancy = occ > 0 ? occ : 1;
+        }
+    }
+    const long long max_imgs = (1LL << 29) / img_elems;  // a buffer descriptor addresses 2 GiB with 32-bit offsets
+    const int chunk_imgs = (int)((N < max_imgs) ? N : max_imgs);
+    const Plan plan = plan_conv(family, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu, g_split != 0);
+    const Variant *v = &family[plan.tile];
     const int bk = v->cpb ? v->cpb * R * S : 16;
-    p.nsteps = v->cpb ? (C + v->cpb - 1) / v->cpb : (p.CRS + 15) / 16;
-    snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", v->name);
+    p.nsteps = plan.nsteps;
+    const int gm = (Kf + v->bm - 1) / v->bm;
+    EH_REQUIRE(plan.tiles <= 0x3fffffffLL, "conv2d: too many tiles");
+    const long long leftover = plan.nslices > 1 ? plan.leftover : 0;
+    const int nslices = plan.nslices, slice_steps = plan.slice_steps;
+    const size_t tile_floats = (size_t)v->bm * v->bn;
 
-    // ---- repack the filters (tap-major, zero-padded) into the private workspace
+    // ---- workspace: packed filters, then the partial tiles of the K-split launch
     const int rows = p.nsteps * bk;
-    const size_t wp_bytes = (size_t)rows * p.Mp * sizeof(float);
-    EH_REQUIRE(wp_bytes <= 0x7fffffffu, "conv2d: packed filters exceed 2 GiB");
+    const size_t wp_bytes = ((size_t)rows * p.Mp * sizeof(float) + 255) & ~(size_t)255;
+    const size_t partial_bytes = (size_t)nslices * leftover * tile_floats * sizeof(float);
     void *ws = nullptr;
-    EH_TRY(get_workspace(dev, wp_bytes, &ws));
+    EH_TRY(get_workspace(dev, wp_bytes + partial_bytes, &ws));
     p.Wp = (const float *)ws;
+    p.partial = (float *)((char *)ws + wp_bytes);
     hipLaunchKernelGGL(pack_filters_kernel, dim3((rows + 31) / 32, p.Mp / 32), dim3(256), 0, st, K, (float *)ws, Kf, p.CRS, p.Mp, rows);
     EH_CHECK_LAUNCH();
 
-    // ---- launch, in batch chunks whose input stays below the 2 GiB a buffer descriptor addresses
-    // with 32-bit offsets (one chunk for every shape of the CNN configurations)
-    const long long max_imgs = (1LL << 29) / img_elems;  // 2 GiB / 4 bytes
     if (g_prof_start) EH_TRY_HIP(hipEventRecord(g_prof_start, st));
-    for (long long b0 = 0; b0 < N; b0 += max_imgs) {
-        const int nb = (int)((N - b0 < max_imgs) ? N - b0 : max_imgs);
+    for (long long b0 = 0; b0 < N; b0 += chunk_imgs) {
+        const int nb = (int)((N - b0 < chunk_imgs) ? N - b0 : chunk_imgs);
         ConvParams q = p;
         q.N = nb;
         q.I = I + (size_t)b0 * img_elems;
@@ -684,14 +795,32 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
         if (residual) q.residual = residual + (size_t)b0 * Kf * p.PQ;
         q.npix = (long long)nb * p.PQ;
         q.in_bytes = (unsigned)((size_t)nb * img_elems * sizeof(float));
-        q.gm = (Kf + v->bm - 1) / v->bm;
+        q.gm = gm;
         const long long gn = (q.npix + v->bn - 1) / v->bn;
-        EH_REQUIRE(gn * q.gm <= 0x7fffffffLL, "conv2d: too many tiles");
         q.gn = (int)gn;
-        hipLaunchKernelGGL(v->kernel, dim3((unsigned)(gn * q.gm)), dim3(256), 0, st, q);
-        EH_CHECK_LAUNCH();
+        const long long tiles = gn * gm;
+        const long long split_tiles = (nb == chunk_imgs) ? leftover : 0;  // a short last chunk runs unsplit
+        const long long main_tiles = tiles - split_tiles;
+        if (main_tiles > 0) {
+            q.tile0 = 0;
+            q.nslices = 1;
+            q.slice_steps = p.nsteps;
+            hipLaunchKernelGGL(v->kernel, dim3((unsigned)main_tiles), dim3(256), 0, st, q);
+            EH_CHECK_LAUNCH();
+        }
+        if (split_tiles > 0) {
+            q.tile0 = (int)main_tiles;
+            q.nslices = nslices;
+            q.slice_steps = slice_steps;
+            hipLaunchKernelGGL(v->kernel, dim3((unsigned)(split_tiles * nslices)), dim3(256), 0, st, q);
+            EH_CHECK_LAUNCH();
+            hipLaunchKernelGGL(v->reduce, dim3((unsigned)split_tiles), dim3(256), 0, st, q);
+            EH_CHECK_LAUNCH();
+        }
     }
     if (g_prof_stop) EH_TRY_HIP(hipEventRecord(g_prof_stop, st));
+    if (leftover > 0) snprintf(g_last_kernel, sizeof(g_last_kernel), "%s +ksplit(%lld tiles x %d)", v->name, leftover, nslices);
+    else snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", v->name);
     return 0;
 }
 

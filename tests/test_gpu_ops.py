@@ -179,6 +179,33 @@ def test_conv2d_fused_epilogue(hip, oracle):
             assert np.all(out >= 0)
 
 
+def test_conv2d_ksplit_of_the_last_round(hip, oracle):
+    """Tiles of a mostly idle last round are divided along K and added in slice order: same
+    tolerance, reproducible bit for bit from run to run, and the undivided plan is still there."""
+    rng = np.random.default_rng(302)
+    split_seen = 0
+    for (N, C, H, W, Kf, R) in [(8, 64, 28, 28, 128, 3), (4, 256, 14, 14, 256, 1), (3, 96, 20, 20, 200, 3), (32, 512, 14, 14, 512, 3)]:
+        x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+        w = (rng.standard_normal((Kf, C, R, R)) * np.sqrt(2.0 / (C * R * R))).astype(np.float32)
+        b = rng.standard_normal(Kf, dtype=np.float32)
+        outs = {}
+        for mode in ("ksplit_on", "ksplit_off"):
+            hip.set_conv_algo(mode)
+            try:
+                ref, out = run_conv(hip, oracle, x, w, b, (1, 1), "same", algo="mfma", relu=True)
+                name = hip.last_conv_kernel()
+                _, again = run_conv(hip, oracle, x, w, b, (1, 1), "same", algo="mfma", relu=True)
+            finally:
+                hip.set_conv_algo("ksplit_on")
+            assert mode == "ksplit_on" or "+ksplit" not in name, name
+            split_seen += "+ksplit" in name
+            assert_conv_close(ref, out, name)
+            assert np.array_equal(out, again), "not reproducible: " + name
+            outs[mode] = out
+        np.testing.assert_allclose(outs["ksplit_on"], outs["ksplit_off"], rtol=1e-4, atol=1e-4)
+    assert split_seen >= 1, "the planner never divided a last round along K"
+
+
 def test_conv2d_linearity_and_empty_batch(hip, oracle):
     from eddl_amd.descriptors import ConvolDescriptor
     rng = np.random.default_rng(301)
