@@ -88,3 +88,16 @@ def test_descriptor_errors_follow_the_reference():
         ConvolDescriptor(4, [5, 5], [1, 1], "valid").build([1, 3, 4, 4])
     with pytest.raises(RuntimeError, match="PoolDescriptor::PoolDescriptor"):
         PoolDescriptor([2, 2], [2, 2], "bogus")
+
+
+def test_host_layer_links_against_the_c_abi():
+    """The C++ host layer builds with g++ alone and resolves every symbol against libeddlhip.so."""
+    import subprocess
+    host = os.path.join(ROOT, "eddl_amd", "host")
+    lib = os.path.join(host, "libeddlhip_host.so")
+    if not os.path.exists(lib):
+        subprocess.run(["make", "-C", host, "all"], check=True, stdout=subprocess.DEVNULL)
+    h = ctypes.CDLL(lib)
+    for sym in ("_ZN8eddl_hip10gpu_conv2DEPNS_16ConvolDescriptorE", "_ZN8eddl_hip8tensorNN6Conv2DEPNS_16ConvolDescriptorE",
+                "_ZN8eddl_hip11gpu_mpool2DEPNS_14PoolDescriptorE", "_ZN8eddl_hip8gpu_reluEPNS_6TensorES1_"):
+        assert hasattr(h, sym), sym

@@ -1,0 +1,111 @@
+"""The C++ host layer (eddl_amd/host: Tensor, ConvolDescriptor, PoolDescriptor, gpu_*, tensorNN::*)
+driven at descriptor level the way the reference's unit tests drive its seam, through a small
+C++ program (tests/host/host_driver.cpp); results are compared with the CPU oracle."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import ROOT, tensor_of
+
+pytestmark = pytest.mark.gpu
+
+DRIVER = os.path.join(ROOT, "eddl_amd", "host", "host_driver")
+
+
+def run_driver(case, tmp, params, files):
+    assert os.path.exists(DRIVER), "build the host layer first: make -C eddl_amd/host"
+    with open(tmp / "params.txt", "w") as fh:
+        fh.write(" ".join(str(p) for p in params))
+    for name, arr in files.items():
+        np.ascontiguousarray(arr, np.float32).tofile(tmp / name)
+    res = subprocess.run([DRIVER, case, str(tmp)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr[-2000:]
+    return res
+
+
+def read(tmp, name):
+    shape = [int(v) for v in open(tmp / (name + ".shape")).read().split()]
+    return np.fromfile(tmp / (name + ".bin"), np.float32).reshape(shape)
+
+
+def test_conv2d_through_descriptors(oracle, golden, tmp_path):
+    for case in golden["conv2d"]:
+        x = tensor_of(case["image"])
+        kshape = (case["filters"], x.shape[1], *case["kernel"])
+        w = np.ones(kshape, np.float32) if case["filters_data"] == "ones" else tensor_of(case["filters_data"])
+        b = np.zeros(case["filters"], np.float32) if case["bias_data"] == "zeros" else tensor_of(case["bias_data"])
+        run_driver("conv2d", tmp_path, [*x.shape, case["filters"], *case["kernel"], *case["strides"], int(case["use_bias"]), case["padding"]],
+                   {"I.bin": x, "K.bin": w, "bias.bin": b})
+        assert np.array_equal(read(tmp_path, "O"), tensor_of(case["forward"])), case["name"]
+    rng = np.random.default_rng(50)
+    for (N, C, H, W, Kf, R, S, sr, sc, padding, pads) in [(4, 32, 28, 28, 64, 3, 3, 1, 1, "same", None),
+                                                           (2, 3, 37, 41, 16, 7, 7, 2, 2, "custom", [3, 3, 3, 3]),
+                                                           (3, 5, 17, 13, 7, 3, 3, 2, 2, "same", None)]:
+        x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+        w = (rng.standard_normal((Kf, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32)
+        b = rng.standard_normal(Kf, dtype=np.float32)
+        run_driver("conv2d", tmp_path, [N, C, H, W, Kf, R, S, sr, sc, 1, padding] + (pads or []), {"I.bin": x, "K.bin": w, "bias.bin": b})
+        P, Q, p4 = oracle.conv_geometry(H, W, R, S, sr, sc, padding, pads)
+        ref = oracle.conv2d(x, w, b, (sr, sc), p4[0], p4[2], P, Q)
+        out = read(tmp_path, "O")
+        assert out.shape == ref.shape
+        atol = 1e-5 * float(np.abs(ref).max())
+        assert np.all(np.abs(ref - out) <= atol + 1e-4 * np.abs(ref))
+
+
+def test_pools_through_descriptors(oracle, golden, tmp_path):
+    for case in golden["maxpool2d"]:
+        x = tensor_of(case["image"])
+        run_driver("mpool", tmp_path, [*x.shape, *case["kernel"], *case["strides"], case["padding"]], {"I.bin": x})
+        assert np.array_equal(read(tmp_path, "O"), tensor_of(case["forward"])), case["name"]
+    for case in golden["avgpool2d"]:
+        x = tensor_of(case["image"])
+        run_driver("avgpool", tmp_path, [*x.shape, *case["kernel"], *case["strides"], case["padding"]], {"I.bin": x})
+        np.testing.assert_allclose(read(tmp_path, "O"), tensor_of(case["forward"]), atol=case["atol"])
+    rng = np.random.default_rng(51)
+    x = rng.integers(-3, 4, size=(2, 8, 28, 28)).astype(np.float32)
+    run_driver("mpool", tmp_path, [2, 8, 28, 28, 3, 3, 2, 2, "custom", 1, 1, 1, 1], {"I.bin": x})
+    O, ix, iy = oracle.maxpool2d(x, (3, 3), (2, 2), (1, 1, 1, 1), fill=-1.0)
+    assert np.array_equal(read(tmp_path, "O"), O) and np.array_equal(read(tmp_path, "indX"), ix) and np.array_equal(read(tmp_path, "indY"), iy)
+    x = rng.standard_normal((2, 16, 7, 7), dtype=np.float32)
+    run_driver("avgpool", tmp_path, [2, 16, 7, 7, 7, 7, 1, 1, "none"], {"I.bin": x})
+    assert np.array_equal(read(tmp_path, "O"), oracle.avgpool2d(x, (7, 7), (1, 1), (0, 0, 0, 0)))
+
+
+def test_batchnorm_and_layer_chain(oracle, tmp_path):
+    rng = np.random.default_rng(52)
+    N, C, H, W = 3, 6, 5, 7
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    mean = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    var = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    g = rng.uniform(0.8, 1.2, C).astype(np.float32)
+    b = (rng.standard_normal(C) * 0.1).astype(np.float32)
+    run_driver("bn", tmp_path, [N, C, H, W, 1e-5, 1], {"I.bin": x, "mean.bin": mean, "var.bin": var, "g.bin": g, "b.bin": b})
+    y, opa, sd = oracle.batchnorm_inference(x, mean, var, g, b, 1e-5)
+    assert np.array_equal(read(tmp_path, "O"), y) and np.array_equal(read(tmp_path, "opa"), opa) and np.array_equal(read(tmp_path, "bn_var"), sd)
+
+    ndim = 10
+    skip = rng.standard_normal((N, C, 2 * H + 1, 2 * W + 1), dtype=np.float32)
+    feat = 2 * C * (2 * H + 1) * (2 * W + 1)
+    Wd = (rng.standard_normal((feat, ndim)) * np.sqrt(2.0 / feat)).astype(np.float32)
+    bd = rng.standard_normal(ndim, dtype=np.float32)
+    run_driver("chain", tmp_path, [N, C, H, W, ndim], {"I.bin": x, "skip.bin": skip, "W.bin": Wd, "b.bin": bd})
+    up = oracle.scale_nearest(x, (2 * H, 2 * W))
+    cat = oracle.concat([skip, oracle.pad(up, (0, 1, 1, 0))], 1)
+    assert np.array_equal(read(tmp_path, "cat"), cat)
+    s = oracle.add(cat, cat)
+    act = oracle.relu((np.zeros_like(cat) + cat) + s)
+    assert np.array_equal(read(tmp_path, "act").reshape(act.shape), act)
+    dense = oracle.dense(act.reshape(N, feat), Wd, bd)
+    got = read(tmp_path, "dense")
+    assert np.all(np.abs(dense - got) <= 1e-5 * np.abs(dense).max() + 1e-4 * np.abs(dense))
+    np.testing.assert_allclose(read(tmp_path, "prob"), oracle.softmax(got, 1), rtol=2e-6, atol=1e-8)
+    np.testing.assert_allclose(read(tmp_path, "sig"), oracle.sigmoid(got), rtol=1e-6, atol=1e-7)
+
+
+def test_error_behaviour_follows_the_reference(tmp_path):
+    res = run_driver("errors", tmp_path, [], {})
+    assert "errors OK" in res.stdout
+    assert "⚠️" in res.stderr  # the reference's msg() banner
