@@ -45,25 +45,34 @@ def build_workload(name):
 
 
 def time_ops(hip, model, reps):
-    """Per-op device time (ms, mean over reps) from events on the stream the kernels run on.
-    Convolutions are bracketed inside the library around the matrix-core kernel only."""
+    """Per-op device time (ms, mean over reps) from events on the stream the kernels run on: the
+    whole op (repack + kernels) between two events and, for convolutions, the launches of the
+    convolution kernel alone, each bracketed inside the library."""
     n = len(model.ops)
     ev = [[(hip.event(), hip.event()) for _ in range(n)] for _ in range(reps)]
     kernels = [None] * n
+    kern_ms = [0.0] * n
+    kern_launches = [0] * n
     for r in range(reps):
         for i, op in enumerate(model.ops):
             s, e = ev[r][i]
             if op.kind == "conv2d":
-                hip.set_conv_profile_events(s, e)
+                hip.conv_profile(True)
+                s.record()
                 op.run()
-                hip.set_conv_profile_events(None, None)
+                e.record()
+                launches, ms = hip.conv_profile_read()
+                hip.conv_profile(False)
                 kernels[i] = hip.last_conv_kernel().split(" +ksplit")[0]
+                kern_ms[i] += ms / reps
+                kern_launches[i] = launches
             else:
                 s.record()
                 op.run()
                 e.record()
     hip.synchronize()
-    return [float(np.mean([ev[r][i][0].elapsed_ms(ev[r][i][1]) for r in range(reps)])) for i in range(n)], kernels
+    op_ms = [float(np.mean([ev[r][i][0].elapsed_ms(ev[r][i][1]) for r in range(reps)])) for i in range(n)]
+    return op_ms, kernels, kern_ms, kern_launches
 
 
 def cpu_baseline(workload, want_seconds=20.0):
@@ -122,6 +131,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-op table to stderr")
     ap.add_argument("--conv-algo", default="auto", choices=["auto", "mfma_staged", "mfma_lds"], help="input gather of the convolution kernels")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="after the timed region run one ReLU over 2^26 floats (reads 256 MiB, writes 256 MiB): the plain copy "
+                         "kernel of known size that scales FETCH_SIZE / WRITE_SIZE counter readings")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on ONE GPU (the forward path has no collectives); --gpus %d is not supported" % args.gpus)
@@ -148,14 +160,20 @@ def main():
     if not np.all(np.isfinite(out_host)):
         sys.exit("bench.py: non-finite output")
 
+    if args.copy_probe:
+        probe_in, probe_out = hip.full((1 << 26,), 1.0), hip.empty((1 << 26,))
+        hip.relu(probe_in, probe_out)
+        hip.synchronize()
+        del probe_in, probe_out
+
     # ---- per-op device times (events on the kernels' stream), same resident input
     reps = max(3, min(args.steps, 10))
-    op_ms, op_kernels = time_ops(hip, model, reps)
+    op_ms, op_kernels, kern_ms, kern_launches = time_ops(hip, model, reps)
     rows = []
-    for op, ms, kern in zip(model.ops, op_ms, op_kernels):
+    for op, ms, kern, kms, kl in zip(model.ops, op_ms, op_kernels, kern_ms, kern_launches):
         row = {"op": op.kind, "name": op.name, "ms": ms, "flops": op.flops, "bytes": op.bytes}
         if kern:
-            row["kernel"] = kern
+            row.update(kernel=kern, kernel_ms=kms, kernel_launches=kl)
         if op.kind in ("conv2d", "dense") and ms > 0:
             row["tflops"] = op.flops / ms / 1e9
             row["frac_fp32_mfma_peak"] = row["tflops"] / PEAK_FP32_MFMA_TFLOPS
@@ -170,8 +188,9 @@ def main():
     by_kernel = {}
     for r in conv_rows:
         by_kernel.setdefault(r.get("kernel", "?"), []).append(r)
-    dom_name, dom = max(by_kernel.items(), key=lambda kv: sum(r["ms"] for r in kv[1]))
-    dom_flops, dom_ms = sum(r["flops"] for r in dom), sum(r["ms"] for r in dom)
+    dom_name, dom = max(by_kernel.items(), key=lambda kv: sum(r["kernel_ms"] for r in kv[1]))
+    dom_flops, dom_ms = sum(r["flops"] for r in dom), sum(r["kernel_ms"] for r in dom)
+    dom_launches = sum(r["kernel_launches"] for r in dom)
     achieved = dom_flops / dom_ms / 1e9 if dom_ms > 0 else 0.0
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "traffic_%s.json" % args.workload)
@@ -180,8 +199,9 @@ def main():
             traffic = json.load(fh).get("hbm_bytes_per_launch")
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": traffic,
-                "kernel": dom_name, "launches_per_step": len(dom),
-                "flops_per_launch": dom_flops / max(len(dom), 1), "avg_launch_ms": dom_ms / max(len(dom), 1)}
+                "kernel": dom_name, "launches_per_step": dom_launches, "layers": len(dom),
+                "flops_per_launch": dom_flops / max(dom_launches, 1), "avg_launch_ms": dom_ms / max(dom_launches, 1),
+                "algorithmic_bytes_per_launch": sum(r["bytes"] for r in dom) / max(dom_launches, 1)}
 
     conv_ms = sum(r["ms"] for r in conv_rows)
     conv_flops = sum(r["flops"] for r in conv_rows)

@@ -140,9 +140,15 @@ class Backend:
     def last_conv_kernel(self):
         return self.lib.eddlhip_conv2d_last_kernel().decode()
 
-    def set_conv_profile_events(self, start=None, stop=None):
-        """Bracket the matrix-core kernel of the following conv2D calls with two events (None, None removes them)."""
-        self._check(self.lib.eddlhip_conv2d_set_profile_events(start.handle if start else None, stop.handle if stop else None))
+    def conv_profile(self, collect):
+        """Start (True) or stop (False) bracketing every convolution-kernel launch with events."""
+        self._check(self.lib.eddlhip_conv2d_profile(int(bool(collect))))
+
+    def conv_profile_read(self):
+        """(launches, total milliseconds) of the convolution-kernel launches since collection started."""
+        n, ms = ctypes.c_int(), ctypes.c_float()
+        self._check(self.lib.eddlhip_conv2d_profile_read(ctypes.byref(n), ctypes.byref(ms)))
+        return n.value, ms.value
 
     # ---- operators (names follow the reference's gpu_* functions)
     def fill_(self, A, v):

@@ -37,6 +37,9 @@
 // XCD's L2.
 #include <stdio.h>
 
+#include <utility>
+#include <vector>
+
 #include "common.h"
 
 using namespace eddlhip;
@@ -584,7 +587,32 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvParams p) {
 
 // ---------------------------------------------------------------- host side
 int g_algo = 0;
-hipEvent_t g_prof_start = nullptr, g_prof_stop = nullptr;  // optional: bracket the main kernel of the next calls
+// Measurement: while collecting, every launch of a convolution kernel (not the filter repack, not
+// the K-split finishing kernel) is bracketed by its own pair of events on the launch stream.
+bool g_prof_on = false;
+std::vector<std::pair<hipEvent_t, hipEvent_t>> g_prof_pairs;  // recorded since collection was switched on
+std::vector<std::pair<hipEvent_t, hipEvent_t>> g_prof_free;   // reusable
+
+int prof_begin(hipStream_t st) {
+    if (!g_prof_on) return 0;
+    std::pair<hipEvent_t, hipEvent_t> pr;
+    if (!g_prof_free.empty()) {
+        pr = g_prof_free.back();
+        g_prof_free.pop_back();
+    } else {
+        EH_TRY_HIP(hipEventCreate(&pr.first));
+        EH_TRY_HIP(hipEventCreate(&pr.second));
+    }
+    g_prof_pairs.push_back(pr);
+    EH_TRY_HIP(hipEventRecord(pr.first, st));
+    return 0;
+}
+
+int prof_end(hipStream_t st) {
+    if (!g_prof_on) return 0;
+    EH_TRY_HIP(hipEventRecord(g_prof_pairs.back().second, st));
+    return 0;
+}
 thread_local char g_last_kernel[128] = "";
 int g_split = 1;  // divide the tiles of a mostly idle last round along K (set_algo 5 turns it off)
 
@@ -694,10 +722,24 @@ int eddlhip_conv2d_set_algo(int algo) {
     return 0;
 }
 
-int eddlhip_conv2d_set_profile_events(void *start, void *stop) {
-    EH_REQUIRE((start == nullptr) == (stop == nullptr), "conv2d_set_profile_events: give both events or neither");
-    g_prof_start = (hipEvent_t)start;
-    g_prof_stop = (hipEvent_t)stop;
+int eddlhip_conv2d_profile(int collect) {
+    for (auto &pr : g_prof_pairs) g_prof_free.push_back(pr);
+    g_prof_pairs.clear();
+    g_prof_on = collect != 0;
+    return 0;
+}
+
+int eddlhip_conv2d_profile_read(int *launches, float *total_ms) {
+    EH_REQUIRE(launches && total_ms, "conv2d_profile_read: NULL output");
+    float sum = 0.0f;
+    for (auto &pr : g_prof_pairs) {
+        float ms = 0.0f;
+        EH_TRY_HIP(hipEventSynchronize(pr.second));
+        EH_TRY_HIP(hipEventElapsedTime(&ms, pr.first, pr.second));
+        sum += ms;
+    }
+    *launches = (int)g_prof_pairs.size();
+    *total_ms = sum;
     return 0;
 }
 
@@ -741,10 +783,10 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     if (g_algo == 2) {
         size_t total = (size_t)p.npix * Kf;
         snprintf(g_last_kernel, sizeof(g_last_kernel), "conv_direct_kernel");
-        if (g_prof_start) EH_TRY_HIP(hipEventRecord(g_prof_start, st));
+        EH_TRY(prof_begin(st));
         hipLaunchKernelGGL(conv_direct_kernel, dim3(eh_blocks(total, 256, 1u << 20)), dim3(256), 0, st, p);
         EH_CHECK_LAUNCH();
-        if (g_prof_stop) EH_TRY_HIP(hipEventRecord(g_prof_stop, st));
+        EH_TRY(prof_end(st));
         return 0;
     }
 
@@ -785,7 +827,6 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     hipLaunchKernelGGL(pack_filters_kernel, dim3((rows + 31) / 32, p.Mp / 32), dim3(256), 0, st, K, (float *)ws, Kf, p.CRS, p.Mp, rows);
     EH_CHECK_LAUNCH();
 
-    if (g_prof_start) EH_TRY_HIP(hipEventRecord(g_prof_start, st));
     for (long long b0 = 0; b0 < N; b0 += chunk_imgs) {
         const int nb = (int)((N - b0 < chunk_imgs) ? N - b0 : chunk_imgs);
         ConvParams q = p;
@@ -805,20 +846,23 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
             q.tile0 = 0;
             q.nslices = 1;
             q.slice_steps = p.nsteps;
+            EH_TRY(prof_begin(st));
             hipLaunchKernelGGL(v->kernel, dim3((unsigned)main_tiles), dim3(256), 0, st, q);
             EH_CHECK_LAUNCH();
+            EH_TRY(prof_end(st));
         }
         if (split_tiles > 0) {
             q.tile0 = (int)main_tiles;
             q.nslices = nslices;
             q.slice_steps = slice_steps;
+            EH_TRY(prof_begin(st));
             hipLaunchKernelGGL(v->kernel, dim3((unsigned)(split_tiles * nslices)), dim3(256), 0, st, q);
             EH_CHECK_LAUNCH();
+            EH_TRY(prof_end(st));
             hipLaunchKernelGGL(v->reduce, dim3((unsigned)split_tiles), dim3(256), 0, st, q);
             EH_CHECK_LAUNCH();
         }
     }
-    if (g_prof_stop) EH_TRY_HIP(hipEventRecord(g_prof_stop, st));
     if (leftover > 0) snprintf(g_last_kernel, sizeof(g_last_kernel), "%s +ksplit(%lld tiles x %d)", v->name, leftover, nslices);
     else snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", v->name);
     return 0;

@@ -101,11 +101,15 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
 int eddlhip_conv2d_set_algo(int algo);
 const char *eddlhip_conv2d_last_kernel(void);
 
-/* Measurement hook (no counterpart in the reference): while two events are installed, every
- * eddlhip_conv2d_fwd records `start` on the device's stream immediately before its main
- * (matrix-core) kernel and `stop` immediately after it, leaving the filter repack outside the
- * bracket.  Pass NULL, NULL to remove them. */
-int eddlhip_conv2d_set_profile_events(void *start, void *stop);
+/* Measurement hook (no counterpart in the reference).  eddlhip_conv2d_profile(1) starts a
+ * collection: from then on every launch of a convolution kernel made by eddlhip_conv2d_fwd
+ * (one per call, two when the last round is divided along K; not the filter repack, not the
+ * finishing kernel of a K-split) is bracketed by its own pair of events on the device's stream.
+ * eddlhip_conv2d_profile_read waits for those launches and returns how many there were and the
+ * sum of their durations; eddlhip_conv2d_profile(0) stops collecting.  Either call of
+ * eddlhip_conv2d_profile forgets what was collected before. */
+int eddlhip_conv2d_profile(int collect);
+int eddlhip_conv2d_profile_read(int *launches, float *total_ms);
 
 /* ------------------------------------------------------------------ batch normalisation (inference)
  * Replaces gpu_batchnorm_forward(...) with trmode == false
