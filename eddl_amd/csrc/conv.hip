@@ -141,35 +141,78 @@ __device__ __forceinline__ void store_partial(const ConvParams &p, floatx16 (&ac
             for (int v = 0; v < 16; v++) dst[((tm * TN + tn) * 16 + v) * 64] = acc[tm][tn][v];
 }
 
+// The per-channel constants of a tile's BM channels, computed once per workgroup into LDS
+// (layout: bias[BM], mean[BM], sd[BM], g[BM], b[BM]); the caller synchronises before and after.
+template <int BM>
+__device__ __forceinline__ void stage_channel_constants(const ConvParams &p, float *epi, int m0, int tid) {
+    if (tid < BM) {
+        const int k = m0 + tid;
+        ChannelEpilogue e = {0.0f, 0.0f, 1.0f, 1.0f, 0.0f};
+        if (k < p.Kf) e = load_channel(p, k);
+        epi[tid] = e.bias;
+        epi[BM + tid] = e.mean;
+        epi[2 * BM + tid] = e.sd;
+        epi[3 * BM + tid] = e.g;
+        epi[4 * BM + tid] = e.b;
+    }
+}
+
 // Writes a wavefront's TM x TN blocks.  A lane holds column (pixel) lane%32 and rows
 // 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 block: for a fixed v the 32 lanes of a half
 // wavefront store 32 consecutive pixels of one channel plane (128 contiguous bytes).
-template <int TM, int TN>
-__device__ __forceinline__ void store_tile(const ConvParams &p, floatx16 (&acc)[TM][TN], int m_base, long long n_base, int lane) {
+// `epi` holds the tile's channel constants (stage_channel_constants); m_local is the first of the
+// wavefront's rows within the tile.  The residual values of a 32-row block are all requested
+// before the first of them is used, so their latencies overlap.
+template <int TM, int TN, int BM>
+__device__ __forceinline__ void store_tile(const ConvParams &p, floatx16 (&acc)[TM][TN], const float *epi, int m0, int m_local, int n_base,
+                                           int lane) {
     size_t obase[TN];
     bool nok[TN];
 #pragma unroll
     for (int tn = 0; tn < TN; tn++) {
-        const long long n = n_base + tn * 32 + (lane & 31);
-        nok[tn] = n < p.npix;
-        const long long nc = nok[tn] ? n : 0;
-        const int img = (int)(nc / p.PQ);
-        const int pq = (int)(nc - (long long)img * p.PQ);
+        const int n = n_base + tn * 32 + (lane & 31);
+        nok[tn] = n < (int)p.npix;
+        const unsigned nc = nok[tn] ? (unsigned)n : 0u;
+        const unsigned img = nc / (unsigned)p.PQ;
+        const unsigned pq = nc - img * (unsigned)p.PQ;
         obase[tn] = (size_t)img * p.Kf * p.PQ + pq;
     }
+    const bool has_res = p.residual != nullptr;
 #pragma unroll
     for (int tm = 0; tm < TM; tm++) {
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int m = m_base + tm * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-            if (m < p.Kf) {
-                const ChannelEpilogue e = load_channel(p, m);
+        for (int vh = 0; vh < 16; vh += 8) {  // eight rows at a time: their residual loads are in flight together
+            float res[8][TN];
+            if (has_res) {
+#pragma unroll
+                for (int vv = 0; vv < 8; vv++) {
+                    const int v = vh + vv;
+                    const int ml = m_local + tm * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                    const bool mok = m0 + ml < p.Kf;
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) {
+                        const size_t oidx = (mok && nok[tn]) ? obase[tn] + (size_t)(m0 + ml) * p.PQ : 0;
+                        res[vv][tn] = p.residual[oidx];
+                    }
+                }
+            }
+#pragma unroll
+            for (int vv = 0; vv < 8; vv++) {
+                const int v = vh + vv;
+                const int ml = m_local + tm * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                const bool mok = m0 + ml < p.Kf;
+                const float bias = epi[ml], mean = epi[BM + ml], sd = epi[2 * BM + ml], g = epi[3 * BM + ml], b = epi[4 * BM + ml];
 #pragma unroll
                 for (int tn = 0; tn < TN; tn++) {
-                    if (nok[tn]) {
-                        const size_t oidx = obase[tn] + (size_t)m * p.PQ;
-                        p.O[oidx] = apply_epilogue(p, e, acc[tm][tn][v], oidx);
+                    float x = acc[tm][tn][v];
+                    if (p.bias) x = __fadd_rn(x, bias);
+                    if (p.bn_mean) {
+                        x = __fdiv_rn(__fsub_rn(x, mean), sd);
+                        if (p.bn_g) x = __fadd_rn(__fmul_rn(x, g), b);
                     }
+                    if (has_res) x = __fadd_rn(x, res[vv][tn]);
+                    if (p.relu) x = x > 0.0f ? x : 0.0f;
+                    if (mok && nok[tn]) p.O[obase[tn] + (size_t)(m0 + ml) * p.PQ] = x;
                 }
             }
         }
@@ -202,7 +245,7 @@ __global__ __launch_bounds__(256) void pack_filters_kernel(const float *__restri
 // serves one 64-pixel segment of the tile (its lanes = 64 consecutive output pixels) and CPW of
 // the step's channels; each of its loads is one (channel, tap) row segment of 64 floats.
 template <int WM, int WN, int TM, int TN, int R, int S, int CPB, bool DIRECT>
-__global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
+__global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(const ConvParams p) {  // registers for 3 (4) workgroups per CU
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int RS = R * S, BK = CPB * RS;
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
@@ -236,12 +279,12 @@ __global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
     const int seg = wave % NS, cg = wave / NS;
     int voff[RS];
     {
-        const long long ng = n0 + seg * 64 + lane;
-        const bool pvalid = ng < p.npix;
-        const long long ngc = pvalid ? ng : 0;
-        const int img = (int)(ngc / p.PQ);
-        const int pq = (int)(ngc - (long long)img * p.PQ);
-        const int op = pq / p.Q, oq = pq - op * p.Q;
+        const int ng = (int)n0 + seg * 64 + lane;  // a launch covers fewer than 2^31 pixels
+        const bool pvalid = ng < (int)p.npix;
+        const unsigned ngc = pvalid ? (unsigned)ng : 0u;
+        const int img = (int)(ngc / (unsigned)p.PQ);
+        const int pq = (int)(ngc - (unsigned)img * (unsigned)p.PQ);
+        const int op = (int)((unsigned)pq / (unsigned)p.Q), oq = pq - op * p.Q;
         const int ih0 = op * p.sr - p.pt, iw0 = oq * p.sc - p.pl;
         const int pix = img * (p.C * p.H * p.W) + ih0 * p.W + iw0;
 #pragma unroll
@@ -363,15 +406,21 @@ __global__ __launch_bounds__(256) void conv_tap_kernel(const ConvParams p) {
         __syncthreads();
     }
 
-    if (p.nslices > 1) store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
-    else store_tile<TM, TN>(p, acc, m0 + wm * TM * 32, n0 + wn * TN * 32, lane);
+    if (p.nslices > 1) {
+        store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
+    } else {
+        float *epi = &As[0][0];  // the K loop ended with a barrier: the filter buffers are free
+        stage_channel_constants<BM>(p, epi, m0, tid);
+        __syncthreads();
+        store_tile<TM, TN, BM>(p, acc, epi, m0, wm * TM * 32, (int)n0 + wn * TN * 32, lane);
+    }
 }
 
 // ---------------------------------------------------------------- MFMA kernel, any filter shape
 // K-step = 16 taps.  Thread t gathers pixel t % BN for EPT consecutive taps of the step; the tap
 // walk (c, ky, kx) is uniform in a wavefront and advances with scalar arithmetic.
 template <int WM, int WN, int TM, int TN>
-__global__ __launch_bounds__(256) void conv_gen_kernel(const ConvParams p) {
+__global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(const ConvParams p) {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int BK = 16;
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
@@ -403,12 +452,12 @@ __global__ __launch_bounds__(256) void conv_gen_kernel(const ConvParams p) {
     int ih0, iw0, pix;
     bool pvalid;
     {
-        const long long ng = n0 + bn_l;
-        pvalid = ng < p.npix;
-        const long long ngc = pvalid ? ng : 0;
-        const int img = (int)(ngc / p.PQ);
-        const int pq = (int)(ngc - (long long)img * p.PQ);
-        const int op = pq / p.Q, oq = pq - op * p.Q;
+        const int ng = (int)n0 + bn_l;  // a launch covers fewer than 2^31 pixels
+        pvalid = ng < (int)p.npix;
+        const unsigned ngc = pvalid ? (unsigned)ng : 0u;
+        const int img = (int)(ngc / (unsigned)p.PQ);
+        const int pq = (int)(ngc - (unsigned)img * (unsigned)p.PQ);
+        const int op = (int)((unsigned)pq / (unsigned)p.Q), oq = pq - op * p.Q;
         ih0 = op * p.sr - p.pt;
         iw0 = oq * p.sc - p.pl;
         pix = img * (p.C * p.H * p.W) + ih0 * p.W + iw0;
@@ -513,8 +562,14 @@ __global__ __launch_bounds__(256) void conv_gen_kernel(const ConvParams p) {
         __syncthreads();
     }
 
-    if (p.nslices > 1) store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
-    else store_tile<TM, TN>(p, acc, m0 + wm * TM * 32, n0 + wn * TN * 32, lane);
+    if (p.nslices > 1) {
+        store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
+    } else {
+        float *epi = &As[0][0];  // the K loop ended with a barrier: the filter buffers are free
+        stage_channel_constants<BM>(p, epi, m0, tid);
+        __syncthreads();
+        store_tile<TM, TN, BM>(p, acc, epi, m0, wm * TM * 32, (int)n0 + wn * TN * 32, lane);
+    }
 }
 
 // ---------------------------------------------------------------- finishing kernel of K-split tiles
@@ -550,7 +605,10 @@ __global__ __launch_bounds__(256) void conv_reduce_kernel(const ConvParams p) {
                     acc[tm][tn][v] = sl == 0 ? x : __fadd_rn(acc[tm][tn][v], x);
                 }
     }
-    store_tile<TM, TN>(p, acc, m0 + wm * TM * 32, n0 + wn * TN * 32, lane);
+    __shared__ float epi[5 * BM];
+    stage_channel_constants<BM>(p, epi, m0, tid);
+    __syncthreads();
+    store_tile<TM, TN, BM>(p, acc, epi, m0, wm * TM * 32, (int)n0 + wn * TN * 32, lane);
 }
 
 // ---------------------------------------------------------------- scalar direct kernel
@@ -804,7 +862,11 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
             family[t].occupancy = occ > 0 ? occ : 1;
         }
     }
-    const long long max_imgs = (1LL << 29) / img_elems;  // a buffer descriptor addresses 2 GiB with 32-bit offsets
+    // a launch covers one batch chunk: input within the 2 GiB a buffer descriptor addresses with 32-bit
+    // offsets, and fewer than 2^31 output pixels (32-bit pixel arithmetic in the kernels)
+    long long max_imgs = (1LL << 29) / img_elems;
+    if (max_imgs > 0x7ffffe00LL / p.PQ) max_imgs = 0x7ffffe00LL / p.PQ;
+    EH_REQUIRE(max_imgs >= 1, "conv2d: one output plane of %d pixels is too large", p.PQ);
     const int chunk_imgs = (int)((N < max_imgs) ? N : max_imgs);
     const Plan plan = plan_conv(family, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu, g_split != 0);
     const Variant *v = &family[plan.tile];
