@@ -66,7 +66,7 @@ struct ConvParams {
     int CRS, Mp, nsteps, PQ;
     long long npix;
     int gm, gn;
-    unsigned in_bytes;  // size the input's buffer descriptor covers
+    unsigned in_bytes, wp_bytes;  // sizes the input's and the packed filters' buffer descriptors cover
     // Tiles [tile0, tile0 + gridDim.x / nslices) are computed by this launch.  With nslices > 1 a
     // tile's K-steps are divided over nslices workgroups of slice_steps steps each, which write
     // their raw accumulators to `partial`; conv_reduce_kernel adds the slices and finishes the tile.
@@ -313,16 +313,39 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     }
     const int a_step = BK * p.Mp;
 
-    floatx4 areg[AV];
+    floatx4 areg[DIRECT ? 1 : AV];
     float breg[DIRECT ? 1 : CPW * RS];
 
-    auto load_a = [&](int step) {
+    // LDS-direct filter slice: a wavefront instruction moves one 64-float segment of one row; a row
+    // has BM/64 segments (BM = 32: half a segment, the upper lanes are sent out of range and write zeros
+    // into the row's padding).  Segment u of the slice belongs to wavefront u % 4.
+    constexpr int A_SEGS = BM >= 64 ? BM / 64 : 1;
+    constexpr int A_UNITS = BK * A_SEGS;
+    constexpr int A_UPW = (A_UNITS + 3) / 4;
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc((void *)p.Wp, 0, p.wp_bytes, RSRC_WORD3);
+    const int a_voff_direct = (BM >= 64 || lane < BM) ? (m0 + lane) * 4 : OOB;
+
+    auto load_a = [&](int step, int buf) {
+        if constexpr (DIRECT) {
 #pragma unroll
-        for (int j = 0; j < AV; j++) areg[j] = *reinterpret_cast<const floatx4 *>(a_ptr[j] + (size_t)step * a_step);
+            for (int j = 0; j < A_UPW; j++) {
+                const int u = wave + 4 * j;
+                if (A_UNITS % 4 == 0 || j < A_UPW - 1 || u < A_UNITS) {  // uniform in the wavefront
+                    const int kk = u / A_SEGS, sg = u % A_SEGS;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void *)&As[buf][kk * LDA + sg * 64], 4, a_voff_direct,
+                                                             ((step * BK + kk) * p.Mp + sg * 64) * 4, 0, 0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < AV; j++) areg[j] = *reinterpret_cast<const floatx4 *>(a_ptr[j] + (size_t)step * a_step);
+        }
     };
     auto store_a = [&](int buf) {
+        if constexpr (!DIRECT) {
 #pragma unroll
-        for (int j = 0; j < AV; j++) *reinterpret_cast<floatx4 *>(&As[buf][a_lds[j]]) = areg[j];
+            for (int j = 0; j < AV; j++) *reinterpret_cast<floatx4 *>(&As[buf][a_lds[j]]) = areg[j];
+        }
     };
     // gather of one step; `checked` adds the test for channels past C (last step of an odd channel count)
     auto load_b = [&](int step, int buf, bool checked) {
@@ -361,7 +384,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
             for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.0f;
 
     const int full_steps = p.C / CPB;  // steps whose channels all exist
-    load_a(step_lo);
+    load_a(step_lo, 0);
     load_b(step_lo, 0, step_lo >= full_steps);
     store_a(0);
     store_b(0);
@@ -374,7 +397,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         const int buf = (step - step_lo) & 1;
         const bool more = step + 1 < step_hi;
         if (more) {
-            load_a(step + 1);
+            load_a(step + 1, buf ^ 1);
             if (step + 1 < full_steps) load_b(step + 1, buf ^ 1, false);
             else load_b(step + 1, buf ^ 1, true);
         }
@@ -835,7 +858,7 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     p.gm = p.gn = 0;
     p.nsteps = 0;
     p.Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
-    p.in_bytes = 0;
+    p.in_bytes = p.wp_bytes = 0;
     p.tile0 = 0; p.nslices = 1; p.slice_steps = 0; p.partial = nullptr;
 
     if (g_algo == 2) {
@@ -849,7 +872,7 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     }
 
     // ---- kernel variant and launch plan
-    const int direct = (g_algo == 4) ? 1 : 0;
+    const int direct = (g_algo == 3) ? 0 : 1;  // default: the load unit writes LDS directly
     const Variant *family;
     if (R == 3 && S == 3) family = k3x3[direct];
     else if (R == 1 && S == 1) family = k1x1[direct];
@@ -885,6 +908,7 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     void *ws = nullptr;
     EH_TRY(get_workspace(dev, wp_bytes + partial_bytes, &ws));
     p.Wp = (const float *)ws;
+    p.wp_bytes = (unsigned)((size_t)rows * p.Mp * sizeof(float));
     p.partial = (float *)((char *)ws + wp_bytes);
     hipLaunchKernelGGL(pack_filters_kernel, dim3((rows + 31) / 32, p.Mp / 32), dim3(256), 0, st, K, (float *)ws, Kf, p.CRS, p.Mp, rows);
     EH_CHECK_LAUNCH();

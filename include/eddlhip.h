@@ -93,8 +93,8 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
 /* Selects the convolution kernel: 0 = automatic; 1 = matrix-core (MFMA) implicit GEMM;
  * 2 = the scalar direct kernel (one thread per output; taps summed in the reference's ky,kx,c
  * order with its rounding - used to cross-check the MFMA kernels on the device);
- * 3 = MFMA with the input gather staged through registers; 4 = MFMA with the input gather
- * written by the load unit straight into LDS; 5 / 6 = switch off / on the division along K of
+ * 3 = MFMA with the operand slices staged through registers; 4 = MFMA with the operand slices
+ * written by the load unit straight into LDS (what 0 and 1 select); 5 / 6 = switch off / on the division along K of
  * the tiles of a mostly idle last round of workgroups (on by default; independent of 0-4).
  * eddlhip_conv2d_last_kernel() names the kernel the calling thread's last eddlhip_conv2d_fwd
  * launched, followed by " +ksplit(T tiles x S)" when T tiles were divided into S slices. */
