@@ -49,6 +49,7 @@ namespace {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(3))) float lds_float;
 
 constexpr int M_ALIGN = 128;                  // packed filter rows are padded to this many channels
 constexpr int OOB = (int)0x80000000u;         // byte offset no buffer of <= 2 GiB contains
@@ -107,6 +108,31 @@ __device__ __forceinline__ float apply_epilogue(const ConvParams &p, const Chann
     if (p.residual) v = __fadd_rn(v, p.residual[oidx]);
     if (p.relu) v = v > 0.0f ? v : 0.0f;
     return v;
+}
+
+// LDS-direct load: the load unit writes the dword of lane i to LDS address dst + 4*i (out-of-range
+// lanes write 0).  Written as inline assembly on purpose: the compiler's wait-count insertion
+// makes every LDS read wait for ALL outstanding LDS-direct loads (it cannot tell the buffer being
+// filled from the buffer being read), which would serialise the loads of step t+1 with the MFMAs
+// of step t.  With the instruction opaque to it, the kernel places the one wait that is needed
+// itself: vmcnt(0) before the barrier that publishes the buffer.
+typedef int int32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int32x4 make_rsrc_words(const void *base, unsigned bytes) {
+    const unsigned long long a = (unsigned long long)base;
+    int32x4 r;
+    r.x = __builtin_amdgcn_readfirstlane((int)(a & 0xffffffffu));
+    r.y = __builtin_amdgcn_readfirstlane((int)((a >> 32) & 0xffffu));  // stride 0
+    r.z = __builtin_amdgcn_readfirstlane((int)bytes);
+    r.w = (int)RSRC_WORD3;
+    return r;
+}
+
+__device__ __forceinline__ void lds_dma_b32(int32x4 rsrc, lds_float *dst, int voffset, int soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                 :
+                 : "s"((unsigned)(unsigned long long)dst), "v"(voffset), "s"(rsrc), "s"(soffset)
+                 : "memory");
 }
 
 __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, int voffset, int soffset) {
@@ -322,18 +348,17 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     constexpr int A_SEGS = BM >= 64 ? BM / 64 : 1;
     constexpr int A_UNITS = BK * A_SEGS;
     constexpr int A_UPW = (A_UNITS + 3) / 4;
-    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc((void *)p.Wp, 0, p.wp_bytes, RSRC_WORD3);
+    const int32x4 dma_w = make_rsrc_words(p.Wp, p.wp_bytes), dma_in = make_rsrc_words(p.I, p.in_bytes);
     const int a_voff_direct = (BM >= 64 || lane < BM) ? (m0 + lane) * 4 : OOB;
 
-    auto load_a = [&](int step, int buf) {
+    auto load_a = [&](int step, lds_float *as) {
         if constexpr (DIRECT) {
 #pragma unroll
             for (int j = 0; j < A_UPW; j++) {
                 const int u = wave + 4 * j;
                 if (A_UNITS % 4 == 0 || j < A_UPW - 1 || u < A_UNITS) {  // uniform in the wavefront
                     const int kk = u / A_SEGS, sg = u % A_SEGS;
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void *)&As[buf][kk * LDA + sg * 64], 4, a_voff_direct,
-                                                             ((step * BK + kk) * p.Mp + sg * 64) * 4, 0, 0);
+                    lds_dma_b32(dma_w, as + kk * LDA + sg * 64, a_voff_direct, ((step * BK + kk) * p.Mp + sg * 64) * 4);
                 }
             }
         } else {
@@ -341,14 +366,19 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
             for (int j = 0; j < AV; j++) areg[j] = *reinterpret_cast<const floatx4 *>(a_ptr[j] + (size_t)step * a_step);
         }
     };
-    auto store_a = [&](int buf) {
+    auto store_a = [&](lds_float *as) {
         if constexpr (!DIRECT) {
 #pragma unroll
-            for (int j = 0; j < AV; j++) *reinterpret_cast<floatx4 *>(&As[buf][a_lds[j]]) = areg[j];
+            for (int j = 0; j < AV; j++) {
+                as[a_lds[j] + 0] = areg[j].x;
+                as[a_lds[j] + 1] = areg[j].y;
+                as[a_lds[j] + 2] = areg[j].z;
+                as[a_lds[j] + 3] = areg[j].w;
+            }
         }
     };
     // gather of one step; `checked` adds the test for channels past C (last step of an odd channel count)
-    auto load_b = [&](int step, int buf, bool checked) {
+    auto load_b = [&](int step, lds_float *bs, bool checked) {
 #pragma unroll
         for (int jc = 0; jc < CPW; jc++) {
             const int cl = cg * CPW + jc;
@@ -359,19 +389,19 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
             for (int t = 0; t < RS; t++) {
                 const int vo = cok ? voff[t] : OOB;
                 if constexpr (DIRECT) {
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_void *)&Bs[buf][(cl * RS + t) * LDB + seg * 64], 4, vo, soff, 0, 0);
+                    lds_dma_b32(dma_in, bs + (cl * RS + t) * LDB + seg * 64, vo, soff);
                 } else {
                     breg[jc * RS + t] = buf_load(rsrc_in, vo, soff);
                 }
             }
         }
     };
-    auto store_b = [&](int buf) {
+    auto store_b = [&](lds_float *bs) {
         if constexpr (!DIRECT) {
 #pragma unroll
             for (int jc = 0; jc < CPW; jc++)
 #pragma unroll
-                for (int t = 0; t < RS; t++) Bs[buf][((cg * CPW + jc) * RS + t) * LDB + seg * 64 + lane] = breg[jc * RS + t];
+                for (int t = 0; t < RS; t++) bs[((cg * CPW + jc) * RS + t) * LDB + seg * 64 + lane] = breg[jc * RS + t];
         }
     };
 
@@ -384,37 +414,33 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
             for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.0f;
 
     const int full_steps = p.C / CPB;  // steps whose channels all exist
-    load_a(step_lo, 0);
-    load_b(step_lo, 0, step_lo >= full_steps);
-    store_a(0);
-    store_b(0);
-    __syncthreads();
-
     const int a_off = (lane >> 5) * LDA + wm * TM * 32 + (lane & 31);
     const int b_off = (lane >> 5) * LDB + wn * TN * 32 + (lane & 31);
+    auto as_of = [&](int buf) { return (lds_float *)&As[buf][0]; };
+    auto bs_of = [&](int buf) { return (lds_float *)&Bs[buf][0]; };
 
-    for (int step = step_lo; step < step_hi; step++) {
-        const int buf = (step - step_lo) & 1;
-        const bool more = step + 1 < step_hi;
+    // One K-step: start the loads of the next step into the other buffer, then the MFMAs of this one.
+    auto do_step = [&](const lds_float *__restrict__ a_cur, const lds_float *__restrict__ b_cur, lds_float *__restrict__ a_nxt,
+                       lds_float *__restrict__ b_nxt, int step, bool more) __attribute__((always_inline)) {
         if (more) {
-            load_a(step + 1, buf ^ 1);
-            if (step + 1 < full_steps) load_b(step + 1, buf ^ 1, false);
-            else load_b(step + 1, buf ^ 1, true);
+            load_a(step + 1, a_nxt);
+            if (step + 1 < full_steps) load_b(step + 1, b_nxt, false);
+            else load_b(step + 1, b_nxt, true);
         }
         // operands of tap pair ks+1 are read from LDS while the MFMAs of pair ks run
         float a[2][TM], b[2][TN];
 #pragma unroll
-        for (int tm = 0; tm < TM; tm++) a[0][tm] = As[buf][a_off + tm * 32];
+        for (int tm = 0; tm < TM; tm++) a[0][tm] = a_cur[a_off + tm * 32];
 #pragma unroll
-        for (int tn = 0; tn < TN; tn++) b[0][tn] = Bs[buf][b_off + tn * 32];
+        for (int tn = 0; tn < TN; tn++) b[0][tn] = b_cur[b_off + tn * 32];
 #pragma unroll
         for (int ks = 0; ks < BK / 2; ks++) {
             const int cur = ks & 1, nxt = cur ^ 1;
             if (ks + 1 < BK / 2) {
 #pragma unroll
-                for (int tm = 0; tm < TM; tm++) a[nxt][tm] = As[buf][(ks + 1) * 2 * LDA + a_off + tm * 32];
+                for (int tm = 0; tm < TM; tm++) a[nxt][tm] = a_cur[(ks + 1) * 2 * LDA + a_off + tm * 32];
 #pragma unroll
-                for (int tn = 0; tn < TN; tn++) b[nxt][tn] = Bs[buf][(ks + 1) * 2 * LDB + b_off + tn * 32];
+                for (int tn = 0; tn < TN; tn++) b[nxt][tn] = b_cur[(ks + 1) * 2 * LDB + b_off + tn * 32];
             }
 #pragma unroll
             for (int tm = 0; tm < TM; tm++)
@@ -423,9 +449,24 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
                     acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
         }
         if (more) {
-            store_a(buf ^ 1);
-            store_b(buf ^ 1);
+            store_a(a_nxt);
+            store_b(b_nxt);
         }
+    };
+
+    load_a(step_lo, as_of(0));
+    load_b(step_lo, bs_of(0), step_lo >= full_steps);
+    store_a(as_of(0));
+    store_b(bs_of(0));
+    if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's LDS-direct loads have landed
+    __syncthreads();
+
+    for (int step = step_lo; step < step_hi; step++) {
+        const int buf = (step - step_lo) & 1;
+        do_step(as_of(buf), bs_of(buf), as_of(buf ^ 1), bs_of(buf ^ 1), step, step + 1 < step_hi);
+        // The barrier publishes the next buffer to the other wavefronts, so this wavefront's
+        // LDS-direct loads into it must be complete first.
+        if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
     }
 
