@@ -36,6 +36,7 @@ PROTOTYPES = {
     "eddlhip_conv2d_fwd": [c_int, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_set_algo": [c_int],
     "eddlhip_conv2d_last_kernel": [],
+    "eddlhip_conv2d_force_plan": [c_int, c_int],
     "eddlhip_conv2d_profile": [c_int],
     "eddlhip_conv2d_profile_read": [intp, ctypes.POINTER(c_float)],
     "eddlhip_batchnorm_inference": [c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, c_float],

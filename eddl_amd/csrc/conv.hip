@@ -281,7 +281,10 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     static_assert(BK % 2 == 0, "an MFMA consumes two taps");
     static_assert(NS == 1 || NS == 2 || NS == 4, "BN is 64, 128 or 256");
     static_assert(CPB % WPS == 0, "channels of a step divide over the wavefronts of a segment");
-    constexpr int LDA = BM + 32, LDB = BN + 32;  // +32 floats: the two halves of an operand read use different banks
+    // Rows are not padded: an operand read touches two rows (one per half wavefront) and the two
+    // halves are served in separate passes, so they do not conflict (SQ_LDS_BANK_CONFLICT reads 0),
+    // and without padding four workgroups fit in a CU's LDS instead of three.
+    constexpr int LDA = BM, LDB = BN;
     constexpr int A_VECS = BK * BM / 4;          // float4 in one filter slice
     constexpr int AV = (A_VECS + 255) / 256;     // float4 filter loads per thread per step (last one partial)
 
@@ -342,14 +345,15 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     floatx4 areg[DIRECT ? 1 : AV];
     float breg[DIRECT ? 1 : CPW * RS];
 
-    // LDS-direct filter slice: a wavefront instruction moves one 64-float segment of one row; a row
-    // has BM/64 segments (BM = 32: half a segment, the upper lanes are sent out of range and write zeros
-    // into the row's padding).  Segment u of the slice belongs to wavefront u % 4.
+    // LDS-direct filter slice: a wavefront instruction moves 64 consecutive floats of the slice in LDS:
+    // one 64-float segment of a row (BM >= 64, BM/64 segments per row) or two whole rows (BM = 32).
+    // Unit u of the slice belongs to wavefront u % 4.
     constexpr int A_SEGS = BM >= 64 ? BM / 64 : 1;
-    constexpr int A_UNITS = BK * A_SEGS;
+    constexpr int A_UNITS = BM >= 64 ? BK * A_SEGS : BK / 2;
     constexpr int A_UPW = (A_UNITS + 3) / 4;
     const int32x4 dma_w = make_rsrc_words(p.Wp, p.wp_bytes), dma_in = make_rsrc_words(p.I, p.in_bytes);
-    const int a_voff_direct = (BM >= 64 || lane < BM) ? (m0 + lane) * 4 : OOB;
+    // BM = 32: lanes 32..63 fetch the next row of the packed matrix (one row further = Mp floats)
+    const int a_voff_direct = BM >= 64 ? (m0 + lane) * 4 : (m0 + (lane & 31) + (lane >> 5) * p.Mp) * 4;
 
     auto load_a = [&](int step, lds_float *as) {
         if constexpr (DIRECT) {
@@ -357,7 +361,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
             for (int j = 0; j < A_UPW; j++) {
                 const int u = wave + 4 * j;
                 if (A_UNITS % 4 == 0 || j < A_UPW - 1 || u < A_UNITS) {  // uniform in the wavefront
-                    const int kk = u / A_SEGS, sg = u % A_SEGS;
+                    const int kk = BM >= 64 ? u / A_SEGS : 2 * u, sg = BM >= 64 ? u % A_SEGS : 0;
                     lds_dma_b32(dma_w, as + kk * LDA + sg * 64, a_voff_direct, ((step * BK + kk) * p.Mp + sg * 64) * 4);
                 }
             }
@@ -488,7 +492,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int BK = 16;
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    constexpr int LDA = BM + 32, LDB = BN + 32;
+    constexpr int LDA = BM, LDB = BN;
     constexpr int A_VECS = BK * BM / 4;
     constexpr int AV = (A_VECS + 255) / 256;
     constexpr int EPT = BN / 16;  // gathered elements per thread per step
@@ -737,6 +741,7 @@ int prof_end(hipStream_t st) {
 }
 thread_local char g_last_kernel[128] = "";
 int g_split = 1;  // divide the tiles of a mostly idle last round along K (set_algo 5 turns it off)
+int g_force_tile = -1, g_force_slices = -1;  // eddlhip_conv2d_force_plan
 
 struct Variant {
     const char *name;
@@ -830,9 +835,33 @@ Plan plan_conv(const Variant *family, int Kf, int C, int RS, long long npix, int
     return best;
 }
 
+// A plan with a given tile shape and slice count (every tile of the last round is divided; with
+// fewer tiles than one round that is every tile).
+Plan forced_plan(const Variant *family, int tile, int slices, int Kf, int C, int RS, long long npix, int num_cu) {
+    const Variant &v = family[tile];
+    Plan pl;
+    pl.tile = tile;
+    pl.nsteps = v.cpb ? (C + v.cpb - 1) / v.cpb : (C * RS + 15) / 16;
+    pl.tiles = (long long)((Kf + v.bm - 1) / v.bm) * ((npix + v.bn - 1) / v.bn);
+    pl.leftover = pl.tiles % ((long long)num_cu * v.occupancy);
+    int want = slices < 1 ? 1 : (slices > pl.nsteps ? pl.nsteps : slices);
+    pl.slice_steps = (pl.nsteps + want - 1) / want;
+    pl.nslices = (pl.nsteps + pl.slice_steps - 1) / pl.slice_steps;
+    if (pl.leftover == 0) pl.nslices = 1, pl.slice_steps = pl.nsteps;
+    pl.cost_us = 0.0;
+    return pl;
+}
+
 }  // namespace
 
 extern "C" {
+
+int eddlhip_conv2d_force_plan(int tile, int slices) {
+    EH_REQUIRE(tile >= -1 && tile <= 3, "conv2d_force_plan: tile is -1 (automatic) or 0..3");
+    g_force_tile = tile;
+    g_force_slices = slices;
+    return 0;
+}
 
 int eddlhip_conv2d_set_algo(int algo) {
     EH_REQUIRE(algo >= 0 && algo <= 6, "conv2d_set_algo: unknown algorithm %d", algo);
@@ -932,7 +961,8 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     if (max_imgs > 0x7ffffe00LL / p.PQ) max_imgs = 0x7ffffe00LL / p.PQ;
     EH_REQUIRE(max_imgs >= 1, "conv2d: one output plane of %d pixels is too large", p.PQ);
     const int chunk_imgs = (int)((N < max_imgs) ? N : max_imgs);
-    const Plan plan = plan_conv(family, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu, g_split != 0);
+    Plan plan = plan_conv(family, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu, g_split != 0);
+    if (g_force_tile >= 0) plan = forced_plan(family, g_force_tile, g_force_slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
     const Variant *v = &family[plan.tile];
     const int bk = v->cpb ? v->cpb * R * S : 16;
     p.nsteps = plan.nsteps;

@@ -101,6 +101,11 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
 int eddlhip_conv2d_set_algo(int algo);
 const char *eddlhip_conv2d_last_kernel(void);
 
+/* Overrides the launch planner of the MFMA kernels (tuning and tests): tile = 0 (128x128 outputs per
+ * workgroup), 1 (64x128), 2 (64x64), 3 (32x128) or -1 to give the choice back to the planner;
+ * slices = number of K slices the tiles of the last partial round are divided into (1 = none). */
+int eddlhip_conv2d_force_plan(int tile, int slices);
+
 /* Measurement hook (no counterpart in the reference).  eddlhip_conv2d_profile(1) starts a
  * collection: from then on every launch of a convolution kernel made by eddlhip_conv2d_fwd
  * (one per call, two when the last round is divided along K; not the filter repack, not the

@@ -206,6 +206,29 @@ def test_conv2d_ksplit_of_the_last_round(hip, oracle):
     assert split_seen >= 1, "the planner never divided a last round along K"
 
 
+@pytest.mark.parametrize("algo", ["mfma_staged", "mfma_lds"])
+def test_conv2d_every_tile_shape_and_slice_count(hip, oracle, algo):
+    """The planner's choices are overridden so that every kernel variant (4 tile shapes x filter
+    families 3x3, 1x1, 2x2, general) runs, divided along K and undivided, on ragged shapes."""
+    rng = np.random.default_rng(303)
+    shapes = [(3, 21, 20, 23, 130, 3, 3, "same"), (3, 37, 20, 23, 70, 1, 1, "valid"), (2, 10, 21, 22, 40, 2, 2, "valid"),
+              (2, 9, 19, 17, 33, 3, 2, "same")]
+    for (N, C, H, W, Kf, R, S, padding) in shapes:
+        x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+        w = (rng.standard_normal((Kf, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32)
+        b = rng.standard_normal(Kf, dtype=np.float32)
+        for tile in range(4):
+            for slices in (1, 3):
+                hip.force_conv_plan(tile, slices)
+                try:
+                    ref, out = run_conv(hip, oracle, x, w, b, (1, 1), padding, algo=algo, relu=True)
+                    name = hip.last_conv_kernel()
+                finally:
+                    hip.force_conv_plan(-1, 1)
+                assert ("+ksplit" in name) == (slices > 1), name
+                assert_conv_close(ref, out, "%s tile %d slices %d: %s" % ((N, C, H, W, Kf, R, S), tile, slices, name))
+
+
 def test_conv2d_linearity_and_empty_batch(hip, oracle):
     from eddl_amd.descriptors import ConvolDescriptor
     rng = np.random.default_rng(301)
