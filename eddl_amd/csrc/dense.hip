@@ -2,12 +2,14 @@
 // (what LDense::forward asks of mult2D: src/layers/core/layer_dense.cpp:65-73).
 //
 // At the batch sizes of CNN heads (m = 32..64 rows against a 25088 x 4096 weight matrix) the
-// product is bound by streaming B from HBM once.  One wavefront owns a 32-row x 32-column
-// output block over a slice of k and advances it with v_mfma_f32_32x32x2_f32: the B operand
-// of a step is two 128-byte row segments read straight from global memory (coalesced), the A
-// operand is two columns of the small activation matrix (L2-resident).  k is split over
-// wavefronts so the whole device streams B; the per-slice partial blocks go to the private
-// workspace and a second kernel adds them in slice order (fixed summation order, no atomics).
+// product is bound by streaming B from HBM once.  One wavefront owns a 32-row x 128-column
+// output block over a slice of k: per pair of k it loads ONE float4 of B per lane (lane l of a
+// half wavefront covers columns 4l..4l+3: 512 contiguous bytes per k row) and one dword of the
+// transposed activations, and issues four v_mfma_f32_32x32x2_f32, one per column phase
+// (accumulator j holds columns 4l + j).  The activations are transposed first (At[k][32], a few
+// MB, L2-resident) so that their loads are coalesced too.  k is split over wavefronts so the
+// whole device streams B; the per-slice partial blocks go to the private workspace and a second
+// kernel adds them in slice order (fixed summation order, no atomics).
 #include "common.h"
 
 using namespace eddlhip;
@@ -15,47 +17,103 @@ using namespace eddlhip;
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-// grid: (n tiles, k slices, m tiles); block: one wavefront
-__global__ __launch_bounds__(64) void dense_partial_kernel(const float *__restrict__ A, const float *__restrict__ B,
+// A[m][k] -> At[mt][k][32] (mt = 32-row block), zero-padded rows
+__global__ __launch_bounds__(256) void dense_transpose_kernel(const float *__restrict__ A, float *__restrict__ At, int m, int k) {
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int k0 = blockIdx.x * 32, mt = blockIdx.y;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int r = mt * 32 + ty + 8 * j, kk = k0 + tx;
+        tile[ty + 8 * j][tx] = (r < m && kk < k) ? A[(size_t)r * k + kk] : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int kk = k0 + ty + 8 * j;
+        if (kk < k) At[((size_t)mt * k + kk) * 32 + tx] = tile[tx][ty + 8 * j];
+    }
+}
+
+// grid: (column tiles of 128, k slices, row tiles of 32); block: one wavefront.
+// VEC: n is a multiple of 4 and B is 16-byte aligned, so a lane's four columns are one float4.
+template <bool VEC>
+__global__ __launch_bounds__(64) void dense_partial_kernel(const float *__restrict__ At, const float *__restrict__ B,
                                                            float *__restrict__ part, int m, int k, int n, int kslice) {
-    const int lane = threadIdx.x;
-    const int n0 = blockIdx.x * 32, ks = blockIdx.y, m0 = blockIdx.z * 32;
+    const int lane = threadIdx.x, half = lane >> 5, l = lane & 31;
+    const int n0 = blockIdx.x * 128, ks = blockIdx.y, mt = blockIdx.z;
     const int kbeg = ks * kslice;
     int kend = kbeg + kslice;
     if (kend > k) kend = k;
-    const int row = m0 + (lane & 31), col = n0 + (lane & 31), half = lane >> 5;
-    const bool rok = row < m, cok = col < n;
-    const float *ap = A + (size_t)(rok ? row : 0) * k;
-    const float *bp = B + (cok ? col : 0);
-    floatx16 acc;
+    const int col0 = n0 + 4 * l;
+    const float *ap = At + (size_t)mt * k * 32 + l;
+    floatx16 acc[4];
 #pragma unroll
-    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[j][v] = 0.0f;
+    auto load_b = [&](int ki) -> floatx4 {
+        floatx4 b = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (ki < kend) {
+            const float *row = B + (size_t)ki * n;
+            if (VEC) {
+                if (col0 < n) b = *reinterpret_cast<const floatx4 *>(row + col0);
+            } else {
+                if (col0 + 0 < n) b.x = row[col0 + 0];
+                if (col0 + 1 < n) b.y = row[col0 + 1];
+                if (col0 + 2 < n) b.z = row[col0 + 2];
+                if (col0 + 3 < n) b.w = row[col0 + 3];
+            }
+        }
+        return b;
+    };
     int kk = kbeg;
-    for (; kk + 16 <= kend; kk += 16) {
-        float a[8], b[8];
+    for (; kk + 8 <= kend; kk += 8) {  // four k pairs in flight
+        float a[4];
+        floatx4 b[4];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
+        for (int u = 0; u < 4; u++) {
             const int ki = kk + 2 * u + half;
-            a[u] = rok ? ap[ki] : 0.0f;
-            b[u] = cok ? bp[(size_t)ki * n] : 0.0f;
+            a[u] = ap[(size_t)ki * 32];
+            const float *row = B + (size_t)ki * n;
+            if (VEC) {
+                b[u] = col0 < n ? *reinterpret_cast<const floatx4 *>(row + col0) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            } else {
+                b[u] = load_b(ki);
+            }
         }
 #pragma unroll
-        for (int u = 0; u < 8; u++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+        for (int u = 0; u < 4; u++) {
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].x, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].y, acc[1], 0, 0, 0);
+            acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].z, acc[2], 0, 0, 0);
+            acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].w, acc[3], 0, 0, 0);
+        }
     }
     for (; kk < kend; kk += 2) {
         const int ki = kk + half;
-        const bool kok = ki < kend;
-        float a = (rok && kok) ? ap[ki] : 0.0f;
-        float b = (cok && kok) ? bp[(size_t)ki * n] : 0.0f;
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+        const float a = ki < kend ? ap[(size_t)ki * 32] : 0.0f;
+        const floatx4 b = load_b(ki);
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b.x, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b.y, acc[1], 0, 0, 0);
+        acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b.z, acc[2], 0, 0, 0);
+        acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b.w, acc[3], 0, 0, 0);
     }
-    // part[ks][row][col]
-    if (cok) {
+    // part[ks][row][col]: accumulator j, lane column l -> column col0 + j; rows 8*(v/4) + 4*half + v%4
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int r = m0 + 8 * (v / 4) + 4 * half + (v % 4);
-            if (r < m) part[((size_t)ks * m + r) * n + col] = acc[v];
+    for (int v = 0; v < 16; v++) {
+        const int r = mt * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+        if (r < m) {
+            float *dst = part + ((size_t)ks * m + r) * n + col0;
+            if (VEC) {
+                if (col0 < n) *reinterpret_cast<floatx4 *>(dst) = floatx4{acc[0][v], acc[1][v], acc[2][v], acc[3][v]};
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (col0 + j < n) dst[j] = acc[j][v];
+            }
         }
     }
 }
@@ -78,7 +136,7 @@ extern "C" int eddlhip_mult2d(int dev, const float *A, const float *B, float *C,
     EH_REQUIRE(A && B && C, "mult2d: NULL tensor");
     EH_TRY(use_device(dev));
     hipStream_t st = state(dev).stream;
-    const int nt = (n + 31) / 32, mt = (m + 31) / 32;
+    const int nt = (n + 127) / 128, mt = (m + 31) / 32;
     // enough wavefronts to cover the device several times over, slices of at least 64 taps
     long long want = 8LL * state(dev).num_cu;
     int nslices = (int)((want + (long long)nt * mt - 1) / ((long long)nt * mt));
@@ -88,12 +146,18 @@ extern "C" int eddlhip_mult2d(int dev, const float *A, const float *B, float *C,
     int kslice = ((k + nslices - 1) / nslices + 1) & ~1;  // even, so MFMA tap pairs do not straddle slices
     nslices = (k + kslice - 1) / kslice;
     EH_REQUIRE(nslices <= 65535 && mt <= 65535, "mult2d: shape out of range");
+    const size_t at_bytes = ((size_t)mt * k * 32 * sizeof(float) + 255) & ~(size_t)255;
     void *ws = nullptr;
-    EH_TRY(get_workspace(dev, (size_t)nslices * m * n * sizeof(float), &ws));
-    hipLaunchKernelGGL(dense_partial_kernel, dim3(nt, nslices, mt), dim3(64), 0, st, A, B, (float *)ws, m, k, n, kslice);
+    EH_TRY(get_workspace(dev, at_bytes + (size_t)nslices * m * n * sizeof(float), &ws));
+    float *At = (float *)ws, *part = (float *)((char *)ws + at_bytes);
+    hipLaunchKernelGGL(dense_transpose_kernel, dim3((k + 31) / 32, mt), dim3(256), 0, st, A, At, m, k);
+    EH_CHECK_LAUNCH();
+    const bool vec = (n % 4 == 0) && (((uintptr_t)B & 15u) == 0);
+    if (vec) hipLaunchKernelGGL(dense_partial_kernel<true>, dim3(nt, nslices, mt), dim3(64), 0, st, At, B, part, m, k, n, kslice);
+    else hipLaunchKernelGGL(dense_partial_kernel<false>, dim3(nt, nslices, mt), dim3(64), 0, st, At, B, part, m, k, n, kslice);
     EH_CHECK_LAUNCH();
     size_t mn = (size_t)m * n;
-    hipLaunchKernelGGL(dense_reduce_kernel, dim3(eh_blocks(mn, 256, 65536)), dim3(256), 0, st, (const float *)ws, C, mn, nslices, incC);
+    hipLaunchKernelGGL(dense_reduce_kernel, dim3(eh_blocks(mn, 256, 65536)), dim3(256), 0, st, (const float *)part, C, mn, nslices, incC);
     EH_CHECK_LAUNCH();
     return 0;
 }

@@ -378,7 +378,7 @@ def test_upsample_concat_pad_bit_exact(hip, oracle):
 
 def test_dense_sigmoid_softmax_within_tolerance(hip, oracle):
     rng = np.random.default_rng(405)
-    for m, k, n in [(32, 512, 1000), (5, 37, 300), (64, 2048, 10), (33, 100, 65)]:
+    for m, k, n in [(32, 512, 1000), (5, 37, 300), (64, 2048, 10), (33, 100, 65), (70, 1001, 131), (32, 3136, 4096), (1, 2, 1)]:
         a = rng.standard_normal((m, k), dtype=np.float32)
         w = (rng.standard_normal((k, n)) * np.sqrt(2.0 / k)).astype(np.float32)
         bias = rng.standard_normal(n, dtype=np.float32)
