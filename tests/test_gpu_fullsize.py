@@ -1,0 +1,144 @@
+"""Parity at the full benchmark sizes (VGG-16 batch 32, the 64x64x56x56 block, ResNet-50 batch 64,
+U-Net 4x1x512x512), where the CPU oracle cannot compute whole convolutions in test time.
+
+Every layer is checked on the DEVICE'S OWN input to that layer:
+  * bandwidth operators (BN, ReLU, pools with indices, resize, concat, add, pad): the oracle is
+    fast enough to compute them whole, and they must match bit for bit;
+  * convolutions and dense layers: the oracle's order-defined direct convolution evaluated at a
+    few thousand output coordinates (every image corner and edge region is forced into the
+    sample, so padding, the last partial tile and K-split tiles are all hit), to the conv bar;
+  * size-independent properties on top: scaling the input by a power of two scales a conv
+    output exactly; max-pool outputs equal the input gathered at the reported indices; the
+    fused plan reproduces the layer-by-layer plan bit for bit.
+"""
+import numpy as np
+import pytest
+
+from test_gpu_models import layer_oracle, EXACT
+
+pytestmark = pytest.mark.gpu
+
+NPTS = 6000
+
+
+def sample_coords(rng, shape, n):
+    """n random (b, k, p, q) plus the extremes of every axis and of the flattened pixel index."""
+    N, K, P, Q = shape
+    idx = np.stack([rng.integers(0, N, n), rng.integers(0, K, n), rng.integers(0, P, n), rng.integers(0, Q, n)], 1)
+    ext = [(b, k, p, q) for b in (0, N - 1) for k in (0, K - 1, K // 2) for p in (0, P - 1, P // 2) for q in (0, Q - 1, Q // 2)]
+    # the last pixels of the flattened (image, row, column) index: the last, partly filled tile
+    tail = [(N - 1, int(k), P - 1, Q - 1 - int(d)) for d in range(min(Q, 40)) for k in rng.integers(0, K, 2)]
+    return np.concatenate([idx, np.array(ext, np.int64), np.array(tail, np.int64)]).astype(np.int32)
+
+
+def assert_conv_bar(ref, got, scale, what):
+    tol = 1e-5 * scale + 1e-4 * np.abs(ref)
+    err = np.abs(ref - got)
+    assert np.all(err <= tol), "%s: worst error %g (allowed %g)" % (what, err.max(), tol[np.argmax(err - tol)])
+
+
+def check_fullsize(hip, ora, model, x, seed):
+    from eddl_amd import models
+    rng = np.random.default_rng(seed + 1000)
+    models.init_he_normal(model, seed)
+    model.build(hip, fuse=False)
+    out_unfused = [o.numpy() for o in model.forward([x])]
+    checked = {"conv2d": 0, "dense": 0, "exact": 0}
+    for l in model.layers:
+        if l.kind == "input":
+            continue
+        ins = [model.output_of(p).numpy() for p in l.parents]
+        got = model.output_of(l).numpy()
+        assert np.all(np.isfinite(got)), l.name
+        if l.kind == "conv2d":
+            cd = l.attrs["cd"]
+            idx = sample_coords(rng, got.shape, NPTS)
+            ref = ora.conv2d_at(ins[0], l.params["K"], l.params["bias"] if cd.use_bias else None, (cd.sr, cd.sc), cd.padrt, cd.padcl, idx)
+            pts = got[idx[:, 0], idx[:, 1], idx[:, 2], idx[:, 3]]
+            assert_conv_bar(ref, pts, float(np.abs(got).max()), l.name)
+            checked["conv2d"] += 1
+        elif l.kind == "dense":
+            a = ins[0].reshape(-1, ins[0].shape[-1]).astype(np.float64)
+            cols = rng.integers(0, l.params["W"].shape[1], 64)
+            ref = a @ l.params["W"][:, cols].astype(np.float64)
+            if l.attrs["use_bias"]:
+                ref = ref + l.params["bias"][cols]
+            assert_conv_bar(ref.astype(np.float32), got.reshape(a.shape[0], -1)[:, cols], float(np.abs(got).max()), l.name)
+            checked["dense"] += 1
+        elif l.kind in EXACT:
+            ref = layer_oracle(ora, l, ins)
+            if l.kind == "maxpool2d":
+                ref, ix, iy = ref
+                aux = model.aux[id(l)]
+                gx, gy = aux["indX"].numpy(), aux["indY"].numpy()
+                assert np.array_equal(gx, ix) and np.array_equal(gy, iy), l.name
+                # property: the output is the input at the reported (row, column)
+                n, c = np.indices(got.shape)[:2]
+                assert np.array_equal(ins[0][n, c, gy.astype(np.int64), gx.astype(np.int64)], got), l.name
+            assert np.array_equal(ref.reshape(got.shape), got), l.name
+            checked["exact"] += 1
+        else:  # sigmoid / softmax: libm expf against the device's, to 1e-6 relative
+            ref = layer_oracle(ora, l, ins)
+            np.testing.assert_allclose(got, ref.reshape(got.shape), rtol=2e-6, atol=1e-7, err_msg=l.name)
+        del ins, got
+    model.build(hip, fuse=True)
+    out_fused = [o.numpy() for o in model.forward([x])]
+    for a, b in zip(out_unfused, out_fused):
+        assert np.array_equal(a, b), "fused plan differs from the layer-by-layer plan"
+    return checked
+
+
+def test_vgg16_batch32(hip, oracle):
+    from eddl_amd import models
+    m = models.vgg16(batch=32)
+    x = np.random.default_rng(3).uniform(0, 1, (32, 3, 224, 224)).astype(np.float32)
+    got = check_fullsize(hip, oracle, m, x, 3)
+    assert got["conv2d"] == 13 and got["dense"] == 3
+
+
+def test_block_64x64x56x56(hip, oracle):
+    from eddl_amd import models
+    m = models.conv_bn_relu_pool_block(batch=64, channels=64, size=56, filters=64)
+    x = np.random.default_rng(2).standard_normal((64, 64, 56, 56), dtype=np.float32)
+    check_fullsize(hip, oracle, m, x, 2)
+    # whole-tensor oracle for this one (14.8 GFLOP: seconds on the host cores)
+    conv = [l for l in m.layers if l.kind == "conv2d"][0]
+    cd = conv.attrs["cd"]
+    m.build(hip, fuse=False)
+    m.forward([x])
+    got = m.output_of(conv).numpy()
+    ref = oracle.conv2d(x, conv.params["K"], None, (cd.sr, cd.sc), cd.padrt, cd.padcl, cd.r, cd.c, algo="im2col")
+    assert_conv_bar(ref, got, float(np.abs(ref).max()), "block conv, every output")
+
+
+def test_resnet50_batch64(hip, oracle):
+    from eddl_amd import models
+    m = models.resnet50(batch=64)
+    x = np.random.default_rng(4).standard_normal((64, 3, 224, 224), dtype=np.float32)
+    got = check_fullsize(hip, oracle, m, x, 4)
+    assert got["conv2d"] == 53
+
+
+def test_unet_4x1x512x512(hip, oracle):
+    from eddl_amd import models
+    m = models.unet(batch=4)
+    x = np.random.default_rng(5).uniform(0, 1, (4, 1, 512, 512)).astype(np.float32)
+    got = check_fullsize(hip, oracle, m, x, 5)
+    assert got["conv2d"] == 23
+
+
+def test_conv_scaling_by_powers_of_two_is_exact_at_full_size(hip):
+    """conv(4x) == 4 conv(x) bit for bit (no overflow/underflow at these magnitudes), for the
+    dominant VGG-16 layer shape, and conv(x) is reproducible launch to launch."""
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((32, 256, 56, 56), dtype=np.float32)
+    w = (rng.standard_normal((256, 256, 3, 3)) * np.sqrt(2.0 / 2304)).astype(np.float32)
+    X, Wd = hip.array(x), hip.array(w)
+    O1, O2, O3 = hip.empty((32, 256, 56, 56)), hip.empty((32, 256, 56, 56)), hip.empty((32, 256, 56, 56))
+    hip.conv2D(X, Wd, None, O1, 1, 1, 1, 1)
+    hip.conv2D(X, Wd, None, O2, 1, 1, 1, 1)
+    X.copy_from(x * np.float32(4.0))
+    hip.conv2D(X, Wd, None, O3, 1, 1, 1, 1)
+    a, b, c = O1.numpy(), O2.numpy(), O3.numpy()
+    assert np.array_equal(a, b)
+    assert np.array_equal(a * np.float32(4.0), c)
