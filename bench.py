@@ -108,15 +108,21 @@ def cpu_baseline(workload, want_seconds=20.0):
         rng = np.random.default_rng(seed + 1000)
         shape = model.lin[0].out_shape
         x = rng.uniform(0, 1, shape).astype(np.float32) if dist == "uniform" else rng.standard_normal(shape, dtype=np.float32)
-        t0 = time.perf_counter()
-        net_oracle.forward(ora, model, [x], conv_algo="im2col")
-        dt = time.perf_counter() - t0
+        budget = want_seconds * (0.6 if hpc else 0.4)
+        times = []
+        while not times or (sum(times) < budget and len(times) < 200):
+            t0 = time.perf_counter()
+            net_oracle.forward(ora, model, [x], conv_algo="im2col")
+            times.append(time.perf_counter() - t0)
+        # the first forward pays for page faults of the lowered-matrix buffers: drop it when there are others
+        timed = times[1:] if len(times) > 1 else times
+        dt = sum(timed) / len(timed)
         result["value_" + label] = sample_batch / dt
-        result["seconds_" + label] = dt
-        if label == "hpc" and dt > want_seconds:
-            break  # keep the whole benchmark within minutes
+        result["seconds_" + label] = sum(times)
+        result["forwards_" + label] = len(times)
     result["value"] = result.get("value_hpc") or result.get("value_strict")
-    result["sample"] = ("one forward of the same model on a batch of %d (of %d), same seeds; im2col + single-threaded GEMM per image, "
+    result["sample"] = ("repeated forwards of the same model on a batch of %d (of %d), same seeds, about 20 s of CPU work in all "
+                        "(forwards_*/seconds_* give the counts; mean of all but the first); im2col + single-threaded GEMM per image, "
                         "OpenMP over the batch, %d threads; value = -O3 -march=x86-64-v3 -ffast-math build (the reference's HPC "
                         "flags), value_strict = -O2 without FMA contraction (the parity oracle)" % (sample_batch, full_batch, cores))
     return result

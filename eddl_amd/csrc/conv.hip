@@ -68,10 +68,11 @@ struct ConvParams {
     long long npix;
     int gm, gn;
     unsigned in_bytes, wp_bytes;  // sizes the input's and the packed filters' buffer descriptors cover
-    // Tiles [tile0, tile0 + gridDim.x / nslices) are computed by this launch.  With nslices > 1 a
-    // tile's K-steps are divided over nslices workgroups of slice_steps steps each, which write
-    // their raw accumulators to `partial`; conv_reduce_kernel adds the slices and finishes the tile.
-    int tile0, nslices, slice_steps;
+    // The first main_tiles workgroups of a launch compute one whole tile each (tiles 0..main_tiles-1).
+    // The workgroups after them divide the remaining tiles along K: nslices workgroups per tile, of
+    // slice_steps K-steps each, which write their raw accumulators to `partial`; conv_reduce_kernel
+    // adds the slices and finishes those tiles.
+    int main_tiles, nslices, slice_steps;
     float *partial;
 };
 
@@ -139,15 +140,29 @@ __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, int voffset,
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voffset, soffset, 0));
 }
 
-// workgroup id -> (channel tile, pixel tile, K slice); ids that share an XCD get consecutive tiles
-__device__ __forceinline__ void tile_of_block(const ConvParams &p, int &m_tile, int &n_tile, int &local_tile, int &slice) {
-    const unsigned total = gridDim.x, bid = blockIdx.x;
+// workgroup id -> (channel tile, pixel tile, K slice); ids that share an XCD get consecutive tiles.
+// Workgroups are dealt to the XCDs round-robin by id, so within each of the two groups of a launch
+// (whole tiles, then K slices) the ids that are congruent modulo the XCD count share an XCD.
+__device__ __forceinline__ void tile_of_block(const ConvParams &p, int &m_tile, int &n_tile, int &local_tile, int &slice, bool &split) {
+    unsigned total = (unsigned)p.main_tiles, bid = blockIdx.x;
+    split = bid >= total;
+    if (split) {
+        bid -= total;
+        total = gridDim.x - total;
+    }
     const unsigned q = total / EDDLHIP_NUM_XCD, r = total % EDDLHIP_NUM_XCD;
     const unsigned xcd = bid % EDDLHIP_NUM_XCD, slot = bid / EDDLHIP_NUM_XCD;
     const int vid = (int)((xcd < r ? xcd * (q + 1) : r * (q + 1) + (xcd - r) * q) + slot);
-    slice = vid % p.nslices;
-    local_tile = vid / p.nslices;
-    const int tile = p.tile0 + local_tile;
+    int tile;
+    if (split) {
+        slice = vid % p.nslices;
+        local_tile = vid / p.nslices;
+        tile = p.main_tiles + local_tile;
+    } else {
+        slice = 0;
+        local_tile = vid;
+        tile = vid;
+    }
     m_tile = tile % p.gm;
     n_tile = tile / p.gm;
 }
@@ -157,7 +172,7 @@ __device__ __forceinline__ void tile_of_block(const ConvParams &p, int &m_tile, 
 template <int TM, int TN>
 __device__ __forceinline__ void store_partial(const ConvParams &p, floatx16 (&acc)[TM][TN], int local_tile, int slice, int wave,
                                               int lane) {
-    const size_t tiles = gridDim.x / p.nslices;
+    const size_t tiles = (gridDim.x - (unsigned)p.main_tiles) / p.nslices;
     float *dst = p.partial + (((size_t)slice * tiles + local_tile) * 4 + wave) * (TM * TN * 16 * 64) + lane;
 #pragma unroll
     for (int tm = 0; tm < TM; tm++)
@@ -296,9 +311,10 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     int m_tile, n_tile, local_tile, slice;
-    tile_of_block(p, m_tile, n_tile, local_tile, slice);
-    const int step_lo = slice * p.slice_steps;
-    const int step_hi = min(step_lo + p.slice_steps, p.nsteps);
+    bool split;
+    tile_of_block(p, m_tile, n_tile, local_tile, slice, split);
+    const int step_lo = split ? slice * p.slice_steps : 0;
+    const int step_hi = split ? min(step_lo + p.slice_steps, p.nsteps) : p.nsteps;
     const int m0 = m_tile * BM;
     const long long n0 = (long long)n_tile * BN;
 
@@ -474,7 +490,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         __syncthreads();
     }
 
-    if (p.nslices > 1) {
+    if (split) {
         store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
     } else {
         float *epi = &As[0][0];  // the K loop ended with a barrier: the filter buffers are free
@@ -507,9 +523,10 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
     const int wm = wave / WN, wn = wave % WN;
     const int R = p.R, S = p.S, RS = R * S;
     int m_tile, n_tile, local_tile, slice;
-    tile_of_block(p, m_tile, n_tile, local_tile, slice);
-    const int step_lo = slice * p.slice_steps;
-    const int step_hi = min(step_lo + p.slice_steps, p.nsteps);
+    bool split;
+    tile_of_block(p, m_tile, n_tile, local_tile, slice, split);
+    const int step_lo = split ? slice * p.slice_steps : 0;
+    const int step_hi = split ? min(step_lo + p.slice_steps, p.nsteps) : p.nsteps;
     const int m0 = m_tile * BM;
     const long long n0 = (long long)n_tile * BN;
 
@@ -630,7 +647,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
         __syncthreads();
     }
 
-    if (p.nslices > 1) {
+    if (split) {
         store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
     } else {
         float *epi = &As[0][0];  // the K loop ended with a barrier: the filter buffers are free
@@ -641,42 +658,33 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
 }
 
 // ---------------------------------------------------------------- finishing kernel of K-split tiles
-// One workgroup per tile, same thread -> output mapping as the MFMA kernels: adds the slices
-// in increasing K order (a fixed order: results do not depend on scheduling), then applies the
-// fused tail and stores.
+// One wavefront per 32x32 block of a divided tile (4 wavefronts x TM x TN blocks per tile), same
+// lane -> output mapping as the MFMA kernels: adds the slices in increasing K order (a fixed
+// order: results do not depend on scheduling), then applies the fused tail and stores.
 template <int WM, int WN, int TM, int TN>
-__global__ __launch_bounds__(256) void conv_reduce_kernel(const ConvParams p) {
-    constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;
-    const int local_tile = blockIdx.x;
-    const int tile = p.tile0 + local_tile;
-    const int m0 = (tile % p.gm) * BM;
-    const long long n0 = (long long)(tile / p.gm) * BN;
-    const size_t tiles = gridDim.x;
-    floatx16 acc[TM][TN];
-#pragma unroll
-    for (int tm = 0; tm < TM; tm++)
-#pragma unroll
-        for (int tn = 0; tn < TN; tn++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.0f;
+__global__ __launch_bounds__(64) void conv_reduce_kernel(const ConvParams p) {
+    constexpr int BM = WM * TM * 32, BN = WN * TN * 32, UNITS = 4 * TM * TN;
+    const int lane = threadIdx.x;
+    const int unit = blockIdx.x % UNITS, local_tile = blockIdx.x / UNITS;
+    const int wave = unit / (TM * TN), blk = unit % (TM * TN);
+    const int wm = wave / WN, wn = wave % WN, tm = blk / TN, tn = blk % TN;
+    const int tile = p.main_tiles + local_tile;
+    const int m0 = (tile % p.gm) * BM + (wm * TM + tm) * 32;
+    const long long n0 = (long long)(tile / p.gm) * BN + (wn * TN + tn) * 32;
+    const size_t tiles = gridDim.x / UNITS;
+    floatx16 acc[1][1];
     for (int sl = 0; sl < p.nslices; sl++) {
-        const float *src = p.partial + (((size_t)sl * tiles + local_tile) * 4 + wave) * (TM * TN * 16 * 64) + lane;
+        const float *src = p.partial + ((((size_t)sl * tiles + local_tile) * 4 + wave) * (TM * TN) + blk) * (16 * 64) + lane;
 #pragma unroll
-        for (int tm = 0; tm < TM; tm++)
-#pragma unroll
-            for (int tn = 0; tn < TN; tn++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const float x = src[((tm * TN + tn) * 16 + v) * 64];
-                    acc[tm][tn][v] = sl == 0 ? x : __fadd_rn(acc[tm][tn][v], x);
-                }
+        for (int v = 0; v < 16; v++) {
+            const float x = src[v * 64];
+            acc[0][0][v] = sl == 0 ? x : __fadd_rn(acc[0][0][v], x);
+        }
     }
-    __shared__ float epi[5 * BM];
-    stage_channel_constants<BM>(p, epi, m0, tid);
+    __shared__ float epi[5 * 32];
+    stage_channel_constants<32>(p, epi, m0, lane);
     __syncthreads();
-    store_tile<TM, TN, BM>(p, acc, epi, m0, wm * TM * 32, (int)n0 + wn * TN * 32, lane);
+    store_tile<1, 1, 32>(p, acc, epi, m0, 0, (int)n0, lane);
 }
 
 // ---------------------------------------------------------------- scalar direct kernel
@@ -772,16 +780,18 @@ const Variant k2x2[2][4] = {
     {TAP(2, 2, 2, 2, 2, 2, 4, true), TAP(1, 4, 2, 1, 2, 2, 4, true), TAP(2, 2, 1, 1, 2, 2, 4, true), TAP(1, 4, 1, 1, 2, 2, 4, true)}};
 const Variant kgen[4] = {GEN(2, 2, 2, 2), GEN(1, 4, 2, 1), GEN(2, 2, 1, 1), GEN(1, 4, 1, 1)};
 
-// Launch plan: tile shape and, for the tiles of the last (partial) round of workgroups, the
-// number of K slices.  A grid that is not a whole number of device-filling rounds leaves its
-// last round mostly idle (28x28x512 at batch 32: 784 tiles of 128x128 for 768 resident
-// workgroups).  Those "leftover" tiles can be divided along K over several workgroups each so
-// that they, too, occupy the whole device; conv_reduce_kernel then adds the slices in a fixed
-// order.  The plan minimises a simple time estimate over the four tile shapes and 1..16 slices:
+// Launch plan: tile shape and, for the tiles that do not divide evenly over the CUs, the number
+// of K slices.  The MFMA pipe of a CU is shared by its resident workgroups, so a launch takes as
+// long as the busiest CU's share of the tiles: 784 tiles of 128x128 (28x28x512 at batch 32) on 256
+// CUs cost four tile times where the average CU has 3.06 tiles.  The tiles beyond a whole number
+// per CU ("leftover") can be divided along K over several workgroups each, so that they, too,
+// spread over the whole device; conv_reduce_kernel then adds the slices in a fixed order.  The
+// whole tiles come first in the grid and the slices after them, in ONE launch, so the slices fill
+// CUs as whole tiles retire.  The plan minimises a simple time estimate over the four tile shapes
+// and 1..16 slices:
 //   a K-step of a tile costs its flops over (CU peak x tile efficiency); a workgroup costs its
-//   K-steps plus a fixed prologue/epilogue; a full round keeps `occupancy` workgroups on every
-//   CU; the last round costs ceil(workgroups / CUs) workgroup times; divided tiles add the
-//   traffic of their partial sums and two more launches.
+//   K-steps plus a fixed prologue/epilogue; a CU with few resident workgroups hides less latency;
+//   divided tiles add the traffic of their partial sums and one more launch.
 struct Plan {
     int tile, nsteps, nslices, slice_steps;
     long long tiles, leftover;
@@ -804,23 +814,20 @@ Plan plan_conv(const Variant *family, int Kf, int C, int RS, long long npix, int
         const int bk = v.cpb ? v.cpb * RS : 16;
         const int nsteps = v.cpb ? (C + v.cpb - 1) / v.cpb : (C * RS + 15) / 16;
         const long long tiles = (long long)((Kf + v.bm - 1) / v.bm) * ((npix + v.bn - 1) / v.bn);
-        const long long slots = (long long)num_cu * v.occupancy;
-        const long long full = tiles / slots, left = tiles % slots;
+        const long long full = tiles / num_cu, left = tiles % num_cu;
         const double step_us = 2.0 * v.bm * v.bn * bk / (cu_flops_per_us * kEff[t]);
-        const double base = (double)full * v.occupancy * (nsteps * step_us + kOverheadUs[t]) / crowd(v.occupancy);
-        const int smax = allow_split ? (nsteps / 4 < 16 ? nsteps / 4 : 16) : 1;
+        const double tile_us = nsteps * step_us + kOverheadUs[t];
+        const int smax = (allow_split && left > 0) ? (nsteps / 4 < 16 ? nsteps / 4 : 16) : 1;
         for (int want = 1; want <= (smax < 1 ? 1 : smax); want++) {
             const int ss = (nsteps + want - 1) / want;
             const int sl = (nsteps + ss - 1) / ss;
             if (sl != want && want != 1) continue;  // same plan as a smaller `want`
-            double last = 0.0;
-            if (left > 0) {
-                const long long wgs = left * sl;
-                const long long per_cu = (wgs + num_cu - 1) / num_cu;
-                last = (double)per_cu * (ss * step_us + kOverheadUs[t]) / crowd(per_cu < v.occupancy ? per_cu : v.occupancy);
-                if (sl > 1) last += (double)wgs * v.bm * v.bn * 8.0 / bytes_per_us + 6.0;
-            }
-            const double cost = base + last;
+            const long long wgs = left * sl;
+            const long long per_cu = (wgs + num_cu - 1) / num_cu;
+            const long long resident = full + per_cu;
+            double cost = ((double)full * tile_us + (double)per_cu * (ss * step_us + kOverheadUs[t])) /
+                          crowd(resident < v.occupancy ? resident : v.occupancy);
+            if (sl > 1) cost += (double)wgs * v.bm * v.bn * 8.0 / bytes_per_us + 6.0;
             if (best.cost_us < 0 || cost < best.cost_us) {
                 best.tile = t;
                 best.nsteps = nsteps;
@@ -835,15 +842,15 @@ Plan plan_conv(const Variant *family, int Kf, int C, int RS, long long npix, int
     return best;
 }
 
-// A plan with a given tile shape and slice count (every tile of the last round is divided; with
-// fewer tiles than one round that is every tile).
+// A plan with a given tile shape and slice count (every leftover tile is divided; with fewer
+// tiles than CUs that is every tile).
 Plan forced_plan(const Variant *family, int tile, int slices, int Kf, int C, int RS, long long npix, int num_cu) {
     const Variant &v = family[tile];
     Plan pl;
     pl.tile = tile;
     pl.nsteps = v.cpb ? (C + v.cpb - 1) / v.cpb : (C * RS + 15) / 16;
     pl.tiles = (long long)((Kf + v.bm - 1) / v.bm) * ((npix + v.bn - 1) / v.bn);
-    pl.leftover = pl.tiles % ((long long)num_cu * v.occupancy);
+    pl.leftover = pl.tiles % num_cu;
     int want = slices < 1 ? 1 : (slices > pl.nsteps ? pl.nsteps : slices);
     pl.slice_steps = (pl.nsteps + want - 1) / want;
     pl.nslices = (pl.nsteps + pl.slice_steps - 1) / pl.slice_steps;
@@ -929,7 +936,7 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     p.nsteps = 0;
     p.Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
     p.in_bytes = p.wp_bytes = 0;
-    p.tile0 = 0; p.nslices = 1; p.slice_steps = 0; p.partial = nullptr;
+    p.main_tiles = 0; p.nslices = 1; p.slice_steps = 0; p.partial = nullptr;
 
     if (g_algo == 2) {
         size_t total = (size_t)p.npix * Kf;
@@ -999,24 +1006,15 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
         const long long tiles = gn * gm;
         const long long split_tiles = (nb == chunk_imgs) ? leftover : 0;  // a short last chunk runs unsplit
         const long long main_tiles = tiles - split_tiles;
-        if (main_tiles > 0) {
-            q.tile0 = 0;
-            q.nslices = 1;
-            q.slice_steps = p.nsteps;
-            EH_TRY(prof_begin(st));
-            hipLaunchKernelGGL(v->kernel, dim3((unsigned)main_tiles), dim3(256), 0, st, q);
-            EH_CHECK_LAUNCH();
-            EH_TRY(prof_end(st));
-        }
+        q.main_tiles = (int)main_tiles;
+        q.nslices = split_tiles > 0 ? nslices : 1;
+        q.slice_steps = split_tiles > 0 ? slice_steps : p.nsteps;
+        EH_TRY(prof_begin(st));
+        hipLaunchKernelGGL(v->kernel, dim3((unsigned)(main_tiles + split_tiles * q.nslices)), dim3(256), 0, st, q);
+        EH_CHECK_LAUNCH();
+        EH_TRY(prof_end(st));
         if (split_tiles > 0) {
-            q.tile0 = (int)main_tiles;
-            q.nslices = nslices;
-            q.slice_steps = slice_steps;
-            EH_TRY(prof_begin(st));
-            hipLaunchKernelGGL(v->kernel, dim3((unsigned)(split_tiles * nslices)), dim3(256), 0, st, q);
-            EH_CHECK_LAUNCH();
-            EH_TRY(prof_end(st));
-            hipLaunchKernelGGL(v->reduce, dim3((unsigned)split_tiles), dim3(256), 0, st, q);
+            hipLaunchKernelGGL(v->reduce, dim3((unsigned)(split_tiles * (v->bm / 32) * (v->bn / 32))), dim3(64), 0, st, q);
             EH_CHECK_LAUNCH();
         }
     }
