@@ -137,6 +137,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-op table to stderr")
     ap.add_argument("--conv-algo", default="auto", choices=["auto", "mfma_staged", "mfma_lds"], help="input gather of the convolution kernels")
+    ap.add_argument("--no-device-probe", action="store_true",
+                    help="skip the pure-MFMA probe of the device's sustained fp32 matrix rate (keeps kernel traces to the workload)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="after the timed region run one ReLU over 2^26 floats (reads 256 MiB, writes 256 MiB): the plain copy "
                          "kernel of known size that scales FETCH_SIZE / WRITE_SIZE counter readings")
@@ -208,6 +210,16 @@ def main():
                 "kernel": dom_name, "launches_per_step": dom_launches, "layers": len(dom),
                 "flops_per_launch": dom_flops / max(dom_launches, 1), "avg_launch_ms": dom_ms / max(dom_launches, 1),
                 "algorithmic_bytes_per_launch": sum(r["bytes"] for r in dom) / max(dom_launches, 1)}
+
+    # what the matrix pipe sustains on this device with nothing else running (constant operands, then
+    # operands that change every instruction): the published peak assumes the top clock throughout
+    if not args.no_device_probe:
+        const_mean, const_best, _ = hip.probe_mfma_f32(vary_operands=False, launches=30)
+        vary_mean, vary_best, vary_worst = hip.probe_mfma_f32(vary_operands=True, launches=60)
+        roofline["device_probe"] = {"unit": "TFLOP/s", "pure_mfma_constant_operands": const_mean,
+                                    "pure_mfma_varying_operands_mean": vary_mean, "varying_best_launch": vary_best,
+                                    "varying_worst_launch": vary_worst,
+                                    "frac_of_varying_mean": achieved / vary_mean if vary_mean > 0 else None}
 
     conv_ms = sum(r["ms"] for r in conv_rows)
     conv_flops = sum(r["flops"] for r in conv_rows)

@@ -122,6 +122,13 @@ class Backend:
     def event(self):
         return Event(self)
 
+    def probe_mfma_f32(self, vary_operands=True, launches=40):
+        """Sustained fp32 MFMA rate of the device with nothing else running: (mean, best launch, worst launch) TFLOP/s."""
+        mean, best, worst = ctypes.c_float(), ctypes.c_float(), ctypes.c_float()
+        self._check(self.lib.eddlhip_probe_mfma_f32(self.dev, int(vary_operands), launches, ctypes.byref(mean), ctypes.byref(best),
+                                                    ctypes.byref(worst)))
+        return mean.value, best.value, worst.value
+
     def empty(self, shape):
         return DeviceTensor(self, shape)
 

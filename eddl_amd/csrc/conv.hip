@@ -453,6 +453,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         for (int tm = 0; tm < TM; tm++) a[0][tm] = a_cur[a_off + tm * 32];
 #pragma unroll
         for (int tn = 0; tn < TN; tn++) b[0][tn] = b_cur[b_off + tn * 32];
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // the two reads of pair 0
 #pragma unroll
         for (int ks = 0; ks < BK / 2; ks++) {
             const int cur = ks & 1, nxt = cur ^ 1;
@@ -467,6 +468,10 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
 #pragma unroll
                 for (int tn = 0; tn < TN; tn++)
                     acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
+            // issue order: the LDS reads of pair ks+1 (two instructions: the TM and the TN operands
+            // each pair up into one two-address read, or are one read), then the MFMAs of pair ks
+            if (ks + 1 < BK / 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
         }
         if (more) {
             store_a(a_nxt);
