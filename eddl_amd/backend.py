@@ -181,6 +181,14 @@ class Backend:
                                                 padcl, O.shape[2], O.shape[3], _ptr(g), _ptr(b), _ptr(mean), _ptr(var), eps,
                                                 _ptr(residual), int(relu)))
 
+    def cache_conv_filters(self, K):
+        """Keep the kernels' repacked copy of filter tensor ``K`` (fixed between calls) in the library."""
+        Kf, C, R, S = K.shape
+        self._check(self.lib.eddlhip_conv2d_cache_filters(self.dev, K.ptr, Kf, C, R, S))
+
+    def uncache_conv_filters(self, K=None):
+        self._check(self.lib.eddlhip_conv2d_uncache_filters(self.dev, _ptr(K)))
+
     def batchnorm_inference(self, x, y, opa, gmean, gvar, g, b, variance, eps):
         N, C = x.shape[0], x.shape[1]
         rc = x.size // (N * C) if N * C else 1

@@ -37,6 +37,7 @@
 // XCD's L2.
 #include <stdio.h>
 
+#include <mutex>
 #include <utility>
 #include <vector>
 
@@ -864,9 +865,121 @@ Plan forced_plan(const Variant *family, int tile, int slices, int Kf, int C, int
     return pl;
 }
 
+
+// ---------------------------------------------------------------- cache of repacked filters
+// A caller that keeps its filters fixed between calls (inference) registers them once
+// (eddlhip_conv2d_cache_filters); eddlhip_conv2d_fwd then finds the repacked copy by the filter
+// pointer and skips pack_filters_kernel.  Rows are in OIHW tap order for every kernel variant and
+// only the zero padding behind them differs, so one copy padded for the largest K-step serves all.
+struct CachedFilters {
+    const float *K;
+    int Kf, C, R, S, rows, Mp;
+    float *Wp;
+    bool stale;  // K was written through this library since the last repack
+};
+std::mutex g_cache_mutex;
+std::vector<CachedFilters> g_cache[EDDLHIP_MAX_DEVICES];
+
+int cache_rows(int C, int R, int S) {
+    const int RS = R * S, crs = C * RS;
+    int rows = (crs + 15) / 16 * 16;  // the 16-tap kernel
+    for (int cpb : {2, 4, 16}) {
+        const int r = (C + cpb - 1) / cpb * cpb * RS;
+        if (r > rows) rows = r;
+    }
+    return rows;
+}
+
+int repack(int dev, CachedFilters &e) {
+    hipLaunchKernelGGL(pack_filters_kernel, dim3((e.rows + 31) / 32, e.Mp / 32), dim3(256), 0, state(dev).stream, e.K, e.Wp, e.Kf,
+                       e.C * e.R * e.S, e.Mp, e.rows);
+    EH_CHECK_LAUNCH();
+    e.stale = false;
+    return 0;
+}
+
 }  // namespace
 
+namespace eddlhip {
+
+void conv_filters_written(int dev, const void *dst, size_t bytes) {
+    if (dev < 0 || dev >= EDDLHIP_MAX_DEVICES) return;
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    const char *lo = (const char *)dst, *hi = lo + bytes;
+    for (CachedFilters &e : g_cache[dev]) {
+        const char *klo = (const char *)e.K, *khi = klo + (size_t)e.Kf * e.C * e.R * e.S * sizeof(float);
+        if (lo < khi && klo < hi) e.stale = true;
+    }
+}
+
+void conv_filters_released(int dev, const void *base, size_t bytes) {
+    if (dev < 0 || dev >= EDDLHIP_MAX_DEVICES) return;
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    std::vector<CachedFilters> &c = g_cache[dev];
+    const char *lo = (const char *)base, *hi = lo + bytes;
+    for (size_t i = 0; i < c.size();) {
+        if ((const char *)c[i].K >= lo && (const char *)c[i].K < hi) {
+            // kernels still reading the packed copy finish first
+            (void)hipStreamSynchronize(state(dev).stream);
+            (void)hipFree(c[i].Wp);
+            c[i] = c.back();
+            c.pop_back();
+        } else {
+            i++;
+        }
+    }
+}
+
+}  // namespace eddlhip
+
 extern "C" {
+
+int eddlhip_conv2d_cache_filters(int dev, const float *K, int Kf, int C, int R, int S) {
+    EH_REQUIRE(K != nullptr && Kf > 0 && C > 0 && R > 0 && S > 0, "conv2d_cache_filters: bad filter tensor %dx%dx%dx%d", Kf, C, R, S);
+    EH_REQUIRE((long long)C * R * S <= (1LL << 24), "conv2d_cache_filters: filter too large");
+    EH_TRY(use_device(dev));
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    for (CachedFilters &e : g_cache[dev]) {
+        if (e.K == K) {
+            EH_REQUIRE(e.Kf == Kf && e.C == C && e.R == R && e.S == S,
+                       "conv2d_cache_filters: pointer already registered with shape %dx%dx%dx%d", e.Kf, e.C, e.R, e.S);
+            return repack(dev, e);
+        }
+    }
+    CachedFilters e;
+    e.K = K; e.Kf = Kf; e.C = C; e.R = R; e.S = S;
+    e.rows = cache_rows(C, R, S);
+    e.Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
+    e.Wp = nullptr;
+    e.stale = true;
+    EH_TRY_HIP(hipMalloc((void **)&e.Wp, (size_t)e.rows * e.Mp * sizeof(float)));
+    int rc = repack(dev, e);
+    if (rc != 0) {
+        (void)hipFree(e.Wp);
+        return rc;
+    }
+    g_cache[dev].push_back(e);
+    return 0;
+}
+
+int eddlhip_conv2d_uncache_filters(int dev, const float *K) {
+    EH_TRY(use_device(dev));
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    std::vector<CachedFilters> &c = g_cache[dev];
+    bool synced = false;
+    for (size_t i = 0; i < c.size();) {
+        if (K == nullptr || c[i].K == K) {
+            if (!synced) EH_TRY_HIP(hipStreamSynchronize(state(dev).stream));
+            synced = true;
+            EH_TRY_HIP(hipFree(c[i].Wp));
+            c[i] = c.back();
+            c.pop_back();
+        } else {
+            i++;
+        }
+    }
+    return 0;
+}
 
 int eddlhip_conv2d_force_plan(int tile, int slices) {
     EH_REQUIRE(tile >= -1 && tile <= 3, "conv2d_force_plan: tile is -1 (automatic) or 0..3");
@@ -984,17 +1097,31 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     const int nslices = plan.nslices, slice_steps = plan.slice_steps;
     const size_t tile_floats = (size_t)v->bm * v->bn;
 
-    // ---- workspace: packed filters, then the partial tiles of the K-split launch
+    // ---- packed filters (the registered copy, or a repack into the workspace), then the partial
+    // tiles of the K-split launch
     const int rows = p.nsteps * bk;
-    const size_t wp_bytes = ((size_t)rows * p.Mp * sizeof(float) + 255) & ~(size_t)255;
+    const float *cached = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_cache_mutex);
+        for (CachedFilters &e : g_cache[dev]) {
+            if (e.K == K && e.Kf == Kf && e.C == C && e.R == R && e.S == S && rows <= e.rows) {
+                if (e.stale) EH_TRY(repack(dev, e));
+                cached = e.Wp;
+                break;
+            }
+        }
+    }
+    const size_t wp_bytes = cached ? 0 : (((size_t)rows * p.Mp * sizeof(float) + 255) & ~(size_t)255);
     const size_t partial_bytes = (size_t)nslices * leftover * tile_floats * sizeof(float);
     void *ws = nullptr;
     EH_TRY(get_workspace(dev, wp_bytes + partial_bytes, &ws));
-    p.Wp = (const float *)ws;
+    p.Wp = cached ? cached : (const float *)ws;
     p.wp_bytes = (unsigned)((size_t)rows * p.Mp * sizeof(float));
     p.partial = (float *)((char *)ws + wp_bytes);
-    hipLaunchKernelGGL(pack_filters_kernel, dim3((rows + 31) / 32, p.Mp / 32), dim3(256), 0, st, K, (float *)ws, Kf, p.CRS, p.Mp, rows);
-    EH_CHECK_LAUNCH();
+    if (!cached) {
+        hipLaunchKernelGGL(pack_filters_kernel, dim3((rows + 31) / 32, p.Mp / 32), dim3(256), 0, st, K, (float *)ws, Kf, p.CRS, p.Mp, rows);
+        EH_CHECK_LAUNCH();
+    }
 
     for (long long b0 = 0; b0 < N; b0 += chunk_imgs) {
         const int nb = (int)((N - b0 < chunk_imgs) ? N - b0 : chunk_imgs);

@@ -219,6 +219,7 @@ int eddlhip_fill(int dev, float *A, size_t n, float v) {
     if (n == 0) return 0;
     EH_REQUIRE(A != nullptr, "fill: NULL tensor");
     EH_TRY(use_device(dev));
+    conv_filters_written(dev, A, n * sizeof(float));
     hipLaunchKernelGGL(fill_kernel, dim3(eh_blocks(n / 4 + 1, TPB, 65536)), dim3(TPB), 0, state(dev).stream, A, n, v,
                        (int)aligned16(A));
     EH_CHECK_LAUNCH();
@@ -285,6 +286,7 @@ int eddlhip_add(int dev, float scA, const float *A, float scB, const float *B, f
     if (n == 0) return 0;
     EH_REQUIRE(A && B && C, "add: NULL tensor");
     EH_TRY(use_device(dev));
+    conv_filters_written(dev, C, n * sizeof(float));
     int vec = aligned16(A) && aligned16(B) && aligned16(C);
     hipLaunchKernelGGL(add_kernel, dim3(eh_blocks(n / 4 + 1, TPB, 65536)), dim3(TPB), 0, state(dev).stream, scA, A, scB, B, C,
                        incC, n, vec);
@@ -296,6 +298,7 @@ int eddlhip_inc(int dev, const float *A, float *B, size_t n) {
     if (n == 0) return 0;
     EH_REQUIRE(A && B, "inc: NULL tensor");
     EH_TRY(use_device(dev));
+    conv_filters_written(dev, B, n * sizeof(float));
     int vec = aligned16(A) && aligned16(B);
     hipLaunchKernelGGL(inc_kernel, dim3(eh_blocks(n / 4 + 1, TPB, 65536)), dim3(TPB), 0, state(dev).stream, A, B, n, vec);
     EH_CHECK_LAUNCH();

@@ -89,6 +89,7 @@ int eddlhip_shutdown(int dev) {
     if (!s.inited) return 0;
     EH_TRY_HIP(hipSetDevice(dev));
     EH_TRY_HIP(hipDeviceSynchronize());
+    EH_TRY(eddlhip_conv2d_uncache_filters(dev, nullptr));
     if (s.workspace) EH_TRY_HIP(hipFree(s.workspace));
     if (s.flag) EH_TRY_HIP(hipFree(s.flag));
     s = DeviceState();
@@ -133,6 +134,10 @@ int eddlhip_malloc(int dev, size_t bytes, void **dev_ptr) {
 int eddlhip_free(int dev, void *dev_ptr) {
     if (!dev_ptr) return 0;
     EH_TRY(use_device(dev));
+    void *base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(&base, &size, dev_ptr) == hipSuccess) conv_filters_released(dev, base, size);
+    else (void)hipGetLastError();
     EH_TRY_HIP(hipFree(dev_ptr));
     return 0;
 }
@@ -143,6 +148,7 @@ int eddlhip_memcpy_h2d(int dev, void *dev_dst, const void *host_src, size_t byte
     if (bytes == 0) return 0;
     EH_REQUIRE(dev_dst && host_src, "NULL pointer in h2d copy");
     EH_TRY(use_device(dev));
+    conv_filters_written(dev, dev_dst, bytes);
     EH_TRY_HIP(hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice, state(dev).stream));
     EH_TRY_HIP(hipStreamSynchronize(state(dev).stream));
     return 0;
@@ -161,6 +167,7 @@ int eddlhip_memcpy_d2d(int dev, void *dev_dst, const void *dev_src, size_t bytes
     if (bytes == 0) return 0;
     EH_REQUIRE(dev_dst && dev_src, "NULL pointer in d2d copy");
     EH_TRY(use_device(dev));
+    conv_filters_written(dev, dev_dst, bytes);
     EH_TRY_HIP(hipMemcpyAsync(dev_dst, dev_src, bytes, hipMemcpyDeviceToDevice, state(dev).stream));
     return 0;
 }

@@ -254,9 +254,12 @@ class Net:
                 self.dparams[id(l)][key].copy_from(v)
 
     # ---- build
-    def build(self, backend, fuse=True):
+    def build(self, backend, fuse=True, cache_filters=True):
+        """``cache_filters``: the plan is an inference plan whose parameters change only through
+        ``set_parameters``, so the library may keep each convolution's repacked filters between calls."""
         self.backend = hip = backend
         self.fused = fuse
+        self.cache_filters = cache_filters
         self.dparams = {id(l): {k: hip.empty(v.shape) for k, v in l.params.items()} for l in self.layers}
         self._push_parameters()
         self.out = {}   # id(layer) -> DeviceTensor holding its output (absent for layers folded into a fused op)
@@ -282,6 +285,10 @@ class Net:
         for o in self.lout:
             if id(o) not in self.out:
                 msg("output layer %s was fused away" % o.name, "Net::build")
+        if cache_filters:
+            for l in self.layers:
+                if l.kind == "conv2d":
+                    hip.cache_conv_filters(self.dparams[id(l)]["K"])
         return self
 
     def _emit_conv(self, l, fuse, absorbed, sole_child):
@@ -411,7 +418,7 @@ class Net:
             for key in ("cd", "pd"):
                 if key in l.attrs:
                     l.attrs[key].resize(batch)
-        return self.build(self.backend, self.fused)
+        return self.build(self.backend, self.fused, self.cache_filters)
 
     def forward(self, xs):
         """``xs``: one array (or DeviceTensor) per input layer.  Returns the output DeviceTensors;

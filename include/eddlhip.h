@@ -111,8 +111,24 @@ const char *eddlhip_conv2d_last_kernel(void);
 
 /* Overrides the launch planner of the MFMA kernels (tuning and tests): tile = 0 (128x128 outputs per
  * workgroup), 1 (64x128), 2 (64x64), 3 (32x128) or -1 to give the choice back to the planner;
- * slices = number of K slices the tiles of the last partial round are divided into (1 = none). */
+ * slices = number of K slices the tiles left over after a whole number per CU are divided into
+ * (1 = none). */
 int eddlhip_conv2d_force_plan(int tile, int slices);
+
+/* Filters that stay fixed between calls (inference).  Every eddlhip_conv2d_fwd first repacks its
+ * filters into the kernels' tap-major layout (3-10 us per layer).  After
+ * eddlhip_conv2d_cache_filters(dev, K, ...) the library keeps that repacked copy in device memory
+ * of its own, and calls that pass the same K pointer and shape use it instead.  The caller
+ * promises that K's contents change only through this library: eddlhip_memcpy_h2d/_d2d, _fill,
+ * _add and _inc into a registered tensor mark its copy stale (it is repacked on the next use);
+ * a kernel of the caller's own that writes K must be followed by another
+ * eddlhip_conv2d_cache_filters call.  eddlhip_free of the tensor, eddlhip_conv2d_uncache_filters
+ * (K == NULL: every tensor of the device) and eddlhip_shutdown drop the copy.
+ * No counterpart in the reference, whose gpu_conv2D reads OIHW filters on every call
+ * (src/hardware/gpu/nn/gpu_conv.cu:159-233); the C++ host layer does not register anything, so
+ * training-style callers that update filters between calls see the reference's behaviour. */
+int eddlhip_conv2d_cache_filters(int dev, const float *K, int Kf, int C, int R, int S);
+int eddlhip_conv2d_uncache_filters(int dev, const float *K);
 
 /* Measurement hook (no counterpart in the reference).  eddlhip_conv2d_profile(1) starts a
  * collection: from then on every launch of a convolution kernel made by eddlhip_conv2d_fwd

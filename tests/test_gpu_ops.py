@@ -396,3 +396,48 @@ def test_dense_sigmoid_softmax_within_tolerance(hip, oracle):
         B = hip.empty(shape)
         hip.full_softmax(hip.array(x), B, axis)
         np.testing.assert_allclose(B.numpy(), oracle.softmax(x, axis), rtol=2e-6, atol=1e-8)
+
+
+def test_conv2d_cached_filters_follow_every_write(hip, oracle):
+    """A registered filter tensor gives the results of an unregistered one, bit for bit, before and
+    after its contents are replaced through the library (copy, fill, add, inc), and a freed
+    tensor's entry does not outlive it."""
+    rng = np.random.default_rng(415)
+    N, C, H, W, Kf = 3, 24, 19, 17, 40
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    X = hip.array(x)
+
+    def conv(Kd):
+        O = hip.empty((N, Kf, H, W))
+        hip.conv2D(X, Kd, None, O, 1, 1, 1, 1)
+        return O.numpy()
+
+    w1 = rng.standard_normal((Kf, C, 3, 3), dtype=np.float32)
+    w2 = rng.standard_normal((Kf, C, 3, 3), dtype=np.float32)
+    plain1, plain2 = conv(hip.array(w1)), conv(hip.array(w2))
+    assert not np.array_equal(plain1, plain2)
+    K = hip.array(w1)
+    hip.cache_conv_filters(K)
+    assert np.array_equal(conv(K), plain1)
+    assert np.array_equal(conv(K), plain1)
+    K.copy_from(w2)                                   # host -> device copy into the registered tensor
+    assert np.array_equal(conv(K), plain2)
+    hip.fill_(K, 0.0)
+    assert not conv(K).any()
+    hip.inc(hip.array(w1), K)                         # K += w1
+    assert np.array_equal(conv(K), plain1)
+    W2 = hip.array(w2)
+    hip.add(1.0, W2, 0.0, W2, K)                      # K = w2 (+ 0*w2)
+    assert np.array_equal(conv(K), plain2)
+    with pytest.raises(Exception):
+        hip._check(hip.lib.eddlhip_conv2d_cache_filters(hip.dev, K.ptr, Kf + 1, C, 3, 3))
+    hip.uncache_conv_filters(K)
+    assert np.array_equal(conv(K), plain2)
+    # a registered tensor that is freed: the next tensor at that address starts unregistered
+    hip.cache_conv_filters(K)
+    del K
+    for _ in range(4):
+        K2 = hip.array(w1)
+        assert np.array_equal(conv(K2), plain1)
+        del K2
+    hip.uncache_conv_filters(None)
