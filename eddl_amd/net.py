@@ -218,21 +218,57 @@ class Net:
         self.backend = None
 
     def _topological(self):
-        order, seen = [], set()
-
-        def visit(l):
-            if id(l) in seen:
-                return
-            seen.add(id(l))
-            for p in l.parents:
-                visit(p)
-            order.append(l)
-
-        for o in self.lout:
-            visit(o)
+        """The reference's layer order, which is also the order of a saved parameter file:
+        layers collected by a depth-first walk along the children from every input (stopping at
+        output layers), then the not yet seen ancestors of the outputs (Net::Net, walk, walk_back:
+        src/net/net.cpp:77-114,231-258), then sorted by repeatedly taking the FIRST layer of that
+        list whose parents have all been taken (Net::fts, src/net/net_build.cpp:34-70)."""
+        collected, seen = [], set()
+        outs = {id(o) for o in self.lout}
+        stack = [[l, None] for l in reversed(self.lin)]
+        while stack:  # iterative pre-order walk, children in creation order
+            l, it = stack[-1]
+            if it is None:
+                if id(l) in seen:
+                    stack.pop()
+                    continue
+                seen.add(id(l))
+                collected.append(l)
+                if id(l) in outs:
+                    stack.pop()
+                    continue
+                stack[-1][1] = it = iter(l.children)
+            nxt = next(it, None)
+            if nxt is None:
+                stack.pop()
+            else:
+                stack.append([nxt, None])
+        back, seen_back = [], set()
+        stack = list(reversed(self.lout))
+        while stack:  # pre-order walk along the parents
+            l = stack.pop()
+            if id(l) in seen_back:
+                continue
+            seen_back.add(id(l))
+            back.append(l)
+            stack.extend(reversed(l.parents))
+        collected += [l for l in back if id(l) not in seen]
+        index = {id(l): i for i, l in enumerate(collected)}
         for i in self.lin:
-            if id(i) not in seen:
+            if id(i) not in seen_back:
                 msg("input layer %s does not reach an output" % i.name, "Net::build")
+        pending = [sum(1 for p in l.parents if id(p) in index) for l in collected]
+        taken = [False] * len(collected)
+        order = []
+        for _ in collected:
+            j = next((k for k in range(len(collected)) if pending[k] == 0 and not taken[k]), None)
+            if j is None:
+                msg("error recurrent net", "Net.fts")
+            taken[j] = True
+            order.append(collected[j])
+            for c in collected[j].children:
+                if id(c) in index:
+                    pending[index[id(c)]] -= 1
         return order
 
     # ---- parameters (host side), in the reference's per-layer order
@@ -245,6 +281,49 @@ class Net:
                 if tuple(v.shape) != l.params[key].shape:
                     msg("parameter %s of %s has shape %s, expected %s" % (key, l.name, v.shape, l.params[key].shape), "Net::set_parameters")
                 l.params[key] = np.ascontiguousarray(v, np.float32)
+        if self.backend is not None:
+            self._push_parameters()
+
+    # ---- parameter files: the reference's "bin" format (Net::save / Net::load, src/net/net.cpp:411-449):
+    # for every layer in layer order, for every parameter in the layer's order (Layer::save,
+    # src/layers/layer.cpp:215-227; convolution K, bias; batch-norm bn_g, bn_b, mean, variance;
+    # dense W, bias), one record  int32 ndim | int32 shape[ndim] | float32 data[prod(shape)]
+    # (Tensor::save2bin / load_from_bin, src/tensor/tensor_serialization.cpp:70-110,252-261).
+    def save(self, filename, format="bin"):
+        if format != "bin":
+            msg("Format not implemented: *.'%s'" % format, "Tensor::save")
+        with open(filename, "wb") as fh:
+            for l in self.layers:
+                for v in l.params.values():
+                    fh.write(np.array([v.ndim] + list(v.shape), np.int32).tobytes())
+                    fh.write(np.ascontiguousarray(v, np.float32).tobytes())
+
+    def load(self, filename, format="bin"):
+        if format != "bin":
+            msg("Format not implemented: *.'%s'" % format, "Tensor::load")
+        try:
+            fh = open(filename, "rb")
+        except OSError:
+            raise RuntimeError("File not found. Check the file name and try again (Net::load)")
+        with fh:
+            for l in self.layers:
+                for key, cur in l.params.items():
+                    head = fh.read(4)
+                    if len(head) < 4:
+                        msg("parameter file ends before %s of layer %s" % (key, l.name), "Net::load")
+                    ndim = int(np.frombuffer(head, np.int32)[0])
+                    if ndim < 0 or ndim > 8:
+                        msg("parameter file is not in the bin format (ndim %d at %s of layer %s)" % (ndim, key, l.name), "Net::load")
+                    shape = np.frombuffer(fh.read(4 * ndim), np.int32)
+                    size = int(np.prod(shape, dtype=np.int64)) if ndim else 1
+                    # Tensor::copy accepts any shape of the same size (src/tensor/tensor_core.cpp:316-349)
+                    if len(shape) != ndim or size != cur.size:
+                        msg("Tensors with different size (%s of layer %s: file %s, layer %s)" % (key, l.name, list(shape), list(cur.shape)),
+                            "Tensor::copy")
+                    data = np.frombuffer(fh.read(4 * size), np.float32)
+                    if data.size != size:
+                        msg("parameter file ends inside %s of layer %s" % (key, l.name), "Net::load")
+                    l.params[key] = data.reshape(cur.shape).copy()
         if self.backend is not None:
             self._push_parameters()
 
