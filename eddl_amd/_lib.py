@@ -33,6 +33,14 @@ PROTOTYPES = {
     "eddlhip_event_destroy": [c_int, c_void_p],
     "eddlhip_event_record": [c_int, c_void_p],
     "eddlhip_event_elapsed_ms": [c_int, c_void_p, c_void_p, ctypes.POINTER(c_float)],
+    "eddlhip_host_malloc": [c_int, ctypes.POINTER(c_void_p), c_size_t],
+    "eddlhip_host_free": [c_int, c_void_p],
+    "eddlhip_memcpy_h2d_async": [c_int, P, c_void_p, c_size_t, c_void_p],
+    "eddlhip_memcpy_d2h_async": [c_int, c_void_p, P, c_size_t, c_void_p],
+    "eddlhip_stream_wait_event": [c_int, c_void_p],
+    "eddlhip_upload_wait_event": [c_int, c_void_p],
+    "eddlhip_download_wait_event": [c_int, c_void_p],
+    "eddlhip_event_synchronize": [c_int, c_void_p],
     "eddlhip_probe_mfma_f32": [c_int, c_int, c_int, ctypes.POINTER(c_float), ctypes.POINTER(c_float), ctypes.POINTER(c_float)],
     "eddlhip_conv2d_fwd": [c_int, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_cache_filters": [c_int, P, c_int, c_int, c_int, c_int],

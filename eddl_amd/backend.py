@@ -62,6 +62,29 @@ class _View(DeviceTensor):
         pass
 
 
+class PinnedArray:
+    """A float32 numpy array over page-locked host memory of the library (``.array``)."""
+
+    def __init__(self, backend, shape):
+        self.backend = backend
+        self.shape = tuple(int(d) for d in shape)
+        n = int(np.prod(self.shape)) if len(self.shape) else 1
+        self.nbytes = n * 4
+        p = ctypes.c_void_p()
+        backend._check(backend.lib.eddlhip_host_malloc(backend.dev, ctypes.byref(p), max(self.nbytes, 4)))
+        self.ptr = p.value
+        self.array = np.ctypeslib.as_array((ctypes.c_float * max(n, 1)).from_address(self.ptr))[:n].reshape(self.shape)
+
+    def __del__(self):
+        try:
+            if getattr(self, "ptr", None):
+                self.array = None
+                self.backend.lib.eddlhip_host_free(self.backend.dev, self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+
 class Event:
     def __init__(self, backend):
         self.backend = backend
@@ -72,6 +95,9 @@ class Event:
     def record(self):
         self.backend._check(self.backend.lib.eddlhip_event_record(self.backend.dev, self.handle))
         return self
+
+    def synchronize(self):
+        self.backend._check(self.backend.lib.eddlhip_event_synchronize(self.backend.dev, self.handle))
 
     def elapsed_ms(self, stop):
         ms = ctypes.c_float()
@@ -121,6 +147,25 @@ class Backend:
 
     def event(self):
         return Event(self)
+
+    # ---- batch staging (upload and download streams)
+    def pinned(self, shape):
+        return PinnedArray(self, shape)
+
+    def h2d_async(self, dst, pinned, done=None):
+        self._check(self.lib.eddlhip_memcpy_h2d_async(self.dev, dst.ptr, pinned.ptr, dst.nbytes, done.handle if done else None))
+
+    def d2h_async(self, pinned, src, done=None):
+        self._check(self.lib.eddlhip_memcpy_d2h_async(self.dev, pinned.ptr, src.ptr, src.nbytes, done.handle if done else None))
+
+    def stream_wait(self, event):
+        self._check(self.lib.eddlhip_stream_wait_event(self.dev, event.handle))
+
+    def upload_wait(self, event):
+        self._check(self.lib.eddlhip_upload_wait_event(self.dev, event.handle))
+
+    def download_wait(self, event):
+        self._check(self.lib.eddlhip_download_wait_event(self.dev, event.handle))
 
     def probe_mfma_f32(self, vary_operands=True, launches=40):
         """Sustained fp32 MFMA rate of the device with nothing else running: (mean, best launch, worst launch) TFLOP/s."""

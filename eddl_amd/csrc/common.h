@@ -18,6 +18,7 @@ struct DeviceState {
     void *workspace = nullptr;  // private, grow-only (repacked filters, split-K partials)
     size_t workspace_bytes = 0;
     void *flag = nullptr;  // one int of device memory for kernels that report a condition
+    hipStream_t copy_stream[2] = {nullptr, nullptr};  // uploads, downloads: created on first use (non-blocking, default priority)
 };
 
 DeviceState &state(int dev);

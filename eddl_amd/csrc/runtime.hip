@@ -92,6 +92,8 @@ int eddlhip_shutdown(int dev) {
     EH_TRY(eddlhip_conv2d_uncache_filters(dev, nullptr));
     if (s.workspace) EH_TRY_HIP(hipFree(s.workspace));
     if (s.flag) EH_TRY_HIP(hipFree(s.flag));
+    for (hipStream_t cs : s.copy_stream)
+        if (cs) EH_TRY_HIP(hipStreamDestroy(cs));
     s = DeviceState();
     return 0;
 }
@@ -169,6 +171,93 @@ int eddlhip_memcpy_d2d(int dev, void *dev_dst, const void *dev_src, size_t bytes
     EH_TRY(use_device(dev));
     conv_filters_written(dev, dev_dst, bytes);
     EH_TRY_HIP(hipMemcpyAsync(dev_dst, dev_src, bytes, hipMemcpyDeviceToDevice, state(dev).stream));
+    return 0;
+}
+
+// ---- batch staging: pinned host buffers and copies on a second stream, so that the transfer of
+// batch i+1 and of the results of batch i-1 overlap the kernels of batch i
+int eddlhip_host_malloc(int dev, void **host_ptr, size_t bytes) {
+    EH_REQUIRE(host_ptr != nullptr, "host_ptr is NULL");
+    EH_TRY(use_device(dev));
+    *host_ptr = nullptr;
+    if (bytes == 0) return 0;
+    hipError_t e = hipHostMalloc(host_ptr, bytes, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        *host_ptr = nullptr;
+        (void)hipGetLastError();
+        return set_error(EDDLHIP_ENOMEM, "hipHostMalloc(%zu): %s", bytes, hipGetErrorString(e));
+    }
+    return 0;
+}
+
+int eddlhip_host_free(int dev, void *host_ptr) {
+    if (!host_ptr) return 0;
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipHostFree(host_ptr));
+    return 0;
+}
+
+// which: 0 = upload stream, 1 = download stream (separate, so that an upload queued after a
+// download that is still waiting for kernels does not wait with it)
+static int copy_stream_of(int dev, int which, hipStream_t *out) {
+    DeviceState &s = state(dev);
+    if (!s.copy_stream[which]) EH_TRY_HIP(hipStreamCreateWithFlags(&s.copy_stream[which], hipStreamNonBlocking));
+    *out = s.copy_stream[which];
+    return 0;
+}
+
+int eddlhip_memcpy_h2d_async(int dev, void *dev_dst, const void *host_src, size_t bytes, void *done_event) {
+    EH_REQUIRE(bytes == 0 || (dev_dst && host_src), "NULL pointer in asynchronous h2d copy");
+    EH_TRY(use_device(dev));
+    hipStream_t cs;
+    EH_TRY(copy_stream_of(dev, 0, &cs));
+    if (bytes) {
+        conv_filters_written(dev, dev_dst, bytes);
+        EH_TRY_HIP(hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice, cs));
+    }
+    if (done_event) EH_TRY_HIP(hipEventRecord((hipEvent_t)done_event, cs));
+    return 0;
+}
+
+int eddlhip_memcpy_d2h_async(int dev, void *host_dst, const void *dev_src, size_t bytes, void *done_event) {
+    EH_REQUIRE(bytes == 0 || (host_dst && dev_src), "NULL pointer in asynchronous d2h copy");
+    EH_TRY(use_device(dev));
+    hipStream_t cs;
+    EH_TRY(copy_stream_of(dev, 1, &cs));
+    if (bytes) EH_TRY_HIP(hipMemcpyAsync(host_dst, dev_src, bytes, hipMemcpyDeviceToHost, cs));
+    if (done_event) EH_TRY_HIP(hipEventRecord((hipEvent_t)done_event, cs));
+    return 0;
+}
+
+int eddlhip_stream_wait_event(int dev, void *event) {
+    EH_REQUIRE(event != nullptr, "event is NULL");
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipStreamWaitEvent(state(dev).stream, (hipEvent_t)event, 0));
+    return 0;
+}
+
+int eddlhip_upload_wait_event(int dev, void *event) {
+    EH_REQUIRE(event != nullptr, "event is NULL");
+    EH_TRY(use_device(dev));
+    hipStream_t cs;
+    EH_TRY(copy_stream_of(dev, 0, &cs));
+    EH_TRY_HIP(hipStreamWaitEvent(cs, (hipEvent_t)event, 0));
+    return 0;
+}
+
+int eddlhip_download_wait_event(int dev, void *event) {
+    EH_REQUIRE(event != nullptr, "event is NULL");
+    EH_TRY(use_device(dev));
+    hipStream_t cs;
+    EH_TRY(copy_stream_of(dev, 1, &cs));
+    EH_TRY_HIP(hipStreamWaitEvent(cs, (hipEvent_t)event, 0));
+    return 0;
+}
+
+int eddlhip_event_synchronize(int dev, void *event) {
+    EH_REQUIRE(event != nullptr, "event is NULL");
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipEventSynchronize((hipEvent_t)event));
     return 0;
 }
 

@@ -339,6 +339,7 @@ class Net:
         self.backend = hip = backend
         self.fused = fuse
         self.cache_filters = cache_filters
+        self._staging = None
         self.dparams = {id(l): {k: hip.empty(v.shape) for k, v in l.params.items()} for l in self.layers}
         self._push_parameters()
         self.out = {}   # id(layer) -> DeviceTensor holding its output (absent for layers folded into a fused op)
@@ -529,6 +530,71 @@ class Net:
         """Inference forward; returns host arrays (the reference's predict collects outputs to the CPU)."""
         outs = self.forward(xs)
         return [o.numpy() for o in outs]
+
+    def predict_batches(self, batches):
+        """Inference over a stream of host batches (each a list with one array per input layer, or
+        one array): yields the output arrays of every batch, in order.  Transfers overlap compute:
+        batch i+1 goes through a page-locked host buffer and the upload stream into a second device
+        buffer while the kernels of batch i run, and the results of batch i come back while batch
+        i+1 computes (the reference stages every batch through blocking copies,
+        src/net/net_func.cpp:195-249).  All batches must have the built batch size."""
+        hip = self.backend
+        ins = [self.out[id(l)] for l in self.lin]
+        outs = [self.out[id(o)] for o in self.lout]
+        d2d = lambda dst, src: hip._check(hip.lib.eddlhip_memcpy_d2d(hip.dev, dst.ptr, src.ptr, dst.nbytes))
+        # two staging sets; per set: pinned + device copies of inputs and outputs, and four events:
+        # h2d / d2h on the upload / download stream (upload done, results on the host), consumed / computed on the
+        # compute stream (device input copy read, device output copy written)
+        if getattr(self, "_staging", None) is None:  # kept until the next build (page-locking memory takes milliseconds)
+            self._staging = [{"pin_in": [hip.pinned(t.shape) for t in ins], "dev_in": [hip.empty(t.shape) for t in ins],
+                              "pin_out": [hip.pinned(t.shape) for t in outs], "dev_out": [hip.empty(t.shape) for t in outs],
+                              "h2d": hip.event(), "d2h": hip.event(), "consumed": hip.event(), "computed": hip.event()}
+                             for _ in range(2)]
+        sets = self._staging
+        hip.synchronize()
+        for s in sets:
+            s["used"] = False
+
+        def collect(s):
+            s["d2h"].synchronize()
+            return [p.array.copy() for p in s["pin_out"]]
+
+        pending = None
+        for i, xs in enumerate(batches):
+            if not isinstance(xs, (list, tuple)):
+                xs = [xs]
+            if len(xs) != len(ins):
+                msg("Number of input tensors does not match the number of input layers", "Net::predict_batches")
+            s = sets[i % 2]
+            if s["used"]:
+                s["h2d"].synchronize()            # the upload of batch i-2 has left the pinned buffer
+            for t, pin, x in zip(ins, s["pin_in"], xs):
+                if tuple(x.shape) != t.shape:
+                    msg("input shape %s does not match %s" % (tuple(x.shape), t.shape), "Net::predict_batches")
+                np.copyto(pin.array, x, casting="same_kind")
+            if s["used"]:
+                hip.upload_wait(s["consumed"])  # batch i-2 has been copied out of this device buffer
+            for k, (dst, pin) in enumerate(zip(s["dev_in"], s["pin_in"])):
+                hip.h2d_async(dst, pin, s["h2d"] if k == len(ins) - 1 else None)
+            hip.stream_wait(s["h2d"])
+            for t, src in zip(ins, s["dev_in"]):
+                d2d(t, src)
+            s["consumed"].record()
+            self.run()
+            if s["used"]:
+                hip.stream_wait(s["d2h"])         # the results of batch i-2 have left this device buffer
+            for t, dst in zip(outs, s["dev_out"]):
+                d2d(dst, t)
+            s["computed"].record()
+            hip.download_wait(s["computed"])
+            for k, (pin, src) in enumerate(zip(s["pin_out"], s["dev_out"])):
+                hip.d2h_async(pin, src, s["d2h"] if k == len(outs) - 1 else None)
+            s["used"] = True
+            if pending is not None:
+                yield collect(pending)            # waits for batch i-1 while batch i computes
+            pending = s
+        if pending is not None:
+            yield collect(pending)
 
     def input_tensor(self, i=0):
         return self.out[id(self.lin[i])]

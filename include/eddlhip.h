@@ -58,6 +58,29 @@ int eddlhip_memcpy_d2h(int dev, void *host_dst, const void *dev_src, size_t byte
 int eddlhip_memcpy_d2d(int dev, void *dev_dst, const void *dev_src, size_t bytes);
 int eddlhip_fill(int dev, float *A, size_t n, float v);
 
+/* Batch staging.  The reference moves a batch to the device through pageable host tensors and
+ * blocking copies (Net::distributeTensor / collectTensor, src/net/net_func.cpp:195-249; a D2H +
+ * H2D round trip per batch, src/tensor/tensor_core.cpp:877-895).  These entry points let a host
+ * overlap that traffic with the kernels: page-locked host buffers, copies queued on two more
+ * streams of the device (one for uploads, one for downloads, so neither waits behind the other),
+ * and events to order them against the compute stream.
+ *   eddlhip_memcpy_h2d_async / _d2h_async: queue the copy on the upload / download stream and
+ *     return; the host buffer should come from eddlhip_host_malloc (a pageable one makes the copy
+ *     synchronous) and must stay untouched until done_event (recorded on that stream behind the
+ *     copy; may be NULL) has completed.
+ *   eddlhip_stream_wait_event: work queued later on the device's compute stream waits for event.
+ *   eddlhip_upload_wait_event / eddlhip_download_wait_event: uploads / downloads queued later wait
+ *     for event (e.g. one recorded with eddlhip_event_record after the kernels that last read the
+ *     upload's destination, or that wrote the download's source). */
+int eddlhip_host_malloc(int dev, void **host_ptr, size_t bytes);
+int eddlhip_host_free(int dev, void *host_ptr);
+int eddlhip_memcpy_h2d_async(int dev, void *dev_dst, const void *host_src, size_t bytes, void *done_event);
+int eddlhip_memcpy_d2h_async(int dev, void *host_dst, const void *dev_src, size_t bytes, void *done_event);
+int eddlhip_stream_wait_event(int dev, void *event);
+int eddlhip_upload_wait_event(int dev, void *event);
+int eddlhip_download_wait_event(int dev, void *event);
+int eddlhip_event_synchronize(int dev, void *event);
+
 /* Events on the device's stream, for timing kernels where they run.  No counterpart in the
  * reference (its profiling is host wall-clock, include/eddl/profiling.h:27-66). */
 int eddlhip_event_create(int dev, void **event);

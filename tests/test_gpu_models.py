@@ -145,3 +145,21 @@ def test_set_parameters_after_build_reaches_the_cached_filters(hip, oracle):
     assert np.array_equal(y2, fresh.predict([x])[0]) and not np.array_equal(y1, y2)
     m.set_parameters(params)
     assert np.array_equal(m.predict([x])[0], y1)
+
+
+def test_predict_batches_overlapped_staging_matches_predict(hip, oracle):
+    """Seven different batches through the pipelined path (pinned staging, upload and download streams, two device
+    buffers) give, in order, exactly what one blocking predict per batch gives."""
+    from eddl_amd import models
+    m = models.unet(batch=2, size=32, widths=(4, 8), bottleneck=16)
+    models.init_he_normal(m, 31)
+    m.build(hip)
+    rng = np.random.default_rng(31)
+    batches = [rng.uniform(0, 1, (2, 1, 32, 32)).astype(np.float32) for _ in range(7)]
+    want = [m.predict([x])[0] for x in batches]
+    got = [outs[0] for outs in m.predict_batches(batches)]
+    assert len(got) == len(want)
+    for a, b in zip(want, got):
+        assert np.array_equal(a, b)
+    assert [o[0].shape for o in m.predict_batches([batches[0]])] == [want[0].shape]
+    assert list(m.predict_batches([])) == []
