@@ -183,20 +183,30 @@ __device__ __forceinline__ void store_partial(const ConvParams &p, floatx16 (&ac
             for (int v = 0; v < 16; v++) dst[((tm * TN + tn) * 16 + v) * 64] = acc[tm][tn][v];
 }
 
-// The per-channel constants of a tile's BM channels, computed once per workgroup into LDS
-// (layout: bias[BM], mean[BM], sd[BM], g[BM], b[BM]); the caller synchronises before and after.
+// The per-channel constants of a tile's BM channels reach the epilogue through LDS (layout:
+// bias[BM], mean[BM], sd[BM], g[BM], b[BM]).  Thread t < BM fetches those of channel m0 + t at the
+// START of the kernel, so that their memory latency passes during the K loop instead of standing
+// between the last MFMA and the first store, and writes them to LDS after the loop; the caller
+// synchronises before and after that write.
 template <int BM>
-__device__ __forceinline__ void stage_channel_constants(const ConvParams &p, float *epi, int m0, int tid) {
+__device__ __forceinline__ ChannelEpilogue fetch_channel_constants(const ConvParams &p, int m0, int tid) {
+    ChannelEpilogue e = {0.0f, 0.0f, 1.0f, 1.0f, 0.0f};
+    if (tid < BM && m0 + tid < p.Kf) e = load_channel(p, m0 + tid);
+    return e;
+}
+template <int BM>
+__device__ __forceinline__ void put_channel_constants(float *epi, const ChannelEpilogue &e, int tid) {
     if (tid < BM) {
-        const int k = m0 + tid;
-        ChannelEpilogue e = {0.0f, 0.0f, 1.0f, 1.0f, 0.0f};
-        if (k < p.Kf) e = load_channel(p, k);
         epi[tid] = e.bias;
         epi[BM + tid] = e.mean;
         epi[2 * BM + tid] = e.sd;
         epi[3 * BM + tid] = e.g;
         epi[4 * BM + tid] = e.b;
     }
+}
+template <int BM>
+__device__ __forceinline__ void stage_channel_constants(const ConvParams &p, float *epi, int m0, int tid) {
+    put_channel_constants<BM>(epi, fetch_channel_constants<BM>(p, m0, tid), tid);
 }
 
 // Writes a wavefront's TM x TN blocks.  A lane holds column (pixel) lane%32 and rows
@@ -318,6 +328,8 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     const int step_hi = split ? min(step_lo + p.slice_steps, p.nsteps) : p.nsteps;
     const int m0 = m_tile * BM;
     const long long n0 = (long long)n_tile * BN;
+    ChannelEpilogue chan = {0.0f, 0.0f, 1.0f, 1.0f, 0.0f};
+    if (!split) chan = fetch_channel_constants<BM>(p, m0, tid);
 
     const __amdgpu_buffer_rsrc_t rsrc_in = __builtin_amdgcn_make_buffer_rsrc((void *)p.I, 0, p.in_bytes, RSRC_WORD3);
 
@@ -500,7 +512,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
     } else {
         float *epi = &As[0][0];  // the K loop ended with a barrier: the filter buffers are free
-        stage_channel_constants<BM>(p, epi, m0, tid);
+        put_channel_constants<BM>(epi, chan, tid);
         __syncthreads();
         store_tile<TM, TN, BM>(p, acc, epi, m0, wm * TM * 32, (int)n0 + wn * TN * 32, lane);
     }
@@ -535,6 +547,8 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
     const int step_hi = split ? min(step_lo + p.slice_steps, p.nsteps) : p.nsteps;
     const int m0 = m_tile * BM;
     const long long n0 = (long long)n_tile * BN;
+    ChannelEpilogue chan = {0.0f, 0.0f, 1.0f, 1.0f, 0.0f};
+    if (!split) chan = fetch_channel_constants<BM>(p, m0, tid);
 
     const __amdgpu_buffer_rsrc_t rsrc_in = __builtin_amdgcn_make_buffer_rsrc((void *)p.I, 0, p.in_bytes, RSRC_WORD3);
 
@@ -657,7 +671,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
         store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
     } else {
         float *epi = &As[0][0];  // the K loop ended with a barrier: the filter buffers are free
-        stage_channel_constants<BM>(p, epi, m0, tid);
+        put_channel_constants<BM>(epi, chan, tid);
         __syncthreads();
         store_tile<TM, TN, BM>(p, acc, epi, m0, wm * TM * 32, (int)n0 + wn * TN * 32, lane);
     }
