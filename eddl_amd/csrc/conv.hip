@@ -819,8 +819,8 @@ struct Plan {
 };
 
 Plan plan_conv(const Variant *family, int Kf, int C, int RS, long long npix, int num_cu, bool allow_split) {
-    static const double kEff[4] = {0.80, 0.66, 0.52, 0.40};      // fraction of the MFMA peak a long K loop sustains, per tile shape
-    static const double kOverheadUs[4] = {5.0, 3.5, 2.5, 2.5};   // prologue + epilogue of one workgroup (CU time)
+    static const double kEff[4] = {0.90, 0.875, 0.87, 0.86};      // fraction of the MFMA peak a long K loop sustains, per tile shape
+    static const double kOverheadUs[4] = {5.0, 3.0, 1.5, 2.0};   // prologue + epilogue of one workgroup (CU time)
     const double cu_flops_per_us = 157.3e6 / 256.0;
     const double bytes_per_us = 3.0e6;  // partial-sum traffic
     // a CU with fewer resident workgroups than it can hold hides less latency
