@@ -64,6 +64,7 @@ PROTOTYPES = {
     "eddlhip_pad": [c_int, P, P] + [c_int] * 8,
     "eddlhip_mult2d": [c_int, P, P, P, c_int, c_int, c_int, c_int],
     "eddlhip_sum2d_rowwise": [c_int, P, P, P, c_int, c_int],
+    "eddlhip_dense_fwd": [c_int, P, P, P, P, c_int, c_int, c_int, c_int],
 }
 _RESTYPE = {"eddlhip_version": ctypes.c_char_p, "eddlhip_last_error": ctypes.c_char_p,
             "eddlhip_conv2d_last_kernel": ctypes.c_char_p}

@@ -296,5 +296,13 @@ class Backend:
             raise ValueError("mult2D shapes %s x %s -> %s" % (A.shape, B.shape, C.shape))
         self._check(self.lib.eddlhip_mult2d(self.dev, A.ptr, B.ptr, C.ptr, m, k, n, incC))
 
+    def dense(self, A, W, bias, C, relu=False):
+        """C = A W (+ bias per column) (then ReLU): LDense::forward (+ a following ReLU) in one call."""
+        m, k = A.shape
+        k2, n = W.shape
+        if k != k2 or C.shape != (m, n):
+            raise ValueError("dense shapes %s x %s -> %s" % (A.shape, W.shape, C.shape))
+        self._check(self.lib.eddlhip_dense_fwd(self.dev, A.ptr, W.ptr, _ptr(bias), C.ptr, m, k, n, int(relu)))
+
     def sum2D_rowwise(self, A, B, C):
         self._check(self.lib.eddlhip_sum2d_rowwise(self.dev, A.ptr, B.ptr, C.ptr, A.shape[0], A.shape[1]))

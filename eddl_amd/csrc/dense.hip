@@ -118,22 +118,31 @@ __global__ __launch_bounds__(64) void dense_partial_kernel(const float *__restri
     }
 }
 
+// Adds the K slices in slice order; then, in the reference's order, C += (incC), + bias[column]
+// (sum2D_rowwise) and ReLU - each an fp32 operation of its own, so the fused tail equals the
+// separate launches bit for bit.
 __global__ __launch_bounds__(256) void dense_reduce_kernel(const float *__restrict__ part, float *C, size_t mn, int nslices,
-                                                           int incC) {
+                                                           int incC, const float *__restrict__ bias, int n, int relu) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, stride = (size_t)gridDim.x * 256;
     for (size_t t = i; t < mn; t += stride) {
         float s = part[t];
         for (int ks = 1; ks < nslices; ks++) s = __fadd_rn(s, part[(size_t)ks * mn + t]);
-        C[t] = incC ? __fadd_rn(C[t], s) : s;
+        if (incC) s = __fadd_rn(C[t], s);
+        if (bias) s = __fadd_rn(s, bias[t % (size_t)n]);
+        if (relu) s = s > 0.0f ? s : 0.0f;
+        C[t] = s;
     }
 }
 
 }  // namespace
 
-extern "C" int eddlhip_mult2d(int dev, const float *A, const float *B, float *C, int m, int k, int n, int incC) {
-    EH_REQUIRE(m >= 0 && k > 0 && n > 0, "mult2d: bad shape %dx%d * %dx%d", m, k, k, n);
+namespace {
+
+int dense_impl(int dev, const float *A, const float *B, float *C, int m, int k, int n, int incC, const float *bias, int relu,
+               const char *what) {
+    EH_REQUIRE(m >= 0 && k > 0 && n > 0, "%s: bad shape %dx%d * %dx%d", what, m, k, k, n);
     if (m == 0) return 0;
-    EH_REQUIRE(A && B && C, "mult2d: NULL tensor");
+    EH_REQUIRE(A && B && C, "%s: NULL tensor", what);
     EH_TRY(use_device(dev));
     hipStream_t st = state(dev).stream;
     const int nt = (n + 127) / 128, mt = (m + 31) / 32;
@@ -145,7 +154,7 @@ extern "C" int eddlhip_mult2d(int dev, const float *A, const float *B, float *C,
     if (nslices > max_slices) nslices = max_slices;
     int kslice = ((k + nslices - 1) / nslices + 1) & ~1;  // even, so MFMA tap pairs do not straddle slices
     nslices = (k + kslice - 1) / kslice;
-    EH_REQUIRE(nslices <= 65535 && mt <= 65535, "mult2d: shape out of range");
+    EH_REQUIRE(nslices <= 65535 && mt <= 65535, "%s: shape out of range", what);
     const size_t at_bytes = ((size_t)mt * k * 32 * sizeof(float) + 255) & ~(size_t)255;
     void *ws = nullptr;
     EH_TRY(get_workspace(dev, at_bytes + (size_t)nslices * m * n * sizeof(float), &ws));
@@ -157,7 +166,18 @@ extern "C" int eddlhip_mult2d(int dev, const float *A, const float *B, float *C,
     else hipLaunchKernelGGL(dense_partial_kernel<false>, dim3(nt, nslices, mt), dim3(64), 0, st, At, B, part, m, k, n, kslice);
     EH_CHECK_LAUNCH();
     size_t mn = (size_t)m * n;
-    hipLaunchKernelGGL(dense_reduce_kernel, dim3(eh_blocks(mn, 256, 65536)), dim3(256), 0, st, (const float *)part, C, mn, nslices, incC);
+    hipLaunchKernelGGL(dense_reduce_kernel, dim3(eh_blocks(mn, 256, 65536)), dim3(256), 0, st, (const float *)part, C, mn, nslices, incC,
+                       bias, n, relu);
     EH_CHECK_LAUNCH();
     return 0;
+}
+
+}  // namespace
+
+extern "C" int eddlhip_mult2d(int dev, const float *A, const float *B, float *C, int m, int k, int n, int incC) {
+    return dense_impl(dev, A, B, C, m, k, n, incC, nullptr, 0, "mult2d");
+}
+
+extern "C" int eddlhip_dense_fwd(int dev, const float *A, const float *W, const float *bias, float *C, int m, int k, int n, int relu) {
+    return dense_impl(dev, A, W, C, m, k, n, 0, bias, relu, "dense_fwd");
 }

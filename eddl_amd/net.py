@@ -361,6 +361,9 @@ class Net:
             if l.kind == "conv2d":
                 self._emit_conv(l, fuse, absorbed, sole_child)
                 continue
+            if l.kind == "dense":
+                self._emit_dense(l, fuse, absorbed, sole_child)
+                continue
             self._emit_plain(l)
         for o in self.lout:
             if id(o) not in self.out:
@@ -422,6 +425,35 @@ class Net:
         self.ops.append(Op("conv2d", name, lambda: hip.conv2D(I, dp["K"], bias, O, cd.sr, cd.sc, pt, pl, bn=dbn, residual=R, relu=relu),
                            flops, nbytes, [l] + chain))
 
+    def _emit_dense(self, l, fuse, absorbed, sole_child):
+        """LDense::forward = mult2D + sum2D_rowwise (src/layers/core/layer_dense.cpp:65-73); a fused plan
+        makes it one call and takes a following ReLU along."""
+        hip = self.backend
+        src = self.out[id(l.parents[0])]
+        dp = self.dparams[id(l)]
+        in_dim, ndim = dp["W"].shape
+        rows = int(np.prod(l.out_shape)) // ndim
+        bias = dp["bias"] if l.attrs["use_bias"] else None
+        last, relu = l, False
+        if fuse:
+            c = sole_child(l)
+            if c is not None and c.kind == "relu":
+                last, relu = c, True
+                absorbed.add(id(c))
+        O = hip.empty(last.out_shape)
+        self.out[id(last)] = O
+        A2, C2 = src.reshape((rows, in_dim)), O.reshape((rows, ndim))
+        if fuse:
+            run = lambda: hip.dense(A2, dp["W"], bias, C2, relu=relu)
+        else:
+            def run():
+                hip.mult2D(A2, dp["W"], C2, 0)
+                if bias is not None:
+                    hip.sum2D_rowwise(C2, bias, C2)
+        name = l.name if last is l else l.name + "+" + last.name
+        layers = [l] if last is l else [l, last]
+        self.ops.append(Op("dense", name, run, 2 * rows * in_dim * ndim, 4 * (rows * in_dim + in_dim * ndim + rows * ndim), layers))
+
     def _emit_plain(self, l):
         hip = self.backend
         k = l.kind
@@ -473,19 +505,6 @@ class Net:
             hip.fill_(O, l.attrs["constant"])  # the border is written once, here; forward copies the interior
             n_in = int(np.prod(l.parents[0].out_shape))
             run, nbytes = (lambda: hip.pad(ins[0], O, l.attrs["pads"])), 8 * n_in
-        elif k == "dense":
-            dp = self.dparams[id(l)]
-            in_dim, ndim = dp["W"].shape
-            rows = n_out // ndim
-            A2, C2 = ins[0].reshape((rows, in_dim)), O.reshape((rows, ndim))
-            use_bias = l.attrs["use_bias"]
-
-            def run():
-                hip.mult2D(A2, dp["W"], C2, 0)
-                if use_bias:
-                    hip.sum2D_rowwise(C2, dp["bias"], C2)
-            self.ops.append(Op("dense", l.name, run, 2 * rows * in_dim * ndim, 4 * (rows * in_dim + in_dim * ndim + rows * ndim), [l]))
-            return
         else:
             msg("layer kind %s has no forward on this backend" % k, "Net::build")
         self.ops.append(Op(k, l.name, run, 0, nbytes, [l]))

@@ -235,6 +235,11 @@ int eddlhip_pad(int dev, const float *A, float *B, int N, int C, int H, int W,
  * eddlhip_sum2d_rowwise replaces gpu_sum2D_rowwise: C[i][j] = A[i][j] + B[j]. */
 int eddlhip_mult2d(int dev, const float *A, const float *B, float *C, int m, int k, int n, int incC);
 int eddlhip_sum2d_rowwise(int dev, const float *A, const float *B, float *C, int rows, int cols);
+/* LDense::forward in one call: C[m,n] = A[m,k] * W[k,n], then + bias[column] when bias != NULL
+ * (sum2D_rowwise), then ReLU when relu != 0 (the LActivation that commonly follows; 
+ * src/hardware/cpu/nn/cpu_activations.cpp:18-33).  Each step is the separate call's fp32 operation,
+ * so the result equals eddlhip_mult2d + eddlhip_sum2d_rowwise + eddlhip_relu bit for bit. */
+int eddlhip_dense_fwd(int dev, const float *A, const float *W, const float *bias, float *C, int m, int k, int n, int relu);
 
 #ifdef __cplusplus
 }

@@ -387,6 +387,17 @@ def test_dense_sigmoid_softmax_within_tolerance(hip, oracle):
         hip.mult2D(hip.array(a), hip.array(w), C)
         hip.sum2D_rowwise(C, hip.array(bias), C)
         assert_conv_close(ref, C.numpy(), "dense %dx%dx%d" % (m, k, n))
+        # the one-call form equals mult2D + sum2D_rowwise (+ ReLU) bit for bit
+        F = hip.empty((m, n))
+        hip.dense(hip.array(a), hip.array(w), hip.array(bias), F)
+        assert np.array_equal(F.numpy(), C.numpy())
+        hip.dense(hip.array(a), hip.array(w), hip.array(bias), F, relu=True)
+        R = hip.empty((m, n))
+        hip.relu(C, R)
+        assert np.array_equal(F.numpy(), R.numpy())
+        hip.dense(hip.array(a), hip.array(w), None, F)
+        hip.mult2D(hip.array(a), hip.array(w), R)
+        assert np.array_equal(F.numpy(), R.numpy())
     x = rng.standard_normal((4, 1, 33, 31), dtype=np.float32) * 4
     B = hip.empty(x.shape)
     hip.sigmoid(hip.array(x), B)
