@@ -349,6 +349,12 @@ def test_upsample_concat_pad_bit_exact(hip, oracle):
         B = hip.empty(ref.shape)
         hip.scale(hip.array(x), B, (9 * s, 7 * s))
         assert np.array_equal(B.numpy(), ref)
+    for shape in [(3, 4, 10, 12), (1, 2, 1, 2), (2, 3, 33, 64), (1, 1, 512, 510)]:  # exact doubling, even width: the float4 path
+        y = rng.standard_normal(shape, dtype=np.float32)
+        ref = oracle.scale_nearest(y, (shape[2] * 2, shape[3] * 2))
+        B = hip.empty(ref.shape)
+        hip.scale(hip.array(y), B, (shape[2] * 2, shape[3] * 2))
+        assert np.array_equal(B.numpy(), ref), shape
     ref = oracle.scale_nearest(x, (13, 10))  # non-integer factor, same float rule
     B = hip.empty(ref.shape)
     hip.scale(hip.array(x), B, (13, 10))
