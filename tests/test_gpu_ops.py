@@ -458,3 +458,55 @@ def test_conv2d_cached_filters_follow_every_write(hip, oracle):
         assert np.array_equal(conv(K2), plain1)
         del K2
     hip.uncache_conv_filters(None)
+
+
+def test_conv2d_random_shapes_against_oracle(hip, oracle):
+    """120 seeded random problems: filter sides 1..7 (square and rectangular), strides 1..3, "same" /
+    "valid" / custom symmetric pads, channel and filter counts that are not multiples of anything,
+    batch 1..9, planes down to one pixel; whatever plan the planner picks."""
+    rng = np.random.default_rng(417)
+    done = 0
+    while done < 120:
+        R, S = (int(rng.integers(1, 8)),) * 2 if rng.random() < 0.7 else (int(rng.integers(1, 6)), int(rng.integers(1, 6)))
+        sr, sc = (int(rng.integers(1, 4)),) * 2 if rng.random() < 0.8 else (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        H, W = int(rng.integers(R, 40)), int(rng.integers(S, 40))
+        N, C, Kf = int(rng.integers(1, 10)), int(rng.integers(1, 70)), int(rng.integers(1, 150))
+        mode = rng.choice(["same", "valid", "custom"])
+        pads = None
+        if mode == "custom":
+            pt, pl = int(rng.integers(0, R)), int(rng.integers(0, S))
+            pads = [pt, pt, pl, pl]
+        try:
+            from eddl_amd.descriptors import ConvolDescriptor
+            cd = ConvolDescriptor(Kf, [R, S], [sr, sc], str(mode), pads or [], use_bias=True).build([N, C, H, W])
+        except RuntimeError:
+            continue  # geometry the reference refuses (e.g. an empty output)
+        if min(cd.out_shape) < 1:
+            continue
+        x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+        w = (rng.standard_normal((Kf, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32)
+        b = rng.standard_normal(Kf, dtype=np.float32)
+        ref, out = run_conv(hip, oracle, x, w, b, (sr, sc), str(mode), pads, relu=bool(done % 2))
+        assert_conv_close(ref, out, "%s %s pads %s stride %s %s" % ((N, C, H, W, Kf, R, S), mode, pads, (sr, sc), hip.last_conv_kernel()))
+        done += 1
+
+
+def test_conv2d_input_beyond_2gib_runs_in_batch_chunks(hip, oracle):
+    """An input of 2.7 GB is more than one buffer descriptor addresses: the launch is cut into batch
+    chunks.  Sampled outputs from every chunk (first and last image included) against the oracle's
+    direct form; the residual and the output pointers must advance with the chunks as well."""
+    rng = np.random.default_rng(418)
+    N, C, H, W, Kf = 42, 64, 512, 512, 4
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    w = (rng.standard_normal((Kf, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32)
+    b = rng.standard_normal(Kf, dtype=np.float32)
+    res = rng.standard_normal((N, Kf, H, W), dtype=np.float32)
+    O = hip.empty((N, Kf, H, W))
+    hip.conv2D(hip.array(x), hip.array(w), hip.array(b), O, 1, 1, 1, 1, residual=hip.array(res))
+    got = O.numpy()
+    idx = np.stack([rng.integers(0, N, 4000), rng.integers(0, Kf, 4000), rng.integers(0, H, 4000), rng.integers(0, W, 4000)], 1)
+    idx = np.concatenate([idx, [[0, 0, 0, 0], [N - 1, Kf - 1, H - 1, W - 1], [31, 1, 511, 511], [32, 2, 0, 0]]]).astype(np.int32)
+    ref = oracle.conv2d_at(x, w, b, (1, 1), 1, 1, idx) + res[idx[:, 0], idx[:, 1], idx[:, 2], idx[:, 3]]
+    pts = got[idx[:, 0], idx[:, 1], idx[:, 2], idx[:, 3]]
+    tol = 1e-5 * float(np.abs(got).max()) + 1e-4 * np.abs(ref)
+    assert np.all(np.abs(ref - pts) <= tol), np.abs(ref - pts).max()
