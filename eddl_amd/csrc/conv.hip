@@ -21,14 +21,15 @@
 //   conv_tap_kernel  filter shape known at compile time (3x3, 1x1, 2x2): a K-step is CPB whole
 //                    input channels; every thread gathers ONE fixed output pixel, so the R*S
 //                    tap offsets (and their validity) are computed once, before the loop, and
-//                    the per-step address work is one scalar offset per channel.  Optionally
-//                    the gather goes global -> LDS directly (buffer_load ... lds), skipping
-//                    the register file.
+//                    the per-step address work is one scalar offset per channel.  By default
+//                    both operand slices go global -> LDS directly (buffer_load ... lds),
+//                    skipping the register file; a register-staged form is kept for checking.
 //   conv_gen_kernel  any filter shape, K-step 16 taps, tap validity computed per element.
 //
 // Accumulation order per output: taps in increasing i, two per MFMA (the instruction adds
 // both products of a pair into the fp32 accumulator), one accumulator from the first tap to
-// the last; no split over taps.  The reference CPU order is ky,kx,c per output in its direct
+// the last.  Tiles the launch plan divides along K (plan_conv) are summed slice by slice in
+// increasing K order by conv_reduce_kernel: a fixed order too.  The reference CPU order is ky,kx,c per output in its direct
 // form and Eigen-internal in its GEMM form, so agreement is to a tolerance, not bit-for-bit;
 // the scalar kernel at the end of this file follows the direct form's order and rounding.
 //
@@ -768,7 +769,7 @@ int prof_end(hipStream_t st) {
     return 0;
 }
 thread_local char g_last_kernel[128] = "";
-int g_split = 1;  // divide the tiles of a mostly idle last round along K (set_algo 5 turns it off)
+int g_split = 1;  // divide the tiles left over after a whole number per CU along K (set_algo 5 turns it off)
 int g_force_tile = -1, g_force_slices = -1;  // eddlhip_conv2d_force_plan
 
 struct Variant {

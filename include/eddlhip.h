@@ -125,8 +125,9 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
  * 2 = the scalar direct kernel (one thread per output; taps summed in the reference's ky,kx,c
  * order with its rounding - used to cross-check the MFMA kernels on the device);
  * 3 = MFMA with the operand slices staged through registers; 4 = MFMA with the operand slices
- * written by the load unit straight into LDS (what 0 and 1 select); 5 / 6 = switch off / on the division along K of
- * the tiles of a mostly idle last round of workgroups (on by default; independent of 0-4).
+ * written by the load unit straight into LDS (what 0 and 1 select); 5 / 6 = switch off / on the
+ * division along K of the tiles left over after a whole number of tiles per CU (on by default;
+ * independent of 0-4).
  * eddlhip_conv2d_last_kernel() names the kernel the calling thread's last eddlhip_conv2d_fwd
  * launched, followed by " +ksplit(T tiles x S)" when T tiles were divided into S slices. */
 int eddlhip_conv2d_set_algo(int algo);
@@ -155,7 +156,7 @@ int eddlhip_conv2d_uncache_filters(int dev, const float *K);
 
 /* Measurement hook (no counterpart in the reference).  eddlhip_conv2d_profile(1) starts a
  * collection: from then on every launch of a convolution kernel made by eddlhip_conv2d_fwd
- * (one per call, two when the last round is divided along K; not the filter repack, not the
+ * (one per batch chunk, so one per call for inputs up to 2 GiB; not the filter repack, not the
  * finishing kernel of a K-split) is bracketed by its own pair of events on the device's stream.
  * eddlhip_conv2d_profile_read waits for those launches and returns how many there were and the
  * sum of their durations; eddlhip_conv2d_profile(0) stops collecting.  Either call of
