@@ -820,7 +820,7 @@ struct Plan {
 };
 
 Plan plan_conv(const Variant *family, int Kf, int C, int RS, long long npix, int num_cu, bool allow_split) {
-    static const double kEff[4] = {0.90, 0.875, 0.87, 0.86};      // fraction of the MFMA peak a long K loop sustains, per tile shape
+    static const double kEff[4] = {0.90, 0.905, 0.87, 0.86};      // fraction of the MFMA peak a long K loop sustains, per tile shape
     static const double kOverheadUs[4] = {5.0, 3.0, 1.5, 2.0};   // prologue + epilogue of one workgroup (CU time)
     const double cu_flops_per_us = 157.3e6 / 256.0;
     const double bytes_per_us = 3.0e6;  // partial-sum traffic
@@ -845,9 +845,16 @@ Plan plan_conv(const Variant *family, int Kf, int C, int RS, long long npix, int
             if (sl != want && want != 1) continue;  // same plan as a smaller `want`
             const long long wgs = left * sl;
             const long long per_cu = (wgs + num_cu - 1) / num_cu;
-            const long long resident = full + per_cu;
-            double cost = ((double)full * tile_us + (double)per_cu * (ss * step_us + kOverheadUs[t])) /
-                          crowd(resident < v.occupancy ? resident : v.occupancy);
+            // a CU works through its `full` whole tiles `occupancy` at a time; the last, smaller group
+            // (plus the K slices, which are short) runs with fewer wavefronts to hide latency
+            const long long occ = v.occupancy;
+            const long long tail = full % occ;
+            double cost = (double)(full - tail) * tile_us / crowd(occ);
+            if (tail > 0) cost += (double)tail * tile_us / crowd(tail + (per_cu > 0 ? 1 : 0));
+            if (per_cu > 0) {
+                const long long resident = (tail > 0 ? tail : (full > 0 ? occ - 1 : 0)) + per_cu;
+                cost += (double)per_cu * (ss * step_us + kOverheadUs[t]) / crowd(resident < occ ? resident : occ);
+            }
             if (sl > 1) cost += (double)wgs * v.bm * v.bn * 8.0 / bytes_per_us + 6.0;
             if (best.cost_us < 0 || cost < best.cost_us) {
                 best.tile = t;
