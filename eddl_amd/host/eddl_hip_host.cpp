@@ -130,6 +130,21 @@ Tensor::Tensor(const vector<int> &shp, float *fptr, int dev) : device(dev), ndim
     }
 }
 
+Tensor::Tensor(const vector<int> &shp, Tensor *T) : device(T->device), isshared(true), ndim((unsigned)shp.size()), shape(shp) {
+    size = 1;
+    for (int d : shape) size *= (unsigned long)d;
+    updateStrides();
+    share(T);
+}
+
+void Tensor::share(Tensor *T) {
+    if (!isshared) msg("only a tensor created as a view can be re-pointed", "Tensor::share");
+    if (T->size != size) msg("Tensors with different size", "Tensor::share");
+    device = T->device;
+    gpu_device = T->gpu_device;
+    ptr = T->ptr;
+}
+
 Tensor::~Tensor() { release(); }
 
 void Tensor::toGPU(int dev) {

@@ -41,6 +41,8 @@ class Tensor {
 
     Tensor(const vector<int> &shape, int dev = DEV_CPU);               // allocates (host or device)
     Tensor(const vector<int> &shape, float *fptr, int dev = DEV_CPU);  // adopts fptr (host) or copies it to the device
+    Tensor(const vector<int> &shape, Tensor *T);  // shares T's storage (isshared; src/tensor/tensor.cpp:78-79)
+    void share(Tensor *T);                        // points a shared tensor at T's current storage again (T moved or resized)
     ~Tensor();
     Tensor(const Tensor &) = delete;
     Tensor &operator=(const Tensor &) = delete;

@@ -1,0 +1,700 @@
+// Layers, Net and the eddl:: API of the CNN forward path (see eddl_hip_net.h for what each class mirrors).
+#include "eddl_hip_net.h"
+
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <fstream>
+#include <iomanip>
+#include <iostream>
+#include <set>
+#include <sstream>
+
+namespace eddl_hip {
+
+// ---------------------------------------------------------------- Layer
+int Layer::total_layers = 0;
+
+Layer::Layer(const string &n, const string &default_prefix) : name(n) {
+    if (name.empty()) name = default_prefix + std::to_string(++total_layers);
+}
+
+Layer::~Layer() {
+    delete output;
+    for (Tensor *t : params) delete t;
+    for (Tensor *t : extra) delete t;
+    for (Tensor *t : fixed) delete t;
+}
+
+void Layer::addchild(Layer *l) {
+    child.push_back(l);
+    lout++;
+}
+
+void Layer::addparent(Layer *l) {
+    parent.push_back(l);
+    lin++;
+}
+
+void Layer::resize(int batch) {
+    output->resize(batch);
+    for (Tensor *t : extra) t->resize(batch);
+}
+
+void Layer::toGPU(int device) {
+    dev = device;
+    output->toGPU(device);
+    for (Tensor *t : params) t->toGPU(device);
+    for (Tensor *t : extra) t->toGPU(device);
+    for (Tensor *t : fixed) t->toGPU(device);
+}
+
+// Parameter initialisation of build(init_weights = true): Glorot-uniform filters and weights, zero
+// biases (the reference's defaults, src/layers/conv/layer_conv2D.cpp:109-112 and
+// src/initializers/initializer_glorot.cpp), drawn from a generator of this file's own.
+namespace {
+struct Rng {
+    uint64_t s;
+    explicit Rng(uint64_t seed) : s(seed * 0x9E3779B97F4A7C15ull + 0x632BE59BD9B4E019ull) {}
+    float uniform() {  // [0, 1)
+        s ^= s << 13;
+        s ^= s >> 7;
+        s ^= s << 17;
+        return (float)((s >> 40) * (1.0 / 16777216.0));
+    }
+};
+
+void glorot_uniform(Tensor *t, int fan_in, int fan_out, unsigned seed) {
+    const bool on_gpu = t->isGPU();
+    const int device = t->device;
+    if (on_gpu) t->toCPU();
+    Rng rng(seed);
+    const float limit = std::sqrt(6.0f / (float)(fan_in + fan_out));
+    for (unsigned long i = 0; i < t->size; i++) t->ptr[i] = (2.0f * rng.uniform() - 1.0f) * limit;
+    if (on_gpu) t->toGPU(device);
+}
+}  // namespace
+
+// ---------------------------------------------------------------- LInput
+LInput::LInput(Tensor *in, string n) : Layer(n, "input") {
+    input = output = in;
+}
+
+// ---------------------------------------------------------------- LConv
+LConv::LConv(Layer *p, int filters, const vector<int> &kernel_size, const vector<int> &strides, string padding, const vector<int> &pads,
+             int groups, const vector<int> &dilation_rate, bool use_bias, string n)
+    : Layer(n, "conv2d") {
+    if (p->output->ndim != 4) msg("LConv only works over 4D tensors", "LConv::LConv");
+    cd = new ConvolDescriptor(filters, kernel_size, strides, padding, pads, groups, dilation_rate, use_bias, 0);
+    input = p->output;
+    cd->build(input);
+    output = cd->O;
+    params.push_back(cd->K);
+    params.push_back(cd->bias);
+    if (cd->pads[0] != cd->pads[1] || cd->pads[2] != cd->pads[3]) {
+        string text = "In layer " + name + ": Padding asymmetry detected (top=" + std::to_string(cd->pads[0]) +
+                      ", bottom=" + std::to_string(cd->pads[1]) + ", left=" + std::to_string(cd->pads[2]) +
+                      ", right=" + std::to_string(cd->pads[3]) +
+                      "). The padding asymmetry is not allowed in a Conv layer, we suggest you to use an explicit padding layer "
+                      "before this layer to fix the asymmetry.";
+        vector<int> asym = cd->pads;
+        delete cd;
+        cd = nullptr;
+        throw AsymmetricPaddingException(text, asym);  // the base destructor releases the tensors
+    }
+    p->addchild(this);
+    addparent(p);
+}
+
+LConv::~LConv() { delete cd; }
+
+void LConv::forward() { tensorNN::Conv2D(cd); }
+
+void LConv::resize(int batch) {
+    cd->I = input;
+    cd->resize(batch);
+}
+
+void LConv::initialize(unsigned seed) {
+    glorot_uniform(cd->K, cd->kz * cd->kr * cd->kc, cd->nk * cd->kr * cd->kc, seed);
+    cd->bias->fill_(0.0f);
+}
+
+// ---------------------------------------------------------------- LBatchNorm
+LBatchNorm::LBatchNorm(Layer *p, float mom, float eps, bool aff, string n)
+    : Layer(n, "batchnorm"), momentum(mom), epsilon(eps), affine(aff) {
+    input = p->output;
+    if (input->ndim != 2 && input->ndim != 4)
+        std::cerr << "LBatchNorm only works over 1D or 2D tensors, however, we do not exit here and allow 3D tensors\n";
+    const vector<int> shape = {input->shape[1]};
+    output = new Tensor(input->getShape(), DEV_CPU);
+    opa = Tensor::zeros(input->getShape(), DEV_CPU);
+    extra.push_back(opa);
+    mean = Tensor::zeros(shape, DEV_CPU);
+    variance = Tensor::full(shape, momentum > 0.0f ? 0.0f : 1.0f, DEV_CPU);
+    bn_mean = new Tensor(shape, DEV_CPU);
+    bn_var = new Tensor(shape, DEV_CPU);
+    fixed.push_back(bn_mean);
+    fixed.push_back(bn_var);
+    if (affine) {
+        bn_g = Tensor::ones(shape, DEV_CPU);
+        bn_b = Tensor::zeros(shape, DEV_CPU);
+        params.push_back(bn_g);
+        params.push_back(bn_b);
+    }
+    params.push_back(mean);
+    params.push_back(variance);
+    p->addchild(this);
+    addparent(p);
+}
+
+void LBatchNorm::forward() {
+    tensorNN::BatchNormForward(input, output, opa, mean, variance, affine ? bn_g : nullptr, affine ? bn_b : nullptr, bn_mean, bn_var,
+                               mode == TRMODE, epsilon, momentum);
+}
+
+void LBatchNorm::initialize(unsigned) {
+    if (affine) {
+        bn_g->fill_(1.0f);
+        bn_b->fill_(0.0f);
+    }
+}
+
+// ---------------------------------------------------------------- LActivation
+LActivation::LActivation(Layer *p, string a, vector<float> prm, string n) : Layer(n, a), act(a), act_params(prm) {
+    if (act != "relu" && act != "sigmoid" && act != "softmax")
+        msg("activation " + act + " is outside the forward path this backend implements", "LActivation::LActivation");
+    input = p->output;
+    output = new Tensor(input->shape, DEV_CPU);
+    if (act == "softmax") {
+        if (act_params.empty()) {
+            act_params.push_back(-1);
+            std::cerr << "No axis for 'softmax' was specified. Using last one (-1) as default (LActivation::Softmax)\n";
+        }
+        if (act_params.size() > 1)
+            msg("Only one axis is supported (" + std::to_string(act_params.size()) + " were specified)", "LActivation::Softmax");
+        const int last = (int)input->shape.size() - 1;
+        if ((int)act_params[0] == -1) act_params[0] = (float)last;
+        if ((int)act_params[0] == 0) msg("The axis of a softmax must not be the batch", "LActivation::Softmax");
+        if ((int)act_params[0] < 0 || (int)act_params[0] > last)
+            msg("The axis has to be a number from 0 to (number_of_dimensions - 1)", "LActivation::Softmax");
+    }
+    p->addchild(this);
+    addparent(p);
+}
+
+void LActivation::forward() {
+    if (act == "relu") tensorNN::ReLu(input, output);
+    else if (act == "sigmoid") tensorNN::Sigmoid(input, output);
+    else tensorNN::FullSoftmax(input, output, (int)act_params[0]);
+}
+
+// ---------------------------------------------------------------- pools
+LPool::LPool(Layer *p, PoolDescriptor *D, const string &n, const string &prefix) : Layer(n, prefix), pd(D) {
+    if (p->output->ndim != 4) msg("LPool only works over 4D tensors", "LPool::LPool");
+    input = p->output;
+    pd->build(input);
+    output = pd->O;
+    p->addchild(this);
+    addparent(p);
+}
+
+LPool::~LPool() { delete pd; }
+
+void LPool::resize(int batch) {
+    pd->I = input;
+    pd->resize(batch);
+}
+
+void LMaxPool::make_indices() {
+    delete pd->indX;
+    delete pd->indY;
+    pd->indX = Tensor::zeros(pd->O->getShape(), pd->O->device);
+    pd->indY = Tensor::zeros(pd->O->getShape(), pd->O->device);
+}
+
+LMaxPool::LMaxPool(Layer *p, const vector<int> &pool_size, const vector<int> &strides, const string &padding, string n)
+    : LPool(p, new PoolDescriptor(pool_size, strides, padding, 0), n, "maxpool2d") {
+    make_indices();
+}
+
+LMaxPool::LMaxPool(Layer *p, const vector<int> &pool_size, const vector<int> &strides, const vector<int> &padding, string n)
+    : LPool(p, new PoolDescriptor(pool_size, strides, padding, 0), n, "maxpool2d") {
+    make_indices();
+}
+
+void LMaxPool::forward() { tensorNN::MPool2D(pd); }
+
+void LMaxPool::toGPU(int device) {
+    Layer::toGPU(device);
+    pd->indX->toGPU(device);
+    pd->indY->toGPU(device);
+}
+
+void LMaxPool::resize(int batch) {
+    LPool::resize(batch);
+    make_indices();  // the index tensors are re-created with the output (src/layers/pool/layer_maxpool.cpp:50-60)
+}
+
+LAveragePool::LAveragePool(Layer *p, const vector<int> &pool_size, const vector<int> &strides, const string &padding, string n)
+    : LPool(p, new PoolDescriptor(pool_size, strides, padding, 0), n, "avgpool") {}
+
+LAveragePool::LAveragePool(Layer *p, const vector<int> &pool_size, const vector<int> &strides, const vector<int> &padding, string n)
+    : LPool(p, new PoolDescriptor(pool_size, strides, padding, 0), n, "avgpool") {}
+
+void LAveragePool::forward() { tensorNN::AvgPool2D(pd); }
+
+// ---------------------------------------------------------------- LResize
+LResize::LResize(Layer *p, vector<int> ns, string n) : Layer(n, "resize"), new_shape(ns) {
+    input = p->output;
+    output = new Tensor({input->shape[0], input->shape[1], new_shape[0], new_shape[1]}, DEV_CPU);
+    p->addchild(this);
+    addparent(p);
+}
+
+void LResize::forward() {
+    // WrappingMode::Nearest = 2, TransformationMode::Asymmetric = 3 (include/eddl/utils.h:119-122)
+    Tensor::scale(input, output, new_shape, 2, 0.0f, 3);
+}
+
+// ---------------------------------------------------------------- merges
+LConcat::LConcat(vector<Layer *> ps, unsigned int ax, string n) : Layer(n, "concat") {
+    if (ps.empty()) msg("Error: LConcat layer with empty list");
+    if (ax == (unsigned)-1) ax = (ps[0]->output->ndim - 1) - 1;
+    axis = ax;  // batch is not included
+    if (ps.size() < 2) msg("Error: LConcat must receive at least two layers");
+    const unsigned nd = ps[0]->output->ndim;
+    if (axis + 1 >= nd) msg("The axis is out of range", "LConcat::LConcat");
+    for (size_t i = 0; i + 1 < ps.size(); i++)
+        if (nd != ps[i + 1]->output->ndim) msg("Error: LConcat layers with different tensor dims");
+    for (size_t i = 0; i + 1 < ps.size(); i++)
+        for (unsigned d = 0; d < nd; d++)
+            if (d != axis + 1 && ps[i]->output->shape[d] != ps[i + 1]->output->shape[d])
+                msg("Error: LConcat layers with different size in dim 1 (" + std::to_string(ps[i]->output->shape[d]) +
+                    "!=" + std::to_string(ps[i + 1]->output->shape[d]) + ")");
+    int t = 0;
+    for (Layer *p : ps) t += p->output->shape[axis + 1];
+    vector<int> ns = ps[0]->output->getShape();
+    ns[axis + 1] = t;
+    input = ps[0]->output;
+    output = new Tensor(ns, DEV_CPU);
+    for (Layer *p : ps) {
+        p->addchild(this);
+        addparent(p);
+    }
+}
+
+void LConcat::forward() {
+    vector<Tensor *> outs;
+    for (Layer *p : parent) outs.push_back(p->output);
+    Tensor::concat(outs, axis + 1, output);
+}
+
+LAdd::LAdd(vector<Layer *> ps, string n) : Layer(n, "add") {
+    if (ps.empty()) msg("Error: LAdd layer with empty list");
+    for (size_t i = 0; i + 1 < ps.size(); i++)
+        if (ps[i]->output->shape != ps[i + 1]->output->shape) msg("Error: LAdd layers with different tensor shape");
+    input = ps[0]->output;
+    output = new Tensor(ps[0]->output->shape, DEV_CPU);
+    for (Layer *p : ps) {
+        p->addchild(this);
+        addparent(p);
+    }
+}
+
+void LAdd::forward() {
+    output->fill_(0.0f);
+    for (Layer *p : parent) Tensor::inc(p->output, output);
+}
+
+LSum::LSum(Layer *l1, Layer *l2, string n) : Layer(n, "sum") {
+    if (l1->output->shape != l2->output->shape) msg("Error: LSum layers with different tensor shape", "LSum::LSum");
+    input = l1->output;
+    output = new Tensor(l1->output->shape, DEV_CPU);
+    l1->addchild(this);
+    l2->addchild(this);
+    addparent(l1);
+    addparent(l2);
+}
+
+void LSum::forward() { Tensor::add(1.0f, parent[0]->output, 1.0f, parent[1]->output, output, 0); }
+
+// ---------------------------------------------------------------- LPad
+LPad::LPad(Layer *p, vector<int> pads, float c, string n) : Layer(n, "pad"), constant(c) {
+    if (pads.size() == 2) padding = {pads[0], pads[1], pads[0], pads[1]};
+    else if (pads.size() == 4) padding = pads;
+    else msg("The padding on each border must follow this format (top-bottom, left-right) or (top, right, bottom, left)", "LPad::LPad");
+    input = p->output;
+    if (input->ndim != 4) msg("This method requires two 4D tensors", "LPad::LPad");
+    output = Tensor::full({input->shape[0], input->shape[1], input->shape[2] + (padding[0] + padding[2]),
+                           input->shape[3] + (padding[1] + padding[3])},
+                          constant, DEV_CPU);
+    p->addchild(this);
+    addparent(p);
+}
+
+void LPad::forward() { Tensor::pad(input, output, padding); }
+
+// the border is written when the tensor is created; forward() copies the interior only
+void LPad::resize(int batch) {
+    output->resize(batch);
+    output->fill_(constant);
+}
+
+void LPad::toGPU(int device) {
+    Layer::toGPU(device);
+    output->fill_(constant);
+}
+
+// ---------------------------------------------------------------- LReshape
+LReshape::LReshape(Layer *p, vector<int> shape, string n) : Layer(n, "reshape"), ls(shape) {
+    input = p->output;
+    ls[0] = input->shape[0];
+    const long tin = (long)input->size;
+    long t = 1;
+    int c = 0, ind = -1;
+    for (size_t i = 0; i < ls.size(); i++) {
+        if (ls[i] != -1) t *= ls[i];
+        else if (c) msg("Ambiguous reshape, more than one -1", "Reshape");
+        else {
+            c = 1;
+            ind = (int)i;
+        }
+    }
+    if (c == 1) {
+        if (t > tin || tin % t) msg("Incompatible shape", "Reshape");
+        ls[ind] = (int)(tin / t);
+    } else if (t != tin) {
+        msg("Incompatible shape", "Reshape");
+    }
+    output = new Tensor(ls, input);  // shares the parent's storage
+    p->addchild(this);
+    addparent(p);
+}
+
+LReshape::~LReshape() {}  // the view does not own its storage (Tensor::release skips shared tensors)
+
+void LReshape::resize(int batch) {
+    // the parent has been resized already (layers are walked in forward order)
+    ls[0] = batch;
+    Tensor *old = output;
+    output = new Tensor(ls, input);
+    delete old;
+    for (Layer *c : child) {  // children hold the tensor they read as `input`
+        if (c->input == old) c->input = output;
+    }
+}
+
+void LReshape::toGPU(int device) {
+    dev = device;
+    output->share(input);
+}
+
+// ---------------------------------------------------------------- LDense
+LDense::LDense(Layer *p, int nd, bool ub, string n) : Layer(n, "dense"), ndim(nd), use_bias(ub) {
+    input = p->output;
+    vector<int> outshape(input->shape.begin(), input->shape.end() - 1);
+    outshape.push_back(ndim);
+    output = new Tensor(outshape, DEV_CPU);
+    W = new Tensor(vector<int>{input->shape.back(), ndim}, DEV_CPU);
+    params.push_back(W);
+    if (use_bias) {
+        bias = new Tensor(vector<int>{ndim}, DEV_CPU);
+        params.push_back(bias);
+    }
+    p->addchild(this);
+    addparent(p);
+}
+
+void LDense::forward() {
+    const vector<int> inshape = input->shape, outshape = output->shape;
+    input->reshape_({(int)(input->size / input->shape.back()), input->shape.back()});
+    output->reshape_({(int)(output->size / output->shape.back()), output->shape.back()});
+    Tensor::mult2D(input, 0, W, 0, output, 0);
+    if (use_bias) Tensor::sum2D_rowwise(output, bias, output);
+    input->reshape_(inshape);
+    output->reshape_(outshape);
+}
+
+void LDense::initialize(unsigned seed) {
+    glorot_uniform(W, W->shape[0], W->shape[1], seed);
+    if (use_bias) bias->fill_(0.0f);
+}
+
+// ---------------------------------------------------------------- Net
+namespace {
+bool contains(const vector<Layer *> &v, Layer *l) {
+    for (Layer *x : v)
+        if (x == l) return true;
+    return false;
+}
+
+// Net::walk (src/net/net.cpp:231-245)
+void walk(Layer *l, const vector<Layer *> &lout, vector<Layer *> &seen) {
+    if (contains(seen, l)) return;
+    seen.push_back(l);
+    if (contains(lout, l)) return;
+    for (Layer *c : l->child) walk(c, lout, seen);
+}
+
+// Net::walk_back (src/net/net.cpp:248-258)
+void walk_back(Layer *l, vector<Layer *> &seen) {
+    if (contains(seen, l)) return;
+    seen.push_back(l);
+    for (Layer *p : l->parent) walk_back(p, seen);
+}
+}  // namespace
+
+Net::Net(const vector<Layer *> &in, const vector<Layer *> &out) : lin(in), lout(out) {
+    vector<Layer *> fwd, back;
+    for (Layer *l : lin) walk(l, lout, fwd);
+    for (Layer *l : lout) walk_back(l, back);
+    vector<Layer *> all = fwd;
+    for (Layer *l : back)
+        if (!contains(all, l)) all.push_back(l);
+    // Net::fts (src/net/net_build.cpp:34-70): always the first layer of the list whose parents are done
+    vector<int> pending(all.size(), 0), taken(all.size(), 0);
+    for (size_t i = 0; i < all.size(); i++)
+        for (Layer *p : all[i]->parent)
+            if (contains(all, p)) pending[i]++;
+    for (size_t n = 0; n < all.size(); n++) {
+        size_t j = 0;
+        while (j < all.size() && !(pending[j] == 0 && !taken[j])) j++;
+        if (j == all.size()) msg("error recurrent net", "Net.fts");
+        taken[j] = 1;
+        layers.push_back(all[j]);
+        for (Layer *c : all[j]->child)
+            for (size_t k = 0; k < all.size(); k++)
+                if (all[k] == c) pending[k]--;
+    }
+    for (Layer *l : layers) l->net = this;
+}
+
+Net::~Net() {
+    // an LInput's input and output are one tensor; LReshape outputs are views: both are handled by
+    // the layers' destructors.  Layers are deleted children first so that views go before their base.
+    for (size_t i = layers.size(); i-- > 0;) delete layers[i];
+    delete cs;
+}
+
+void Net::build(CompServ *service, bool init_weights) {
+    if (cs != nullptr) msg("the net has been built already", "Net::build");
+    cs = service;
+    int device = -1, count = 0;
+    for (size_t i = 0; i < cs->local_gpus.size(); i++)
+        if (cs->local_gpus[i]) {
+            if (device < 0) device = (int)i;
+            count++;
+        }
+    if (count == 0) msg("the computing service names no GPU", "Net::build");
+    if (count > 1) msg("this backend runs a net on one GPU; the computing service names " + std::to_string(count), "Net::build");
+    if (device >= gpu_devices()) msg("GPU " + std::to_string(device) + " is not present", "Net::build");
+    gpu_init(device);
+    if (init_weights) {
+        unsigned seed = 1;
+        for (Layer *l : layers) l->initialize(seed++);
+    }
+    dev = DEV_GPU + device;
+    for (Layer *l : layers) l->toGPU(dev);
+}
+
+void Net::resize(int batch) {
+    if (batch == batch_size) return;
+    batch_size = batch;
+    for (Layer *l : layers) l->resize(batch);
+}
+
+void Net::setmode(int m) {
+    for (Layer *l : layers) l->setmode(m);
+}
+
+void Net::forward() {
+    for (Layer *l : layers) l->forward();
+}
+
+void Net::forward(const vector<Tensor *> &in) {
+    if (dev == DEV_CPU) msg("build the net with a computing service first", "Net.forward(vtensor)");
+    if (!in.empty()) {
+        if (in.size() != lin.size()) msg("size missmatch in list of tensors", "Net.forward(vtensor)");
+        if (batch_size != in[0]->shape[0]) resize(in[0]->shape[0]);
+        for (size_t i = 0; i < in.size(); i++) Tensor::copy(in[i], lin[i]->output);
+    }
+    forward();
+}
+
+vector<Tensor *> Net::predict(const vector<Tensor *> &in) {
+    setmode(TSMODE);
+    forward(in);
+    vector<Tensor *> out;
+    for (Layer *l : lout) {
+        Tensor *t = new Tensor(l->output->getShape(), DEV_CPU);
+        Tensor::copy(l->output, t);
+        out.push_back(t);
+    }
+    return out;
+}
+
+// "bin" files: for every layer in `layers` order, for every parameter in the layer's order,
+// int32 ndim | int32 shape[ndim] | float32 data (src/net/net.cpp:411-449, src/layers/layer.cpp:215-227,
+// src/tensor/tensor_serialization.cpp:70-110,252-261)
+void Net::save(const string &filename, const string &format) {
+    if (format != "bin") msg("Format not implemented: *.'" + format + "'", "Tensor::save");
+    std::ofstream ofs(filename, std::ios::out | std::ios::binary);
+    for (Layer *l : layers)
+        for (Tensor *p : l->params) {
+            Tensor host(p->getShape(), DEV_CPU);
+            Tensor::copy(p, &host);
+            int nd = (int)host.ndim;
+            ofs.write(reinterpret_cast<const char *>(&nd), sizeof(int));
+            ofs.write(reinterpret_cast<const char *>(host.shape.data()), host.shape.size() * sizeof(int));
+            ofs.write(reinterpret_cast<const char *>(host.ptr), host.size * sizeof(float));
+        }
+}
+
+void Net::load(const string &filename, const string &format) {
+    if (format != "bin") msg("Format not implemented: *.'" + format + "'", "Tensor::load");
+    std::ifstream ifs(filename, std::ios::in | std::ios::binary);
+    if (!ifs.good()) throw std::runtime_error(string("File not found. Check the file name and try again (Net::load)"));
+    for (Layer *l : layers)
+        for (Tensor *p : l->params) {
+            int nd = 0;
+            ifs.read(reinterpret_cast<char *>(&nd), sizeof(int));
+            if (!ifs.good() || nd < 0 || nd > 8) msg("the file ends early or is not in the bin format (layer " + l->name + ")", "Net::load");
+            vector<int> shape(nd);
+            ifs.read(reinterpret_cast<char *>(shape.data()), nd * sizeof(int));
+            Tensor host(shape, DEV_CPU);
+            ifs.read(reinterpret_cast<char *>(host.ptr), host.size * sizeof(float));
+            if (!ifs.good()) msg("the file ends inside a parameter of layer " + l->name, "Net::load");
+            Tensor::copy(&host, p);  // any shape of the same size, as the reference's copy accepts
+        }
+}
+
+string Net::summary(bool print_stdout) {
+    std::stringstream ss;
+    ss << "-------------------------------------------------------------------------------\n" << name << "\n";
+    ss << "-------------------------------------------------------------------------------\n";
+    size_t maxl = 0;
+    for (Layer *l : layers) maxl = std::max(maxl, l->name.size());
+    long total = 0;
+    for (Layer *l : layers) {
+        long np = 0;
+        for (Tensor *p : l->params) np += (long)p->size;
+        total += np;
+        auto shp = [](const vector<int> &s) {
+            string r = "(";
+            for (size_t i = 1; i < s.size(); i++) r += (i > 1 ? ", " : "") + std::to_string(s[i]);
+            return r + ")";
+        };
+        ss << std::setw((int)maxl) << std::left << l->name << "|  " << std::setw(20) << shp(l->input->shape) << "=>   " << std::setw(20)
+           << shp(l->output->shape) << std::setw(12) << np << "\n";
+    }
+    ss << "-------------------------------------------------------------------------------\n";
+    ss << "Total params: " << total << "\n";
+    if (print_stdout) std::cout << ss.str();
+    return ss.str();
+}
+
+// ---------------------------------------------------------------- eddl:: API
+namespace eddl {
+
+model Model(vlayer in, vlayer out) { return new Net(in, out); }
+void setName(model m, string name) { m->name = name; }
+
+compserv CS_HIP(const vector<int> &g, const string &mem) {
+    CompServ *cs = new CompServ();
+    cs->local_gpus = g;
+    cs->mem = mem;
+    return cs;
+}
+compserv CS_GPU(const vector<int> &g, const string &mem) { return CS_HIP(g, mem); }
+
+void build(model net, compserv cs, bool init_weights) { net->build(cs, init_weights); }
+void set_mode(model net, int mode) { net->setmode(mode); }
+void summary(model m) { m->summary(true); }
+void load(model m, const string &fname, const string &format) { m->load(fname, format); }
+void save(model m, const string &fname, const string &format) { m->save(fname, format); }
+
+vlayer forward(model m, vtensor in) {
+    m->forward(in);
+    return m->lout;
+}
+
+vtensor predict(model m, const vtensor &in) { return m->predict(in); }
+
+Tensor *getOutput(layer l1) {
+    Tensor *t = new Tensor(l1->output->getShape(), DEV_CPU);
+    Tensor::copy(l1->output, t);
+    return t;
+}
+
+layer Input(const vector<int> &shape, string name) {
+    vector<int> s(shape);
+    s.insert(s.begin(), 1);  // batch 1 until a forward says otherwise (src/apis/eddl.cpp:604-608)
+    return new LInput(new Tensor(s, DEV_CPU), name);
+}
+
+layer Conv2D(layer parent, int filters, const vector<int> &kernel_size, const vector<int> &strides, string padding, bool use_bias,
+             int groups, const vector<int> &dilation_rate, string name) {
+    return new LConv(parent, filters, kernel_size, strides, padding, {}, groups, dilation_rate, use_bias, name);
+}
+
+layer Dense(layer parent, int ndim, bool use_bias, string name) { return new LDense(parent, ndim, use_bias, name); }
+
+layer Activation(layer parent, string activation, vector<float> params, string name) {
+    return new LActivation(parent, activation, params, name);
+}
+layer ReLu(layer parent, string name) { return new LActivation(parent, "relu", {}, name); }
+layer Sigmoid(layer parent, string name) { return new LActivation(parent, "sigmoid", {}, name); }
+layer Softmax(layer parent, int axis, string name) { return new LActivation(parent, "softmax", {(float)axis}, name); }
+
+layer BatchNormalization(layer parent, float momentum, float epsilon, bool affine, string name) {
+    return new LBatchNorm(parent, momentum, epsilon, affine, name);
+}
+layer BatchNormalization(layer parent, bool affine, float momentum, float epsilon, string name) {
+    return new LBatchNorm(parent, momentum, epsilon, affine, name);
+}
+
+layer MaxPool2D(layer parent, vector<int> pool_size, vector<int> strides, string padding, string name) {
+    return new LMaxPool(parent, pool_size, strides, padding, name);
+}
+layer AveragePool2D(layer parent, vector<int> pool_size, vector<int> strides, string padding, string name) {
+    return new LAveragePool(parent, pool_size, strides, padding, name);
+}
+layer AvgPool2D(layer parent, vector<int> pool_size, vector<int> strides, string padding, string name) {
+    return AveragePool2D(parent, pool_size, strides, padding, name);
+}
+layer GlobalAveragePool2D(layer parent, string name) {
+    if (parent->output->ndim != 4) msg("GlobalAveragePool only works over 4D tensors", "GlobalAveragePool2D");
+    if (name.empty()) name = "GlobalAveragePool2D";
+    return AveragePool2D(parent, {parent->output->shape[2], parent->output->shape[3]}, {1, 1}, "none", name);
+}
+
+layer UpSampling2D(layer parent, const vector<int> &size, string interpolation, string name) {
+    if (interpolation != "nearest")
+        std::cerr << "Warning: In UpSampling2D the interpolation type \"" << interpolation
+                  << "\" is not valid. Only \"nearest\" is available.\n";
+    const vector<int> ps = parent->output->getShape();
+    if (ps.size() != 4) msg("The number of dimensions of the input tensor must be 4", "EDDL::UpSampling2D");
+    if (size.size() != 2) msg("The number of dimensions of the \"size\" parameter must be 2", "EDDL::UpSampling2D");
+    vector<int> target;
+    for (int i : {2, 3}) {
+        if (size[i - 2] < 1) msg("The scale factors in \"size\" parameter must be greater or equal to 1", "EDDL::UpSampling2D");
+        target.push_back(ps[i] * size[i - 2]);
+    }
+    return new LResize(parent, target, name);
+}
+
+layer Concat(const vector<layer> &layers, unsigned int axis, string name) { return new LConcat(layers, axis, name); }
+layer Add(const vector<layer> &layers, string name) { return new LAdd(layers, name); }
+layer Add(layer l1, layer l2) { return new LSum(l1, l2, ""); }
+layer Pad(layer parent, vector<int> padding, float constant, string name) { return new LPad(parent, padding, constant, name); }
+
+layer Reshape(layer parent, const vector<int> &shape, string name) {
+    vector<int> s(shape);
+    s.insert(s.begin(), 1);
+    return new LReshape(parent, s, name);
+}
+layer Flatten(layer parent, string name) { return Reshape(parent, {-1}, name); }
+
+}  // namespace eddl
+}  // namespace eddl_hip

@@ -78,7 +78,8 @@ def BatchNormalization(parent, affine=True, momentum=0.99, epsilon=1e-3, name=""
         l.params["bn_g"] = np.ones(C, np.float32)
         l.params["bn_b"] = np.zeros(C, np.float32)
     l.params["mean"] = np.zeros(C, np.float32)
-    l.params["variance"] = np.ones(C, np.float32)
+    # the running variance starts at 0 when momentum > 0 (layer_batchnorm.cpp:51-56)
+    l.params["variance"] = np.zeros(C, np.float32) if momentum > 0.0 else np.ones(C, np.float32)
     return l
 
 

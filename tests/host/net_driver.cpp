@@ -1,0 +1,201 @@
+// Model-level test driver of the C++ host layer: builds one of the benchmark graphs with the
+// eddl:: API (the same constructions, in the same order, as eddl_amd/models.py), loads its
+// parameters from a "bin" file, runs predict on an input read from a raw float file and writes
+// the outputs to another.  The Python test compares the result with the Python graph runner on
+// the same parameters, bit for bit.
+//
+// usage: net_driver <block|vgg16|resnet50|unet> <params.bin|-> <input.raw> <output.raw> <batch> <size> [model arguments]
+//        net_driver errors
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+
+#include "eddl_hip_net.h"
+
+using namespace eddl_hip;
+using namespace eddl_hip::eddl;
+
+static layer bn(layer l) { return BatchNormalization(l, true, 0.99f, 1e-5f); }
+
+static model block(int channels, int size, int filters) {
+    layer x = Input({channels, size, size});
+    layer l = Conv2D(x, filters, {3, 3}, {1, 1}, "same", false);
+    l = MaxPool2D(ReLu(bn(l)), {2, 2}, {2, 2}, "none");
+    return Model({x}, {l});
+}
+
+static model vgg16(int size, int num_classes, const vector<int> &widths, int dense) {
+    layer x = Input({3, size, size});
+    layer l = x;
+    const int reps[5] = {2, 2, 3, 3, 3};
+    for (int s = 0; s < 5; s++) {
+        for (int r = 0; r < reps[s]; r++) l = ReLu(Conv2D(l, widths[s], {3, 3}, {1, 1}, "same", true));
+        l = MaxPool2D(l, {2, 2}, {2, 2}, "none");
+    }
+    l = Flatten(l);
+    l = ReLu(Dense(l, dense));
+    l = ReLu(Dense(l, dense));
+    l = Softmax(Dense(l, num_classes));
+    return Model({x}, {l});
+}
+
+static model resnet50(int size, int num_classes, int base) {
+    const int stages[4] = {3, 4, 6, 3};
+    layer x = Input({3, size, size});
+    layer l = ReLu(bn(new LConv(x, base, {7, 7}, {2, 2}, "custom", {3, 3, 3, 3}, 1, {1, 1}, false, "")));
+    l = new LMaxPool(l, vector<int>{3, 3}, vector<int>{2, 2}, vector<int>{1, 1, 1, 1}, "");
+    int width = base;
+    for (int si = 0; si < 4; si++) {
+        for (int bi = 0; bi < stages[si]; bi++) {
+            const int stride = (bi == 0 && si > 0) ? 2 : 1;
+            const int out_ch = width * 4;
+            layer sc = l;
+            if (bi == 0) sc = bn(Conv2D(l, out_ch, {1, 1}, {stride, stride}, "valid", false));
+            layer m = ReLu(bn(Conv2D(l, width, {1, 1}, {1, 1}, "valid", false)));
+            if (stride == 1) m = Conv2D(m, width, {3, 3}, {1, 1}, "same", false);
+            else m = new LConv(m, width, {3, 3}, {2, 2}, "custom", {1, 1, 1, 1}, 1, {1, 1}, false, "");
+            m = ReLu(bn(m));
+            m = bn(Conv2D(m, out_ch, {1, 1}, {1, 1}, "valid", false));
+            l = ReLu(Add(m, sc));
+        }
+        width *= 2;
+    }
+    l = Dense(Flatten(GlobalAveragePool2D(l)), num_classes);
+    return Model({x}, {l});
+}
+
+static layer twice(layer l, int w) {
+    for (int i = 0; i < 2; i++) l = ReLu(bn(Conv2D(l, w, {3, 3}, {1, 1}, "same", true)));
+    return l;
+}
+
+static model unet(int size, const vector<int> &widths, int bottleneck) {
+    layer x = Input({1, size, size});
+    layer l = x;
+    vector<layer> skips;
+    for (int w : widths) {
+        l = twice(l, w);
+        skips.push_back(l);
+        l = MaxPool2D(l, {2, 2}, {2, 2}, "none");
+    }
+    l = twice(l, bottleneck);
+    for (size_t i = widths.size(); i-- > 0;) {
+        l = UpSampling2D(l, {2, 2});
+        l = Conv2D(Pad(l, {0, 1, 1, 0}), widths[i], {2, 2}, {1, 1}, "valid", true);
+        l = Concat({skips[i], l});
+        l = twice(l, widths[i]);
+    }
+    l = Sigmoid(Conv2D(l, 1, {1, 1}, {1, 1}, "valid", true));
+    return Model({x}, {l});
+}
+
+template <class F>
+static bool throws(F f, const char *what) {
+    try {
+        f();
+    } catch (const std::exception &e) {
+        printf("ok %s: %s\n", what, e.what());
+        return true;
+    }
+    printf("FAILED %s: no exception\n", what);
+    return false;
+}
+
+static int errors() {
+    bool ok = true;
+    ok &= throws([] { Conv2D(Input({3, 224, 224}), 64, {7, 7}, {2, 2}, "same"); }, "asymmetric 7x7 s2 same");
+    try {
+        Conv2D(Input({3, 8, 8}), 4, {2, 2}, {1, 1}, "same");
+        ok = false;
+    } catch (const AsymmetricPaddingException &e) {
+        vector<int> p = e.get_asymmetric_pads();
+        printf("ok asymmetric pads %d %d %d %d\n", p[0], p[1], p[2], p[3]);
+        ok &= p == vector<int>({0, 1, 0, 1});
+    }
+    ok &= throws([] { Dense(Input({4}), 3)->forward(); }, "forward before build");
+    ok &= throws([] { Reshape(Input({4, 4}), {-1, -1}); }, "ambiguous reshape");
+    ok &= throws([] { Reshape(Input({4, 4}), {5}); }, "incompatible reshape");
+    ok &= throws([] { Concat({Input({4, 4, 4})}); }, "concat of one layer");
+    ok &= throws([] { Concat({Input({4, 4, 4}), Input({4, 5, 4})}); }, "concat of different planes");
+    ok &= throws([] { Add(Input({4, 4, 4}), Input({4, 5, 4})); }, "add of different shapes");
+    ok &= throws([] { Softmax(Input({4}), 0); }, "softmax over the batch");
+    ok &= throws([] { Activation(Input({4}), "elu"); }, "activation outside the path");
+    ok &= throws([] {
+        model m = block(3, 8, 4);
+        build(m, CS_HIP({1, 1}));
+    }, "two GPUs");
+    ok &= throws([] {
+        model m = block(3, 8, 4);
+        build(m, CS_HIP({1}));
+        load(m, "/nonexistent/file.bin");
+    }, "missing parameter file");
+    ok &= throws([] {
+        model m = block(3, 8, 4);
+        build(m, CS_HIP({1}));
+        Tensor a({2, 3, 8, 8}), b({2, 3, 8, 8});
+        predict(m, {&a, &b});
+    }, "two inputs for one input layer");
+    return ok ? 0 : 1;
+}
+
+int main(int argc, char **argv) {
+    if (argc >= 2 && !strcmp(argv[1], "errors")) return errors();
+    if (argc < 7) {
+        fprintf(stderr, "usage: net_driver <model> <params.bin|-> <input.raw> <output.raw> <batch> <size> [model arguments]\n");
+        return 2;
+    }
+    const string which = argv[1], params = argv[2], in_path = argv[3], out_path = argv[4];
+    const int batch = atoi(argv[5]), size = atoi(argv[6]);
+    vector<int> extra;
+    for (int i = 7; i < argc; i++) extra.push_back(atoi(argv[i]));
+    try {
+        model m = nullptr;
+        if (which == "block") m = block(extra.at(0), size, extra.at(1));
+        else if (which == "vgg16") m = vgg16(size, extra.at(0), {extra.at(1), extra.at(2), extra.at(3), extra.at(4), extra.at(5)}, extra.at(6));
+        else if (which == "resnet50") m = resnet50(size, extra.at(0), extra.at(1));
+        else if (which == "unet") m = unet(size, vector<int>(extra.begin(), extra.end() - 1), extra.back());
+        else {
+            fprintf(stderr, "unknown model %s\n", which.c_str());
+            return 2;
+        }
+        build(m, CS_HIP({1}));
+        if (params != "-") load(m, params);
+        printf("layers:");
+        for (Layer *l : m->layers) printf(" %s", l->kind().c_str());
+        printf("\n");
+        vector<int> ishape = m->lin[0]->output->getShape();
+        ishape[0] = batch;
+        Tensor x(ishape, DEV_CPU);
+        std::ifstream ifs(in_path, std::ios::binary);
+        ifs.read(reinterpret_cast<char *>(x.ptr), x.size * sizeof(float));
+        if (!ifs.good()) {
+            fprintf(stderr, "short input file\n");
+            return 2;
+        }
+        // two forwards at two batch sizes first: every tensor is re-created on the way (resize)
+        if (batch > 1) {
+            vector<int> one = ishape;
+            one[0] = 1;
+            Tensor x1(one, DEV_CPU);
+            memcpy(x1.ptr, x.ptr, x1.size * sizeof(float));
+            for (Tensor *t : predict(m, {&x1})) delete t;
+        }
+        vtensor out = predict(m, {&x});
+        std::ofstream ofs(out_path, std::ios::binary);
+        for (Tensor *t : out) {
+            printf("output");
+            for (int d : t->shape) printf(" %d", d);
+            printf("\n");
+            ofs.write(reinterpret_cast<const char *>(t->ptr), t->size * sizeof(float));
+            delete t;
+        }
+        if (params == "-") save(m, out_path + ".params");  // round trip of freshly initialised parameters
+        delete m;
+    } catch (const std::exception &e) {
+        fprintf(stderr, "exception: %s\n", e.what());
+        return 1;
+    }
+    return 0;
+}

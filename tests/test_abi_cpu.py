@@ -99,5 +99,10 @@ def test_host_layer_links_against_the_c_abi():
         subprocess.run(["make", "-C", host, "all"], check=True, stdout=subprocess.DEVNULL)
     h = ctypes.CDLL(lib)
     for sym in ("_ZN8eddl_hip10gpu_conv2DEPNS_16ConvolDescriptorE", "_ZN8eddl_hip8tensorNN6Conv2DEPNS_16ConvolDescriptorE",
-                "_ZN8eddl_hip11gpu_mpool2DEPNS_14PoolDescriptorE", "_ZN8eddl_hip8gpu_reluEPNS_6TensorES1_"):
+                "_ZN8eddl_hip11gpu_mpool2DEPNS_14PoolDescriptorE", "_ZN8eddl_hip8gpu_reluEPNS_6TensorES1_",
+                # the model-building API: eddl::Model, eddl::Conv2D, eddl::predict, Net::load
+                "_ZN8eddl_hip4eddl5ModelESt6vectorIPNS_5LayerESaIS3_EES5_",
+                "_ZN8eddl_hip4eddl6Conv2DEPNS_5LayerEiRKSt6vectorIiSaIiEES7_NSt7__cxx1112basic_stringIcSt11char_traitsIcESaIcEEEbiS7_SD_",
+                "_ZN8eddl_hip4eddl7predictEPNS_3NetERKSt6vectorIPNS_6TensorESaIS5_EE",
+                "_ZN8eddl_hip3Net4loadERKNSt7__cxx1112basic_stringIcSt11char_traitsIcESaIcEEES8_"):
         assert hasattr(h, sym), sym
