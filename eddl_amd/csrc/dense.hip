@@ -69,12 +69,13 @@ __global__ __launch_bounds__(64) void dense_partial_kernel(const float *__restri
         }
         return b;
     };
+    constexpr int U = 8;
     int kk = kbeg;
-    for (; kk + 8 <= kend; kk += 8) {  // four k pairs in flight
-        float a[4];
-        floatx4 b[4];
+    for (; kk + 2 * U <= kend; kk += 2 * U) {  // U k pairs (U float4 of weights per lane) in flight
+        float a[U];
+        floatx4 b[U];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < U; u++) {
             const int ki = kk + 2 * u + half;
             a[u] = ap[(size_t)ki * 32];
             const float *row = B + (size_t)ki * n;
@@ -85,7 +86,7 @@ __global__ __launch_bounds__(64) void dense_partial_kernel(const float *__restri
             }
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < U; u++) {
             acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].x, acc[0], 0, 0, 0);
             acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].y, acc[1], 0, 0, 0);
             acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].z, acc[2], 0, 0, 0);
