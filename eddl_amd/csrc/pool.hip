@@ -60,6 +60,51 @@ __global__ __launch_bounds__(TPB) void maxpool_kernel(const float *__restrict__ 
     }
 }
 
+// Window shape known at compile time (3x3 here): the KR*KC loads of an output are independent and all
+// issued before the first comparison; a tap outside the image reads -FLT_MAX, which is below the
+// running maximum's start value and so never wins - the reference's own rule (cpu_pool.cpp:20-30).
+template <int KR, int KC>
+__global__ __launch_bounds__(TPB) void maxpool_window_kernel(const float *__restrict__ I, float *__restrict__ O,
+                                                             float *__restrict__ indX, float *__restrict__ indY, size_t total,
+                                                             PoolShape s) {
+    size_t t0 = (size_t)blockIdx.x * TPB + threadIdx.x, stride = (size_t)gridDim.x * TPB;
+    for (size_t p = t0; p < total; p += stride) {
+        const int oj = (int)(p % s.LQ);
+        const size_t r = p / s.LQ;
+        const int oi = (int)(r % s.LP);
+        const size_t plane = r / s.LP;
+        const float *img = I + plane * s.H * s.W;
+        const int i = oi * s.sr - s.pt, j = oj * s.sc - s.pl;
+        float v[KR][KC];
+#pragma unroll
+        for (int ki = 0; ki < KR; ki++)
+#pragma unroll
+            for (int kj = 0; kj < KC; kj++) {
+                const int py = i + ki, px = j + kj;
+                const bool in = (unsigned)py < (unsigned)s.H && (unsigned)px < (unsigned)s.W;
+                v[ki][kj] = in ? img[py * s.W + px] : -3.402823466e+38f;
+            }
+        float mx = LOWEST;
+        int bx = 0, by = 0;
+        bool found = false;
+#pragma unroll
+        for (int ki = 0; ki < KR; ki++)
+#pragma unroll
+            for (int kj = 0; kj < KC; kj++)
+                if (v[ki][kj] > mx) {
+                    mx = v[ki][kj];
+                    bx = j + kj;
+                    by = i + ki;
+                    found = true;
+                }
+        O[p] = mx;
+        if (found) {
+            indX[p] = (float)bx;
+            indY[p] = (float)by;
+        }
+    }
+}
+
 // 2x2 window, stride 2, no padding, even W, 16-byte aligned rows: each thread reads a float4
 // from two consecutive input rows and writes two outputs (float2 stores).
 __global__ __launch_bounds__(TPB) void maxpool_2x2s2_kernel(const float *__restrict__ I, float *__restrict__ O,
@@ -228,6 +273,9 @@ int eddlhip_maxpool2d(int dev, const float *I, float *O, float *indX, float *ind
         size_t pairs = total / 2;
         hipLaunchKernelGGL(maxpool_2x2s2_kernel, dim3(eh_blocks(pairs, TPB, 1u << 18)), dim3(TPB), 0, st, I, O, indX, indY, pairs, H,
                            W, s.LP, s.LQ);
+    } else if (kr == 3 && kc == 3 && (long long)H * W < (1LL << 31)) {
+        hipLaunchKernelGGL((maxpool_window_kernel<3, 3>), dim3(eh_blocks(total, TPB, 1u << 18)), dim3(TPB), 0, st, I, O, indX, indY,
+                           total, s);
     } else if (kr * kc >= 64) {
         hipLaunchKernelGGL(maxpool_wave_kernel, dim3(eh_blocks(total, TPB / 64, 1u << 18)), dim3(TPB), 0, st, I, O, indX, indY, total,
                            s);
