@@ -1,0 +1,44 @@
+"""bench.py pieces that need no GPU: the refusal of more than one GPU, the workload table (FLOP
+counts of the four configurations against the figures the survey of the reference gives), and
+the CPU-baseline leg on a tiny sample."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+
+from conftest import ROOT
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                         text=True, timeout=120)
+    assert res.returncode != 0 and "ONE GPU" in res.stderr and res.stdout.strip() == ""
+
+
+def test_workload_flops_match_the_configurations():
+    sys.path.insert(0, ROOT)
+    import bench
+    from eddl_amd import models
+    want = {"vgg16": 982.18e9, "resnet50": 523.15e9, "unet": 1745.1e9, "block": 14.797e9}
+    builders = {"vgg16": models.vgg16, "block": models.conv_bn_relu_pool_block, "resnet50": models.resnet50, "unet": models.unet}
+    for name, (kwargs, seed, dist, desc) in bench.WORKLOADS.items():
+        m = builders[name](**kwargs)
+        flops = 0
+        for l in m.layers:
+            if l.kind == "conv2d":
+                cd = l.attrs["cd"]
+                N, Kf, P, Q = cd.out_shape
+                flops += 2 * N * Kf * cd.kz * cd.kr * cd.kc * P * Q
+        assert abs(flops - want[name]) / want[name] < 2e-3, (name, flops)
+
+
+def test_cpu_baseline_leg_runs_on_a_small_sample(monkeypatch):
+    sys.path.insert(0, ROOT)
+    import bench
+    monkeypatch.setitem(bench.WORKLOADS, "block", ({"batch": 2, "channels": 4, "size": 8, "filters": 4}, 2, "normal", "tiny block"))
+    out = bench.cpu_baseline("block", want_seconds=0.2)
+    assert out["kind"] == "port" and out["unit"] == "images/sec" and out["cores"] >= 1
+    assert out["value"] > 0 and out["value_strict"] > 0 and "sample" in out
+    json.dumps(out)
