@@ -138,6 +138,14 @@ __device__ __forceinline__ void lds_dma_b32(int32x4 rsrc, lds_float *dst, int vo
                  : "memory");
 }
 
+// 16 bytes per lane: lane l's four floats land at dst + 4*l .. 4*l + 3 (1 KB per wavefront instruction)
+__device__ __forceinline__ void lds_dma_b128(int32x4 rsrc, lds_float *dst, int voffset, int soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"((unsigned)(unsigned long long)dst), "v"(voffset), "s"(rsrc), "s"(soffset)
+                 : "memory");
+}
+
 __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, int voffset, int soffset) {
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voffset, soffset, 0));
 }
@@ -375,15 +383,17 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     floatx4 areg[DIRECT ? 1 : AV];
     float breg[DIRECT ? 1 : CPW * RS];
 
-    // LDS-direct filter slice: a wavefront instruction moves 64 consecutive floats of the slice in LDS:
-    // one 64-float segment of a row (BM >= 64, BM/64 segments per row) or two whole rows (BM = 32).
-    // Unit u of the slice belongs to wavefront u % 4.
-    constexpr int A_SEGS = BM >= 64 ? BM / 64 : 1;
-    constexpr int A_UNITS = BM >= 64 ? BK * A_SEGS : BK / 2;
+    // LDS-direct filter slice: a wavefront instruction moves 256 consecutive floats of the slice in LDS
+    // (16 bytes per lane), i.e. RPI = 256 / BM whole rows; unit u (rows u*RPI ...) belongs to wavefront
+    // u % 4.  The last unit may reach past the slice: it then reads rows of the next step (or zeros
+    // past the end of the packed matrix, which the buffer descriptor bounds) into the parking area
+    // behind the slice.
+    constexpr int RPI = 256 / BM;
+    constexpr int A_UNITS = (BK + RPI - 1) / RPI;
     constexpr int A_UPW = (A_UNITS + 3) / 4;
+    static_assert((RPI - 1) * BM <= 256, "the parking area holds the surplus rows of the last unit");
     const int32x4 dma_w = make_rsrc_words(p.Wp, p.wp_bytes), dma_in = make_rsrc_words(p.I, p.in_bytes);
-    // BM = 32: lanes 32..63 fetch the next row of the packed matrix (one row further = Mp floats)
-    const int a_voff_direct = BM >= 64 ? (m0 + lane) * 4 : (m0 + (lane & 31) + (lane >> 5) * p.Mp) * 4;
+    const int a_voff_direct = ((lane / (BM / 4)) * p.Mp + m0 + 4 * (lane % (BM / 4))) * 4;
 
     auto load_a = [&](int step, lds_float *as) {
         if constexpr (DIRECT) {
@@ -391,8 +401,8 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
             for (int j = 0; j < A_UPW; j++) {
                 const int u = wave + 4 * j;
                 if (A_UNITS % 4 == 0 || j < A_UPW - 1 || u < A_UNITS) {  // uniform in the wavefront
-                    const int kk = BM >= 64 ? u / A_SEGS : 2 * u, sg = BM >= 64 ? u % A_SEGS : 0;
-                    lds_dma_b32(dma_w, as + kk * LDA + sg * 64, a_voff_direct, ((step * BK + kk) * p.Mp + sg * 64) * 4);
+                    const int kk = u * RPI;
+                    lds_dma_b128(dma_w, as + kk * LDA, a_voff_direct, (step * BK + kk) * p.Mp * 4);
                 }
             }
         } else {
