@@ -25,14 +25,24 @@ void msg(const string &text, const string &title) {
 // A failed C ABI call becomes the reference's device-error exception
 // (check_cuda throws std::runtime_error("[CUDA ERROR]: ..."), src/hardware/gpu/gpu_tensor.cu:103-112);
 // a rejected argument becomes a msg().
-static void check(int rc, const char *where) {
+void gpu_check(int rc, const char *where) {
     if (rc == 0) return;
     string text = eddlhip_last_error();
     if (rc == EDDLHIP_EINVAL) msg(text, where);
     throw std::runtime_error(string("[HIP ERROR]: ") + text + " (" + where + ")");
 }
 
-static void sync(int gpu_device) { check(eddlhip_synchronize(gpu_device), "gpu_synchronize"); }
+static void check(int rc, const char *where) { gpu_check(rc, where); }
+
+static bool g_synchronous = true;
+
+void gpu_set_synchronous(bool on) { g_synchronous = on; }
+bool gpu_get_synchronous() { return g_synchronous; }
+void gpu_synchronize(int gpu_device) { check(eddlhip_synchronize(gpu_device), "gpu_synchronize"); }
+
+static void sync(int gpu_device) {
+    if (g_synchronous) gpu_synchronize(gpu_device);
+}
 
 // ---------------------------------------------------------------- runtime
 static bool g_init[16] = {false};

@@ -12,7 +12,9 @@
 //                       tensor_bn.cpp:93-129, tensor_activations.cpp:47-65,345-360,567-585
 //   msg()               src/utils.cpp:57-67 (banner on stderr, then std::runtime_error("RuntimeError: " + title))
 // Every gpu_* function here is synchronous on return, as the reference's wrappers are
-// (they call cudaDeviceSynchronize after each launch, e.g. src/hardware/gpu/nn/gpu_pool.cu:27-33).
+// (they call cudaDeviceSynchronize after each launch, e.g. src/hardware/gpu/nn/gpu_pool.cu:27-33),
+// unless gpu_set_synchronous(false) has been called: then compute calls return once queued on the
+// device's stream, in order, and copies to the host still wait for everything queued before them.
 // Everything lives in namespace eddl_hip so that it can be linked next to EDDL itself.
 #pragma once
 #include <string>
@@ -128,6 +130,10 @@ class PoolDescriptor {
 
 // ---- the backend seam: same signatures as the reference's gpu_* declarations
 void gpu_init(int device);
+void gpu_set_synchronous(bool on);      // no counterpart in the reference: see the note at the top
+bool gpu_get_synchronous();
+void gpu_synchronize(int gpu_device);   // waits for everything queued on the device
+void gpu_check(int rc, const char *where);  // a C ABI return code -> the reference's exceptions
 void gpu_set_device(int device);
 int gpu_devices();
 float *gpu_create_tensor(int dev, int size);

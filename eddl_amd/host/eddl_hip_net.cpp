@@ -10,6 +10,8 @@
 #include <set>
 #include <sstream>
 
+#include "../../include/eddlhip.h"
+
 namespace eddl_hip {
 
 // ---------------------------------------------------------------- Layer
@@ -509,7 +511,132 @@ void Net::setmode(int m) {
 }
 
 void Net::forward() {
-    for (Layer *l : layers) l->forward();
+    if (plan.empty()) {
+        for (Layer *l : layers) l->forward();
+        return;
+    }
+    // the steps are queued in order on the device's stream; one wait at the end
+    const bool was_synchronous = gpu_get_synchronous();
+    gpu_set_synchronous(false);
+    try {
+        for (const FusedStep &s : plan) run_step(s);
+    } catch (...) {
+        gpu_set_synchronous(was_synchronous);
+        throw;
+    }
+    gpu_set_synchronous(was_synchronous);
+    if (was_synchronous) gpu_synchronize(dev - DEV_GPU);
+}
+
+bool Net::is_fused_away(const Layer *l) const {
+    for (const Layer *x : fused_away)
+        if (x == l) return true;
+    return false;
+}
+
+// The chains follow one rule: a layer is taken into the step of the layer before it only when it is
+// that layer's sole child and the layer before it is not an output of the net, so that nothing else
+// reads the tensor that is no longer written.
+void Net::fuse() {
+    if (dev == DEV_CPU) msg("build the net with a computing service first", "Net::fuse");
+    plan.clear();
+    fused_away.clear();
+    auto sole_child = [this](Layer *l) -> Layer * { return (l->child.size() == 1 && !contains(lout, l)) ? l->child[0] : nullptr; };
+    vector<Layer *> done;      // layers whose output tensor the plan writes
+    vector<Layer *> absorbed;  // layers computed by the step of an earlier layer
+    for (Layer *l : layers) {
+        if (contains(absorbed, l)) continue;
+        FusedStep s;
+        s.first = s.last = l;
+        if (LPad *pad = dynamic_cast<LPad *>(l)) {
+            Layer *c = sole_child(l);
+            if (pad->constant == 0.0f && c != nullptr && dynamic_cast<LConv *>(c) != nullptr) {
+                fused_away.push_back(l);  // the convolution reads the pad's parent with larger paddings
+                continue;
+            }
+        }
+        if (LConv *conv = dynamic_cast<LConv *>(l)) {
+            s.chain = true;
+            s.src = l->parent[0];
+            s.pad_top = conv->cd->padrt;
+            s.pad_left = conv->cd->padcl;
+            if (LPad *pad = dynamic_cast<LPad *>(s.src)) {
+                if (is_fused_away(pad)) {
+                    s.pad_top += pad->padding[0];   // (top, right, bottom, left)
+                    s.pad_left += pad->padding[3];
+                    s.src = pad->parent[0];
+                }
+            }
+            Layer *c = sole_child(s.last);
+            if (LBatchNorm *bn = dynamic_cast<LBatchNorm *>(c)) {
+                s.bn = bn;
+                s.last = bn;
+                c = sole_child(s.last);
+            }
+            if (LSum *sum = dynamic_cast<LSum *>(c)) {
+                Layer *other = sum->parent[0] == s.last ? sum->parent[1] : sum->parent[0];
+                if (other != s.last && contains(done, other)) {
+                    s.res = other;
+                    s.last = sum;
+                    c = sole_child(s.last);
+                }
+            }
+            if (LActivation *a = dynamic_cast<LActivation *>(c)) {
+                if (a->act == "relu") {
+                    s.relu = true;
+                    s.last = a;
+                }
+            }
+            for (Layer *m = l; m != s.last; m = m->child[0]) {
+                fused_away.push_back(m);
+                absorbed.push_back(m->child[0]);
+            }
+        } else if (dynamic_cast<LDense *>(l) != nullptr) {
+            s.chain = true;
+            LActivation *a = dynamic_cast<LActivation *>(sole_child(l));
+            if (a != nullptr && a->act == "relu") {
+                s.relu = true;
+                s.last = a;
+                fused_away.push_back(l);
+                absorbed.push_back(a);
+            }
+        }
+        done.push_back(s.last);
+        plan.push_back(s);
+    }
+    for (Layer *o : lout)
+        if (is_fused_away(o)) msg("output layer " + o->name + " was fused away", "Net::fuse");
+    for (Layer *l : layers)
+        if (LConv *conv = dynamic_cast<LConv *>(l))
+            gpu_check(eddlhip_conv2d_cache_filters(dev - DEV_GPU, conv->cd->K->ptr, conv->cd->nk, conv->cd->kz, conv->cd->kr, conv->cd->kc),
+                      "Net::fuse");
+}
+
+void Net::run_step(const FusedStep &s) {
+    if (!s.chain) {
+        s.first->forward();
+        return;
+    }
+    const int device = dev - DEV_GPU;
+    if (LConv *conv = dynamic_cast<LConv *>(s.first)) {
+        const ConvolDescriptor *D = conv->cd;
+        const Tensor *I = s.src->output;
+        Tensor *O = s.last->output;
+        const LBatchNorm *bn = s.bn;
+        gpu_check(eddlhip_conv2d_fwd(device, I->ptr, D->K->ptr, D->use_bias ? D->bias->ptr : nullptr, O->ptr, I->shape[0], I->shape[1],
+                                     I->shape[2], I->shape[3], D->nk, D->kr, D->kc, D->sr, D->sc, s.pad_top, s.pad_left, D->r, D->c,
+                                     bn && bn->affine ? bn->bn_g->ptr : nullptr, bn && bn->affine ? bn->bn_b->ptr : nullptr,
+                                     bn ? bn->mean->ptr : nullptr, bn ? bn->variance->ptr : nullptr, bn ? bn->epsilon : 0.0f,
+                                     s.res ? s.res->output->ptr : nullptr, s.relu ? 1 : 0),
+                  "Net::forward (fused convolution)");
+        return;
+    }
+    LDense *dense = static_cast<LDense *>(s.first);
+    const Tensor *A = dense->input;
+    const int k = A->shape.back(), n = dense->ndim;
+    gpu_check(eddlhip_dense_fwd(device, A->ptr, dense->W->ptr, dense->use_bias ? dense->bias->ptr : nullptr, s.last->output->ptr,
+                                (int)(A->size / k), k, n, s.relu ? 1 : 0),
+              "Net::forward (fused dense)");
 }
 
 void Net::forward(const vector<Tensor *> &in) {
@@ -609,6 +736,7 @@ compserv CS_HIP(const vector<int> &g, const string &mem) {
 compserv CS_GPU(const vector<int> &g, const string &mem) { return CS_HIP(g, mem); }
 
 void build(model net, compserv cs, bool init_weights) { net->build(cs, init_weights); }
+void fuse(model net) { net->fuse(); }
 void set_mode(model net, int mode) { net->setmode(mode); }
 void summary(model m) { m->summary(true); }
 void load(model m, const string &fname, const string &format) { m->load(fname, format); }
@@ -622,6 +750,8 @@ vlayer forward(model m, vtensor in) {
 vtensor predict(model m, const vtensor &in) { return m->predict(in); }
 
 Tensor *getOutput(layer l1) {
+    if (l1->net != nullptr && l1->net->is_fused_away(l1))
+        msg("layer " + l1->name + " is computed inside a fused step of the plan; its output is not kept", "getOutput");
     Tensor *t = new Tensor(l1->output->getShape(), DEV_CPU);
     Tensor::copy(l1->output, t);
     return t;

@@ -212,6 +212,19 @@ struct CompServ {
     string mem = "full_mem";
 };
 
+// One step of a fused inference plan (Net::fuse): either one layer's forward(), or a convolution /
+// dense layer together with the layers that follow it and are computed in the same kernel.
+struct FusedStep {
+    Layer *first = nullptr;     // the layer the step starts at
+    Layer *last = nullptr;      // the layer whose output tensor the step writes
+    Layer *src = nullptr;       // conv chains: the layer whose output is read (a folded zero pad's parent)
+    LBatchNorm *bn = nullptr;   // conv chains: inference batch norm applied to the sums
+    Layer *res = nullptr;       // conv chains: the other operand of a residual LSum
+    bool relu = false;
+    int pad_top = 0, pad_left = 0;
+    bool chain = false;         // false: first->forward()
+};
+
 class Net {
   public:
     string name = "model";
@@ -231,6 +244,21 @@ class Net {
     void save(const string &filename, const string &format = "bin");
     void load(const string &filename, const string &format = "bin");
     string summary(bool print_stdout = true);
+
+    // Inference plan with the layer chains conv [+ batchnorm] [+ sum] [+ relu], zero pad + conv and
+    // dense + relu each computed by one kernel, and the repacked filters of every convolution kept
+    // between calls.  No counterpart in the reference (whose forward() always walks `layers`);
+    // results are the ones of the layer-by-layer walk, bit for bit.  Layers inside a chain leave
+    // their own output tensors unwritten (is_fused_away tells which); batch-norm layers inside a
+    // chain do not update their side outputs.  forward() queues the plan without waiting between
+    // steps and waits once at the end.
+    void fuse();
+    bool is_fused_away(const Layer *l) const;
+    vector<FusedStep> plan;  // empty until fuse()
+
+  private:
+    void run_step(const FusedStep &s);
+    vector<const Layer *> fused_away;
 };
 
 namespace eddl {
@@ -247,6 +275,7 @@ void setName(model m, string name);
 compserv CS_HIP(const vector<int> &g, const string &mem = "full_mem");
 compserv CS_GPU(const vector<int> &g, const string &mem = "full_mem");  // the reference's spelling, same service
 void build(model net, compserv cs, bool init_weights = true);
+void fuse(model net);  // Net::fuse: the fused inference plan (this backend's addition)
 void set_mode(model net, int mode);
 void summary(model m);
 void load(model m, const string &fname, const string &format = "bin");

@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <chrono>
 #include <fstream>
 #include <iostream>
 
@@ -146,7 +147,17 @@ int main(int argc, char **argv) {
         fprintf(stderr, "usage: net_driver <model> <params.bin|-> <input.raw> <output.raw> <batch> <size> [model arguments]\n");
         return 2;
     }
-    const string which = argv[1], params = argv[2], in_path = argv[3], out_path = argv[4];
+    // <model> may carry flags in front: "fused:vgg16", "time:vgg16", "fused+time:vgg16"
+    string which = argv[1];
+    bool fused = false, timed = false;
+    const size_t colon = which.find(':');
+    if (colon != string::npos) {
+        const string flags = which.substr(0, colon);
+        fused = flags.find("fused") != string::npos;
+        timed = flags.find("time") != string::npos;
+        which = which.substr(colon + 1);
+    }
+    const string params = argv[2], in_path = argv[3], out_path = argv[4];
     const int batch = atoi(argv[5]), size = atoi(argv[6]);
     vector<int> extra;
     for (int i = 7; i < argc; i++) extra.push_back(atoi(argv[i]));
@@ -161,7 +172,13 @@ int main(int argc, char **argv) {
             return 2;
         }
         build(m, CS_HIP({1}));
-        if (params != "-") load(m, params);
+        if (fused) {
+            fuse(m);
+            int away = 0;
+            for (Layer *l : m->layers) away += m->is_fused_away(l) ? 1 : 0;
+            printf("plan: %zu steps, %d layers computed inside another layer's step\n", m->plan.size(), away);
+        }
+        if (params != "-") load(m, params);  // after fuse(): the kept filter copies must follow the new values
         printf("layers:");
         for (Layer *l : m->layers) printf(" %s", l->kind().c_str());
         printf("\n");
@@ -190,6 +207,27 @@ int main(int argc, char **argv) {
             printf("\n");
             ofs.write(reinterpret_cast<const char *>(t->ptr), t->size * sizeof(float));
             delete t;
+        }
+        if (timed) {  // forwards with the input already on the device
+            for (int i = 0; i < 5; i++) m->forward();
+            const auto t0 = std::chrono::steady_clock::now();
+            const int reps = 20;
+            for (int i = 0; i < reps; i++) m->forward();
+            const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / reps;
+            printf("ms_per_forward %.4f images_per_s %.1f\n", ms, batch * 1000.0 / ms);
+        }
+        if (fused) {  // a layer inside a chain has no output to hand out
+            for (Layer *l : m->layers)
+                if (m->is_fused_away(l)) {
+                    bool threw = false;
+                    try {
+                        delete getOutput(l);
+                    } catch (const std::runtime_error &) {
+                        threw = true;
+                    }
+                    printf("%s getOutput of a fused-away layer\n", threw ? "ok " : "FAILED");
+                    break;
+                }
         }
         if (params == "-") save(m, out_path + ".params");  // round trip of freshly initialised parameters
         delete m;

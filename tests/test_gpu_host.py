@@ -122,12 +122,15 @@ def run_net_driver(args, timeout=300):
     return res.stdout
 
 
+@pytest.mark.parametrize("fused", [False, True], ids=["layerwise", "fused"])
 @pytest.mark.parametrize("which", ["block", "vgg16", "resnet50", "unet"])
-def test_cpp_graphs_match_the_python_runner_bit_for_bit(hip, which, tmp_path):
+def test_cpp_graphs_match_the_python_runner_bit_for_bit(hip, which, fused, tmp_path):
     """The same graph built through the C++ eddl:: API and through eddl_amd.net, the same parameters
     (written by Net.save in the reference's bin format, read by the C++ Net::load), the same input:
     identical layer order and identical outputs, after the C++ net has also been through a batch
-    resize."""
+    resize.  With Net::fuse() the C++ net runs its fused plan (parameters loaded after the plan was
+    made, so the kept filter copies have to follow them) and must still give the layer-by-layer
+    result of the Python runner bit for bit."""
     from eddl_amd import models
     batch = 3
     if which == "block":
@@ -143,7 +146,13 @@ def test_cpp_graphs_match_the_python_runner_bit_for_bit(hip, which, tmp_path):
     rng = np.random.default_rng(41)
     x = rng.standard_normal(m.lin[0].out_shape, dtype=np.float32)
     x.tofile(tmp_path / "x.raw")
-    out = run_net_driver([which, tmp_path / "params.bin", tmp_path / "x.raw", tmp_path / "y.raw", batch, size] + extra)
+    out = run_net_driver([("fused:" if fused else "") + which, tmp_path / "params.bin", tmp_path / "x.raw", tmp_path / "y.raw", batch, size] + extra)
+    if fused:
+        assert "FAILED" not in out and "ok  getOutput of a fused-away layer" in out, out
+        steps = int([l for l in out.splitlines() if l.startswith("plan:")][0].split()[1])
+        m.build(hip, fuse=True)
+        views = sum(1 for l in m.layers if l.kind in ("input", "reshape"))   # steps of the C++ plan that launch nothing
+        assert steps == len(m.ops) + views, (steps, len(m.ops), views)
     kinds = [l for l in out.splitlines() if l.startswith("layers:")][0].split()[1:]
     rename = {"input": "input", "relu": "relu", "sigmoid": "sigmoid", "softmax": "softmax"}
     assert kinds == [rename.get(l.kind, l.kind) for l in m.layers], "layer order differs"
