@@ -104,5 +104,7 @@ def test_host_layer_links_against_the_c_abi():
                 "_ZN8eddl_hip4eddl5ModelESt6vectorIPNS_5LayerESaIS3_EES5_",
                 "_ZN8eddl_hip4eddl6Conv2DEPNS_5LayerEiRKSt6vectorIiSaIiEES7_NSt7__cxx1112basic_stringIcSt11char_traitsIcESaIcEEEbiS7_SD_",
                 "_ZN8eddl_hip4eddl7predictEPNS_3NetERKSt6vectorIPNS_6TensorESaIS5_EE",
-                "_ZN8eddl_hip3Net4loadERKNSt7__cxx1112basic_stringIcSt11char_traitsIcESaIcEEES8_"):
+                "_ZN8eddl_hip3Net4loadERKNSt7__cxx1112basic_stringIcSt11char_traitsIcESaIcEEES8_",
+                # this backend's additions: the fused plan and the asynchronous mode of the wrappers
+                "_ZN8eddl_hip4eddl4fuseEPNS_3NetE", "_ZN8eddl_hip3Net4fuseEv", "_ZN8eddl_hip19gpu_set_synchronousEb"):
         assert hasattr(h, sym), sym
