@@ -10,6 +10,8 @@
 // MB, L2-resident) so that their loads are coalesced too.  k is split over wavefronts so the
 // whole device streams B; the per-slice partial blocks go to the private workspace and a second
 // kernel adds them in slice order (fixed summation order, no atomics).
+#include <algorithm>
+
 #include "common.h"
 
 using namespace eddlhip;
@@ -126,8 +128,17 @@ __global__ __launch_bounds__(256) void dense_reduce_kernel(const float *__restri
                                                            int incC, const float *__restrict__ bias, int n, int relu) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, stride = (size_t)gridDim.x * 256;
     for (size_t t = i; t < mn; t += stride) {
+        // eight slices' loads in flight at a time; the additions keep the slice order
         float s = part[t];
-        for (int ks = 1; ks < nslices; ks++) s = __fadd_rn(s, part[(size_t)ks * mn + t]);
+        int ks = 1;
+        for (; ks + 8 <= nslices; ks += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = part[(size_t)(ks + u) * mn + t];
+#pragma unroll
+            for (int u = 0; u < 8; u++) s = __fadd_rn(s, v[u]);
+        }
+        for (; ks < nslices; ks++) s = __fadd_rn(s, part[(size_t)ks * mn + t]);
         if (incC) s = __fadd_rn(C[t], s);
         if (bias) s = __fadd_rn(s, bias[t % (size_t)n]);
         if (relu) s = s > 0.0f ? s : 0.0f;
@@ -147,12 +158,15 @@ int dense_impl(int dev, const float *A, const float *B, float *C, int m, int k, 
     EH_TRY(use_device(dev));
     hipStream_t st = state(dev).stream;
     const int nt = (n + 127) / 128, mt = (m + 31) / 32;
-    // enough wavefronts to cover the device several times over, slices of at least 64 taps
-    long long want = 8LL * state(dev).num_cu;
-    int nslices = (int)((want + (long long)nt * mt - 1) / ((long long)nt * mt));
-    if (nslices < 1) nslices = 1;
-    int max_slices = (k + 63) / 64;
-    if (nslices > max_slices) nslices = max_slices;
+    // Wavefronts to cover the device eight times over, in slices of at least 128 taps (shorter
+    // slices cost more in partial blocks written and read back than they gain) - unless that
+    // leaves fewer than four wavefronts per CU, when slices go down to 64 taps.
+    const long long blocks = (long long)nt * mt;
+    const long long num_cu = state(dev).num_cu;
+    long long nsl = (8 * num_cu + blocks - 1) / blocks;
+    const long long max128 = (k + 127) / 128, max64 = (k + 63) / 64;
+    if (nsl > max128) nsl = std::max(max128, std::min((4 * num_cu + blocks - 1) / blocks, max64));
+    int nslices = (int)std::max(1LL, nsl);
     int kslice = ((k + nslices - 1) / nslices + 1) & ~1;  // even, so MFMA tap pairs do not straddle slices
     nslices = (k + kslice - 1) / kslice;
     EH_REQUIRE(nslices <= 65535 && mt <= 65535, "%s: shape out of range", what);
