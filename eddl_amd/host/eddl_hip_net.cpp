@@ -197,6 +197,18 @@ LPool::LPool(Layer *p, PoolDescriptor *D, const string &n, const string &prefix)
     input = p->output;
     pd->build(input);
     output = pd->O;
+    // src/layers/pool/layer_maxpool.cpp:46-51, layer_avgpool2D.cpp:43-48
+    if (pd->pad[0] != pd->pad[1] || pd->pad[2] != pd->pad[3]) {
+        string text = "In layer " + name + ": Padding asymmetry detected (top=" + std::to_string(pd->pad[0]) +
+                      ", bottom=" + std::to_string(pd->pad[1]) + ", left=" + std::to_string(pd->pad[2]) +
+                      ", right=" + std::to_string(pd->pad[3]) + "). The padding asymmetry is not allowed in a " +
+                      (prefix == "maxpool2d" ? "MaxPool" : "AveragePool") +
+                      " layer, we suggest you to use an explicit padding layer before this layer to fix the asymmetry.";
+        vector<int> asym = pd->pad;
+        delete pd;  // the output tensor stays with the Layer base, whose destructor releases it
+        pd = nullptr;
+        throw AsymmetricPaddingException(text, asym);
+    }
     p->addchild(this);
     addparent(p);
 }
@@ -579,6 +591,18 @@ void Net::fuse() {
                     s.res = other;
                     s.last = sum;
                     c = sole_child(s.last);
+                }
+            } else if (LAdd *add = dynamic_cast<LAdd *>(c)) {
+                // an LAdd of two layers computes (0 + a) + b, which differs from a + b only in the sign of a
+                // zero result; a ReLU behind it maps both to +0, so the pair is taken only together
+                if (add->parent.size() == 2) {
+                    Layer *other = add->parent[0] == s.last ? add->parent[1] : add->parent[0];
+                    LActivation *nxt = dynamic_cast<LActivation *>(sole_child(add));
+                    if (other != s.last && contains(done, other) && nxt != nullptr && nxt->act == "relu") {
+                        s.res = other;
+                        s.last = add;
+                        c = nxt;
+                    }
                 }
             }
             if (LActivation *a = dynamic_cast<LActivation *>(c)) {

@@ -102,6 +102,12 @@ def Softmax(parent, axis=-1, name=""):
 
 def _pool(kind, parent, pool_size, strides, padding, name):
     pd = PoolDescriptor(pool_size, strides, padding).build(parent.out_shape)
+    if pd.pad[0] != pd.pad[1] or pd.pad[2] != pd.pad[3]:
+        # src/layers/pool/layer_maxpool.cpp:46-51, layer_avgpool2D.cpp:43-48 (the layer is not linked to its parent)
+        raise AsymmetricPaddingException(
+            "In layer %s: Padding asymmetry detected (top=%d, bottom=%d, left=%d, right=%d). The padding asymmetry is not "
+            "allowed in a %s layer, we suggest you to use an explicit padding layer before this layer to fix the asymmetry."
+            % (name or kind, pd.pad[0], pd.pad[1], pd.pad[2], pd.pad[3], "MaxPool" if kind == "maxpool2d" else "AveragePool"), pd.pad)
     if pd.loop_rows != pd.r or pd.loop_cols != pd.c:
         msg("pooling window walk (%dx%d) disagrees with the descriptor's output shape (%dx%d)"
             % (pd.loop_rows, pd.loop_cols, pd.r, pd.c), "LPool::LPool")
@@ -396,6 +402,14 @@ class Net:
                 if id(other) in self.out and other is not last:
                     res, last = other, c
                     c = sole_child(last)
+            elif c is not None and c.kind == "add_n" and len(c.parents) == 2:
+                # an LAdd of two layers computes (0 + a) + b, which differs from a + b only in the sign of a zero
+                # result; a ReLU behind it maps both to +0, so the pair is taken only together
+                other = c.parents[1] if c.parents[0] is last else c.parents[0]
+                nxt = sole_child(c)
+                if id(other) in self.out and other is not last and nxt is not None and nxt.kind == "relu":
+                    res, last = other, c
+                    c = nxt
             if c is not None and c.kind == "relu":
                 relu, last = True, c
         # collect absorbed layers (everything between l and last)

@@ -115,6 +115,16 @@ static int errors() {
         printf("ok asymmetric pads %d %d %d %d\n", p[0], p[1], p[2], p[3]);
         ok &= p == vector<int>({0, 1, 0, 1});
     }
+    try {  // pools refuse asymmetric paddings as well: "same" 2x2 stride 2 on an odd plane pads (0,1)
+        MaxPool2D(Input({3, 5, 5}), {2, 2}, {2, 2}, "same");
+        ok = false;
+        printf("FAILED asymmetric pool pads: no exception\n");
+    } catch (const AsymmetricPaddingException &e) {
+        vector<int> p = e.get_asymmetric_pads();
+        printf("ok asymmetric pool pads %d %d %d %d\n", p[0], p[1], p[2], p[3]);
+        ok &= p == vector<int>({0, 1, 0, 1});
+    }
+    ok &= throws([] { AveragePool2D(Input({3, 5, 5}), {2, 2}, {2, 2}, "same"); }, "asymmetric average pool");
     ok &= throws([] { Dense(Input({4}), 3)->forward(); }, "forward before build");
     ok &= throws([] { Reshape(Input({4, 4}), {-1, -1}); }, "ambiguous reshape");
     ok &= throws([] { Reshape(Input({4, 4}), {5}); }, "incompatible reshape");

@@ -1,0 +1,225 @@
+"""ONNX import / export of the forward path, on the CPU.
+
+What pins the importer: three files written by PyTorch's exporter (tests/golden/onnx/*.onnx, made by
+tests/golden/make_onnx_fixtures.py) with PyTorch's own outputs for a seeded input.  The imported
+graph is run on the CPU oracle and has to reproduce those outputs, which also cross-checks the
+oracle's batch norm, pools, upsampling, pad, concat, dense, softmax and sigmoid against a second,
+unrelated implementation.  The repairs the reference's importer makes (asymmetric paddings, constants
+added onto a layer) are exercised with small files written by this package's own encoder.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from eddl_amd import models, onnx_io as O
+from eddl_amd import net as N
+from oracle import net_oracle
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+FIX = os.path.join(HERE, "golden", "onnx")
+
+EXPECTED_KINDS = {
+    "vgg_like": ["input", "conv2d", "relu", "maxpool2d", "conv2d", "relu", "batchnorm", "avgpool2d", "reshape", "dense", "relu", "dense",
+                 "softmax"],
+    "resnet_like": ["input", "conv2d", "relu", "maxpool2d", "conv2d", "relu", "conv2d", "add_n", "relu", "conv2d", "relu", "conv2d",
+                    "conv2d", "add_n", "relu", "avgpool2d", "reshape", "dense"],
+    "unet_like": ["input", "conv2d", "relu", "maxpool2d", "conv2d", "relu", "resize", "pad", "conv2d", "concat", "conv2d", "relu",
+                  "conv2d", "sigmoid"],
+}
+
+
+def close(ref, out):
+    ref = np.asarray(ref, np.float32)
+    return bool(np.all(np.abs(ref - out) <= 1e-5 * np.abs(ref).max() + 1e-4 * np.abs(ref)))
+
+
+# ---------------------------------------------------------------------------- wire format
+def test_varints_and_packed_fields_round_trip():
+    for v in (0, 1, 127, 128, 300, 2**31 - 1, 2**63 - 1, -1, -2**63):
+        got, pos = O._varint(O._wvarint(v), 0)
+        assert O._signed(got) == v and pos == len(O._wvarint(v))
+    # 300 is the two bytes AC 02 in every protobuf text
+    assert O._wvarint(300) == b"\xac\x02"
+    # an attribute with negative and large ints, packed as this encoder writes them and unpacked as older writers do
+    packed = O.AttributeProto(O._attr("pads", [0, -1, 2**40, 3]))
+    assert packed.name == "pads" and packed.ints == [0, -1, 2**40, 3]
+    unpacked = O._wbytes(1, "pads") + b"".join(O._wint(8, v) for v in [0, -1, 2**40, 3])
+    assert O.AttributeProto(unpacked).ints == [0, -1, 2**40, 3]
+    a = O.AttributeProto(O._attr("epsilon", 1e-5))
+    assert a.f == np.float32(1e-5)
+    assert O.AttributeProto(O._attr("mode", "nearest")).s == "nearest"
+
+
+def test_tensor_encodings():
+    w = np.arange(24, dtype=np.float32).reshape(2, 3, 4) - 7.5
+    t = O.TensorProto(O._tensor("w", w))
+    assert t.name == "w" and t.dims == [2, 3, 4] and t.data_type == O.FLOAT and np.array_equal(t.values, w.ravel())
+    # raw_data, the form PyTorch writes
+    raw = O._wbytes(1, O._wvarint(2) + O._wvarint(2)) + O._wint(2, O.FLOAT) + O._wbytes(9, np.float32([1, -2, 3.5, 4]).tobytes())
+    assert np.array_equal(O.TensorProto(raw).values, np.float32([1, -2, 3.5, 4]))
+    # int64 tensors (shapes, paddings) come out as floats, as in the reference's initializer maps
+    i = O.TensorProto(O._tensor("shape", np.array([-1, 128], np.int64), O.INT64))
+    assert i.data_type == O.INT64 and list(i.values) == [-1.0, 128.0]
+    raw64 = O._wbytes(1, O._wvarint(3)) + O._wint(2, O.INT64) + O._wbytes(9, np.array([0, -3, 2**33], np.int64).tobytes())
+    assert list(O.TensorProto(raw64).values) == [0.0, -3.0, float(2**33)]
+    scalar = O.TensorProto(O._tensor("c", np.array(0.25, np.float32)))
+    assert scalar.dims == [] and list(scalar.values) == [0.25]
+
+
+def test_truncated_and_missing_files(tmp_path):
+    data = open(os.path.join(FIX, "vgg_like.onnx"), "rb").read()
+    with pytest.raises(RuntimeError, match="ONNX::ImportNet"):
+        O.import_net_from_onnx_bytes(data[:len(data) // 2])
+    with pytest.raises(RuntimeError, match="ONNX::ImportNet"):
+        O.import_net_from_onnx_file(str(tmp_path / "absent.onnx"))
+
+
+# ---------------------------------------------------------------------------- files written by PyTorch
+@pytest.mark.parametrize("name", sorted(EXPECTED_KINDS))
+def test_pytorch_files_import_and_reproduce_pytorch_outputs(oracle, name):
+    net = O.import_net_from_onnx_file(os.path.join(FIX, name + ".onnx"))
+    d = np.load(os.path.join(FIX, name + ".npz"))
+    assert [l.kind for l in net.layers] == EXPECTED_KINDS[name]
+    assert net.lin[0].out_shape == [1] + list(d["x"].shape[1:])  # batch 1 until a forward says otherwise
+    y = net_oracle.forward(oracle, net, [d["x"]], conv_algo="direct")[0]
+    assert y.shape == d["y"].shape
+    assert close(d["y"], y), np.abs(y - d["y"]).max()
+
+
+def test_details_of_the_imported_layers():
+    net = O.import_net_from_onnx_file(os.path.join(FIX, "vgg_like.onnx"))
+    by_kind = {}
+    for l in net.layers:
+        by_kind.setdefault(l.kind, []).append(l)
+    c1, c2 = by_kind["conv2d"]
+    assert c1.attrs["cd"].use_bias and not c2.attrs["cd"].use_bias
+    assert c1.attrs["cd"].pads == [1, 1, 1, 1] and c1.params["K"].shape == (6, 3, 3, 3)
+    bn = by_kind["batchnorm"][0]
+    assert bn.attrs["affine"] and abs(bn.attrs["epsilon"] - 1e-5) < 1e-12 and abs(bn.attrs["momentum"] - 0.9) < 1e-6
+    assert list(bn.params) == ["bn_g", "bn_b", "mean", "variance"] and bn.params["variance"].min() >= 0.5
+    d1, d2 = by_kind["dense"]
+    assert d1.params["W"].shape == (128, 12) and d2.params["W"].shape == (12, 5)  # transB = 1 in the file: [out, in] -> [in, out]
+    assert by_kind["softmax"][0].attrs["axis"] == 1
+    # the ResNet-like file: 3x3 stride-2 max-pool with paddings 1, GlobalAveragePool as an average pool over the plane
+    net = O.import_net_from_onnx_file(os.path.join(FIX, "resnet_like.onnx"))
+    mp = [l for l in net.layers if l.kind == "maxpool2d"][0].attrs["pd"]
+    assert (mp.kr, mp.kc, mp.sr, mp.sc, mp.pad) == (3, 3, 2, 2, [1, 1, 1, 1])
+    gap = [l for l in net.layers if l.kind == "avgpool2d"][0]
+    assert gap.attrs["pd"].ksize == gap.parents[0].out_shape[2:] and gap.out_shape[2:] == [1, 1]
+    # the U-Net-like file: Upsample by 2, Pad (bottom 1, right 1) as (top, right, bottom, left), concat over the channels
+    net = O.import_net_from_onnx_file(os.path.join(FIX, "unet_like.onnx"))
+    pad = [l for l in net.layers if l.kind == "pad"][0]
+    assert pad.attrs["pads"] == [0, 1, 1, 0] and pad.attrs["constant"] == 0.0
+    rs = [l for l in net.layers if l.kind == "resize"][0]
+    assert rs.out_shape[2:] == [2 * d for d in rs.parents[0].out_shape[2:]]
+    assert [l for l in net.layers if l.kind == "concat"][0].attrs["axis"] == 1
+
+
+def test_input_shape_override():
+    net = O.import_net_from_onnx_file(os.path.join(FIX, "unet_like.onnx"), input_shape=[1, 32, 48])
+    assert net.lin[0].out_shape == [1, 1, 32, 48] and net.lout[0].out_shape == [1, 1, 32, 48]
+
+
+# ---------------------------------------------------------------------------- export -> import
+@pytest.mark.parametrize("which", ["block", "vgg16", "resnet50", "unet"])
+def test_export_import_round_trip(which):
+    if which == "block":
+        m = models.conv_bn_relu_pool_block(batch=1, channels=5, size=12, filters=7)
+    elif which == "vgg16":
+        m = models.vgg16(batch=1, size=32, num_classes=10, widths=(4, 8, 8, 16, 16), dense=32)
+    elif which == "resnet50":
+        m = models.resnet50(batch=1, size=64, num_classes=10, base=4)
+    else:
+        m = models.unet(batch=1, size=32, widths=(4, 8), bottleneck=16)
+    models.init_he_normal(m, 5)
+    data = O.export_net_to_onnx_bytes(m)
+    model = O.ModelProto(data)
+    assert model.producer_name == "EDDL" and model.opset_import == [("", 11)] and model.graph.name == "Computational Graph"
+    assert model.graph.input[0].dims[0] == "batch" and model.graph.input[0].dims[1:] == m.lin[0].out_shape[1:]
+    back = O.import_net_from_onnx_bytes(data)
+    # LSum comes back as LSum (Sum node), everything else as itself; names are the layers' names
+    assert [(l.kind, l.name, l.out_shape) for l in back.layers] == [(l.kind, l.name, l.out_shape) for l in m.layers]
+    for a, b in zip(m.layers, back.layers):
+        assert list(a.params) == list(b.params)
+        for key in a.params:
+            used = key != "bias" or (a.attrs["cd"].use_bias if a.kind == "conv2d" else a.attrs.get("use_bias", True))
+            if used:
+                assert np.array_equal(a.params[key], b.params[key]), (a.name, key)
+        if a.kind == "conv2d":
+            ca, cb = a.attrs["cd"], b.attrs["cd"]
+            assert (ca.pads, ca.sr, ca.sc, ca.use_bias) == (cb.pads, cb.sr, cb.sc, cb.use_bias)
+        if a.kind == "batchnorm":
+            assert abs(a.attrs["epsilon"] - b.attrs["epsilon"]) < 1e-12
+        if a.kind == "pad":
+            assert a.attrs["pads"] == b.attrs["pads"]
+    # parameters are written as float_data, the form the reference's exporter uses (no raw_data field 9 in an initializer)
+    for f, wt, v in O._fields(next(v for f, wt, v in O._fields(data) if f == 7)):
+        if f == 5:
+            assert 9 not in [f2 for f2, _, _ in O._fields(v)]
+
+
+# ---------------------------------------------------------------------------- the importer's repairs
+def tiny_model(nodes, inits, in_shape, out_name, out_shape):
+    graph = b"".join(O._wbytes(1, n) for n in nodes) + b"".join(O._wbytes(5, t) for t in inits)
+    graph += O._wbytes(11, O._value_info("x", [1] + in_shape)) + O._wbytes(12, O._value_info(out_name, [1] + out_shape))
+    return O._wint(1, 6) + O._wbytes(7, graph) + O._wbytes(8, O._wint(2, 11))
+
+
+def test_asymmetric_paddings_become_a_pad_layer(oracle):
+    rng = np.random.default_rng(3)
+    K = rng.standard_normal((4, 2, 2, 2)).astype(np.float32)
+    conv = O._node("Conv", "c", ["x", "c_W"], ["c"], [("kernel_shape", [2, 2]), ("pads", [0, 0, 1, 1]), ("strides", [1, 1])])
+    pool = O._node("MaxPool", "p", ["c"], ["p"], [("kernel_shape", [2, 2]), ("pads", [1, 0, 0, 1]), ("strides", [2, 2])])
+    net = O.import_net_from_onnx_bytes(tiny_model([conv, pool], [O._tensor("c_W", K)], [2, 6, 6], "p", [4, 3, 3]))
+    assert [(l.kind, l.name) for l in net.layers] == [("input", "x"), ("pad", "c__asymmetric_padding"), ("conv2d", "c"),
+                                                      ("pad", "p__asymmetric_padding"), ("maxpool2d", "p")]
+    pads = [l.attrs["pads"] for l in net.layers if l.kind == "pad"]
+    assert pads == [[0, 1, 1, 0], [1, 1, 0, 0]]  # (top, right, bottom, left)
+    assert net.layers[2].attrs["cd"].pads == [0, 0, 0, 0] and net.layers[2].out_shape == [1, 4, 6, 6]
+    assert net.layers[1].children == [net.layers[2]] and net.layers[0].children == [net.layers[1]]  # the refused layers left no trace
+    # the convolution with a zero border on the bottom and right equals the padded "valid" convolution
+    x = rng.standard_normal((1, 2, 6, 6)).astype(np.float32)
+    y = net_oracle.forward(oracle, net, [x], conv_algo="direct", keep=True)[1]["c"]
+    want = oracle.conv2d(np.pad(x, ((0, 0), (0, 0), (0, 1), (0, 1))), K, None, (1, 1), 0, 0, 6, 6, algo="direct")
+    assert np.array_equal(y, want)
+
+
+def test_constants_added_onto_layers_become_biases():
+    rng = np.random.default_rng(4)
+    K, b0, b1 = rng.standard_normal((3, 2, 1, 1)).astype(np.float32), np.float32([1, 2, 3]), np.float32([0.5, 0.25, 0.125])
+    W, wb = rng.standard_normal((27, 4)).astype(np.float32), np.float32([1, -1, 2, -2])
+    nodes = [O._node("Conv", "c", ["x", "K"], ["c"], [("kernel_shape", [1, 1])]),
+             O._node("Add", "a0", ["c", "b0"], ["a0"]),      # no bias yet: becomes the bias
+             O._node("Add", "a1", ["b1", "a0"], ["a1"]),     # constant on the left, bias present: added to it
+             O._node("Flatten", "f", ["a1"], ["f"]),
+             O._node("MatMul", "mm", ["f", "W"], ["mm"]),
+             O._node("Add", "a2", ["mm", "wb"], ["a2"])]
+    inits = [O._tensor("K", K), O._tensor("b0", b0), O._tensor("b1", b1), O._tensor("W", W), O._tensor("wb", wb)]
+    net = O.import_net_from_onnx_bytes(tiny_model(nodes, inits, [2, 3, 3], "a2", [4]))
+    assert [l.kind for l in net.layers] == ["input", "conv2d", "reshape", "dense"]
+    conv, dense = net.layers[1], net.layers[3]
+    assert conv.attrs["cd"].use_bias and np.array_equal(conv.params["bias"], b0 + b1)
+    assert dense.attrs["use_bias"] and np.array_equal(dense.params["bias"], wb) and np.array_equal(dense.params["W"], W)
+    assert net.lout == [dense]
+
+
+def test_nodes_outside_the_path_are_refused():
+    node = O._node("LSTM", "r", ["x"], ["r"])
+    with pytest.raises(RuntimeError, match="ONNX::ImportNet"):
+        O.import_net_from_onnx_bytes(tiny_model([node], [], [4, 4], "r", [4]))
+    up = O._node("Resize", "u", ["x", "", "s"], ["u"], [("mode", "linear")])
+    with pytest.raises(RuntimeError, match="ONNX::ImportNet"):
+        O.import_net_from_onnx_bytes(tiny_model([up], [O._tensor("s", np.float32([1, 1, 2, 2]))], [1, 4, 4], "u", [1, 8, 8]))
+    cat = O._node("Concat", "k", ["x", "x"], ["k"], [("axis", 0)])
+    with pytest.raises(RuntimeError, match="ONNX::ImportNet"):
+        O.import_net_from_onnx_bytes(tiny_model([cat], [], [1, 4, 4], "k", [1, 4, 4]))
+
+
+def test_pools_refuse_asymmetric_paddings_like_the_reference():
+    x = N.Input([3, 5, 5])
+    with pytest.raises(N.AsymmetricPaddingException) as e:
+        N.MaxPool2D(x, [2, 2], [2, 2], "same")
+    assert e.value.pads == [0, 1, 0, 1]
+    with pytest.raises(N.AsymmetricPaddingException):
+        N.AveragePool2D(x, [2, 2], [2, 2], [0, 1, 0, 1])
