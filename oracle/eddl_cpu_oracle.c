@@ -32,8 +32,11 @@
  *                        sequence (sub, div, mul, add) is from source reading only.
  *   relu/add/concat/
  *   upsample/sigmoid     closed forms, torch cross-checks
- *   dense (mult2D)       parity unpinned in the reference's tests (textbook GEMM; numpy
- *                        float64 cross-check only)
+ *   dense (mult2D)       no vector in the reference's tests; a textbook matrix product, pinned
+ *                        by library routines: numpy float64 matmul, and PyTorch's Linear
+ *                        through networks exported to ONNX with PyTorch's own outputs
+ *   whole graphs         three PyTorch-exported networks (conv, batch norm, pools, upsample,
+ *                        pad, concat, add, dense, softmax, sigmoid) reproduce PyTorch's outputs
  */
 #include <math.h>
 #include <stddef.h>
@@ -488,8 +491,9 @@ void eddl_oracle_pad(const float *A, float *B, int N, int C, int H, int W, int t
 /* src/hardware/cpu/cpu_math.cpp:302-328 as used by src/layers/core/layer_dense.cpp:65-73
  * (tA = tB = 0, incC = 0): C[m x n] = A[m x k] * B[k x n], row-major, B = W[in, out].
  * The reference's product is an Eigen GEMM (summation order Eigen-internal); this sums each
- * output's k products in increasing index with one fp32 accumulator.  PARITY UNPINNED by
- * any numeric test in the reference. */
+ * output's k products in increasing index with one fp32 accumulator.  The reference's tests
+ * hold no vector for it; it is pinned as a textbook matrix product against numpy (float64)
+ * and against PyTorch's Linear layers in the exported-network fixtures. */
 void eddl_oracle_mult2d(const float *A, const float *B, float *C, int m, int k, int n) {
 #pragma omp parallel for schedule(static)
     for (int j0 = 0; j0 < n; j0 += 256) {
