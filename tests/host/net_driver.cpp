@@ -14,6 +14,7 @@
 #include <iostream>
 
 #include "eddl_hip_net.h"
+#include "eddl_hip_onnx.h"
 
 using namespace eddl_hip;
 using namespace eddl_hip::eddl;
@@ -151,8 +152,59 @@ static int errors() {
     return ok ? 0 : 1;
 }
 
+// onnx <file.onnx> <input.raw> <output.raw> <batch> <fused 0|1> [<re-export.onnx>]: imports the file, runs one
+// batch, writes the output; with a last argument also writes the built net back out as ONNX.
+static int onnx(int argc, char **argv) {
+    if (argc < 7) {
+        fprintf(stderr, "usage: net_driver onnx <file.onnx> <input.raw> <output.raw> <batch> <fused> [<re-export.onnx>]\n");
+        return 2;
+    }
+    try {
+        model m = eddl_hip::import_net_from_onnx_file(argv[2]);
+        printf("layers:");
+        for (Layer *l : m->layers) printf(" %s", l->kind().c_str());
+        printf("\nnames:");
+        for (Layer *l : m->layers) printf(" %s", l->name.c_str());
+        printf("\n");
+        build(m, CS_HIP({1}), false);  // keep the imported parameters
+        if (atoi(argv[6])) {
+            fuse(m);
+            printf("plan: %zu steps\n", m->plan.size());
+        }
+        vector<int> ishape = m->lin[0]->output->getShape();
+        ishape[0] = atoi(argv[5]);
+        Tensor x(ishape, DEV_CPU);
+        std::ifstream ifs(argv[3], std::ios::binary);
+        ifs.read(reinterpret_cast<char *>(x.ptr), x.size * sizeof(float));
+        if (!ifs.good()) {
+            fprintf(stderr, "short input file\n");
+            return 2;
+        }
+        vtensor out = predict(m, {&x});
+        std::ofstream ofs(argv[4], std::ios::binary);
+        for (Tensor *t : out) {
+            ofs.write(reinterpret_cast<const char *>(t->ptr), t->size * sizeof(float));
+            delete t;
+        }
+        if (argc > 7) eddl_hip::save_net_to_onnx_file(m, argv[7]);
+        bool threw = false;
+        try {
+            eddl_hip::import_net_from_onnx_file(string(argv[2]) + ".absent");
+        } catch (const std::runtime_error &) {
+            threw = true;
+        }
+        printf("%s missing ONNX file\n", threw ? "ok " : "FAILED");
+        delete m;
+    } catch (const std::exception &e) {
+        fprintf(stderr, "exception: %s\n", e.what());
+        return 1;
+    }
+    return 0;
+}
+
 int main(int argc, char **argv) {
     if (argc >= 2 && !strcmp(argv[1], "errors")) return errors();
+    if (argc >= 2 && !strcmp(argv[1], "onnx")) return onnx(argc, argv);
     if (argc < 7) {
         fprintf(stderr, "usage: net_driver <model> <params.bin|-> <input.raw> <output.raw> <batch> <size> [model arguments]\n");
         return 2;

@@ -106,5 +106,9 @@ def test_host_layer_links_against_the_c_abi():
                 "_ZN8eddl_hip4eddl7predictEPNS_3NetERKSt6vectorIPNS_6TensorESaIS5_EE",
                 "_ZN8eddl_hip3Net4loadERKNSt7__cxx1112basic_stringIcSt11char_traitsIcESaIcEEES8_",
                 # this backend's additions: the fused plan and the asynchronous mode of the wrappers
-                "_ZN8eddl_hip4eddl4fuseEPNS_3NetE", "_ZN8eddl_hip3Net4fuseEv", "_ZN8eddl_hip19gpu_set_synchronousEb"):
+                "_ZN8eddl_hip4eddl4fuseEPNS_3NetE", "_ZN8eddl_hip3Net4fuseEv", "_ZN8eddl_hip19gpu_set_synchronousEb",
+                # ONNX: import_net_from_onnx_file / _pointer, save_net_to_onnx_file
+                "_ZN8eddl_hip25import_net_from_onnx_fileERKNSt7__cxx1112basic_stringIcSt11char_traitsIcESaIcEEERKSt6vectorIiSaIiEEi",
+                "_ZN8eddl_hip28import_net_from_onnx_pointerEPKvmi",
+                "_ZN8eddl_hip21save_net_to_onnx_fileEPNS_3NetERKNSt7__cxx1112basic_stringIcSt11char_traitsIcESaIcEEE"):
         assert hasattr(h, sym), sym

@@ -177,3 +177,35 @@ def test_cpp_graph_errors_and_parameter_round_trip(hip, tmp_path):
     m.build(hip, fuse=False)
     want = m.predict([x])[0]
     assert np.array_equal(np.fromfile(tmp_path / "y.raw", np.float32).reshape(want.shape), want)
+
+
+# ---------------------------------------------------------------------------- ONNX through the C++ host layer
+@pytest.mark.parametrize("fused", [0, 1], ids=["layerwise", "fused"])
+@pytest.mark.parametrize("name", ["vgg_like", "resnet_like", "unet_like"])
+def test_cpp_onnx_import_matches_pytorch_and_the_python_importer(hip, name, fused, tmp_path):
+    """The files PyTorch wrote (tests/golden/onnx), imported by the C++ import_net_from_onnx_file: same
+    layers and names as the Python importer builds, PyTorch's outputs within the convolution tolerance,
+    the Python runner's outputs bit for bit; the net written back by the C++ exporter loads in the
+    Python importer with identical layers and parameters."""
+    from eddl_amd import onnx_io
+    fix = os.path.join(ROOT, "tests", "golden", "onnx")
+    d = np.load(os.path.join(fix, name + ".npz"))
+    d["x"].tofile(tmp_path / "x.raw")
+    out = run_net_driver(["onnx", os.path.join(fix, name + ".onnx"), tmp_path / "x.raw", tmp_path / "y.raw", d["x"].shape[0], fused,
+                          tmp_path / "back.onnx"])
+    assert "FAILED" not in out and "ok  missing ONNX file" in out, out
+    net = onnx_io.import_net_from_onnx_file(os.path.join(fix, name + ".onnx"))
+    kinds = [l for l in out.splitlines() if l.startswith("layers:")][0].split()[1:]
+    names = [l for l in out.splitlines() if l.startswith("names:")][0].split()[1:]
+    assert kinds == [l.kind for l in net.layers] and names == [l.name for l in net.layers]
+    got = np.fromfile(tmp_path / "y.raw", np.float32).reshape(d["y"].shape)
+    assert np.all(np.abs(got - d["y"]) <= 1e-5 * np.abs(d["y"]).max() + 1e-4 * np.abs(d["y"]))
+    net.build(hip, fuse=False)
+    assert np.array_equal(got, net.predict([d["x"]])[0])
+    back = onnx_io.import_net_from_onnx_file(str(tmp_path / "back.onnx"))
+    assert [(l.kind, l.name, l.out_shape[1:]) for l in back.layers] == [(l.kind, l.name, l.out_shape[1:]) for l in net.layers]
+    for a, b in zip(net.layers, back.layers):
+        for key in a.params:
+            if key == "bias" and not (a.attrs["cd"].use_bias if a.kind == "conv2d" else a.attrs.get("use_bias", True)):
+                continue
+            assert np.array_equal(a.params[key], b.params[key]), (a.name, key)
