@@ -3,11 +3,11 @@
 
 A step is one forward pass of the workload over one batch of synthetic input that is already
 resident in HBM (default workload: VGG-16, batch 32, fp32, 3x224x224 - the configuration the
-headline metric is quoted on).  Prints ONE JSON line on stdout; a per-layer table goes to
-stderr and to gpurun_out/bench_layers.json when that directory exists.
+headline metric is quoted on).  Prints ONE JSON line on stdout; the per-layer table goes to
+stderr with --layers and to DIR/bench_layers_<workload>.{json,txt} with --out DIR.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vgg16|block|resnet50|unet]
-                    [--no-cpu-baseline] [--layers]
+                    [--no-cpu-baseline] [--layers] [--out DIR]
 """
 import argparse
 import json
@@ -136,6 +136,7 @@ def main():
     ap.add_argument("--workload", default="vgg16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-op table to stderr")
+    ap.add_argument("--out", default=None, metavar="DIR", help="also write the per-op table and the result into this directory")
     ap.add_argument("--conv-algo", default="auto", choices=["auto", "mfma_staged", "mfma_lds"], help="input gather of the convolution kernels")
     ap.add_argument("--no-device-probe", action="store_true",
                     help="skip the pure-MFMA probe of the device's sustained fp32 matrix rate (keeps kernel traces to the workload)")
@@ -245,8 +246,9 @@ def main():
             r.get("kernel", "")))
     if args.layers:
         print("\n".join(table), file=sys.stderr)
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out_dir):
+    out_dir = args.out
+    if out_dir:
+        os.makedirs(out_dir, exist_ok=True)
         with open(os.path.join(out_dir, "bench_layers_%s.json" % args.workload), "w") as fh:
             json.dump({"result": result, "ops": rows}, fh, indent=1)
         with open(os.path.join(out_dir, "bench_layers_%s.txt" % args.workload), "w") as fh:
