@@ -24,7 +24,11 @@
 //                    the per-step address work is one scalar offset per channel.  By default
 //                    both operand slices go global -> LDS directly (buffer_load ... lds),
 //                    skipping the register file; a register-staged form is kept for checking.
-//   conv_gen_kernel  any filter shape, K-step 16 taps, tap validity computed per element.
+//   conv_gen_kernel  any filter shape, K-step 16 taps.  What a tap needs (its byte offset from
+//                    the window origin, its channel's byte offset, its row and column in the
+//                    filter) comes from a table written once per call and read with scalar
+//                    loads, so a gathered element costs two bounds tests and one address add.
+//                    Same LDS-direct loads as conv_tap_kernel.
 //
 // Accumulation order per output: taps in increasing i, two per MFMA (the instruction adds
 // both products of a pair into the fp32 accumulator), one accumulator from the first tap to
@@ -57,6 +61,8 @@ constexpr int M_ALIGN = 128;                  // packed filter rows are padded t
 constexpr int OOB = (int)0x80000000u;         // byte offset no buffer of <= 2 GiB contains
 constexpr unsigned RSRC_WORD3 = 0x00020000u;  // raw buffer, 32-bit data format
 
+typedef int int32x4 __attribute__((ext_vector_type(4)));
+
 struct ConvParams {
     const float *I;
     const float *Wp;  // packed filters [rows][Mp]
@@ -76,6 +82,8 @@ struct ConvParams {
     // adds the slices and finishes those tiles.
     int main_tiles, nslices, slice_steps;
     float *partial;
+    // conv_gen_kernel only: one entry per tap of the padded K range (tap_table_kernel)
+    const int32x4 *taps;
 };
 
 // The fused tail of a Conv -> BatchNorm(inference) -> Add -> ReLU chain; every step rounded
@@ -119,8 +127,6 @@ __device__ __forceinline__ float apply_epilogue(const ConvParams &p, const Chann
 // filled from the buffer being read), which would serialise the loads of step t+1 with the MFMAs
 // of step t.  With the instruction opaque to it, the kernel places the one wait that is needed
 // itself: vmcnt(0) before the barrier that publishes the buffer.
-typedef int int32x4 __attribute__((ext_vector_type(4)));
-
 __device__ __forceinline__ int32x4 make_rsrc_words(const void *base, unsigned bytes) {
     const unsigned long long a = (unsigned long long)base;
     int32x4 r;
@@ -532,7 +538,30 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
 // ---------------------------------------------------------------- MFMA kernel, any filter shape
 // K-step = 16 taps.  Thread t gathers pixel t % BN for EPT consecutive taps of the step; the tap
 // walk (c, ky, kx) is uniform in a wavefront and advances with scalar arithmetic.
-template <int WM, int WN, int TM, int TN>
+// Tap table of conv_gen_kernel: entry k of the padded K range (k = (c*R + ky)*S + kx) holds
+// { byte offset of the tap relative to the window origin, byte offset of channel c, ky, kx }.
+// Taps past C*R*S get a row offset no image reaches, so their gathers read zeros.
+constexpr int TAP_NOWHERE = 0x40000000;
+__global__ __launch_bounds__(256) void tap_table_kernel(int32x4 *table, int rows, int C, int R, int S, int W, int HW) {
+    const int k = blockIdx.x * 256 + threadIdx.x;
+    if (k >= rows) return;
+    const int c = k / (R * S), rem = k - c * (R * S), ky = rem / S, kx = rem - ky * S;
+    int32x4 t;
+    if (c < C) {
+        t.x = (ky * W + kx) * 4;
+        t.y = c * HW * 4;
+        t.z = ky;
+        t.w = kx;
+    } else {
+        t.x = 0;
+        t.y = 0;
+        t.z = TAP_NOWHERE;
+        t.w = 0;
+    }
+    table[k] = t;
+}
+
+template <int WM, int WN, int TM, int TN, bool DIRECT>
 __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(const ConvParams p) {
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     constexpr int BK = 16;
@@ -550,7 +579,6 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
-    const int R = p.R, S = p.S, RS = R * S;
     int m_tile, n_tile, local_tile, slice;
     bool split;
     tile_of_block(p, m_tile, n_tile, local_tile, slice, split);
@@ -564,21 +592,20 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
     const __amdgpu_buffer_rsrc_t rsrc_in = __builtin_amdgcn_make_buffer_rsrc((void *)p.I, 0, p.in_bytes, RSRC_WORD3);
 
     const int bn_l = tid % BN;
-    const int bg = __builtin_amdgcn_readfirstlane(tid / BN);  // tap group (BN >= 64: uniform in a wavefront)
-    int ih0, iw0, pix;
-    bool pvalid;
+    const int bg = __builtin_amdgcn_readfirstlane(tid / BN);           // tap group (BN >= 64: uniform in a wavefront)
+    const int seg_off = __builtin_amdgcn_readfirstlane((tid - lane) % BN);  // first pixel column of this wavefront
+    int ih0, iw0, pix4;
     {
         const int ng = (int)n0 + bn_l;  // a launch covers fewer than 2^31 pixels
-        pvalid = ng < (int)p.npix;
+        const bool pvalid = ng < (int)p.npix;
         const unsigned ngc = pvalid ? (unsigned)ng : 0u;
         const int img = (int)(ngc / (unsigned)p.PQ);
         const int pq = (int)(ngc - (unsigned)img * (unsigned)p.PQ);
         const int op = (int)((unsigned)pq / (unsigned)p.Q), oq = pq - op * p.Q;
-        ih0 = op * p.sr - p.pt;
+        ih0 = pvalid ? op * p.sr - p.pt : TAP_NOWHERE;  // a pixel past the end of the launch gathers zeros
         iw0 = oq * p.sc - p.pl;
-        pix = img * (p.C * p.H * p.W) + ih0 * p.W + iw0;
+        pix4 = (img * (p.C * p.H * p.W) + (op * p.sr - p.pt) * p.W + iw0) * 4;
     }
-    const int HW4 = p.H * p.W * 4;
 
     // (plain 16-byte loads: the packed matrix is padded to whole steps and whole tiles, so every address exists)
     // Every thread loads in every round, without a condition: in a partial last round the lanes past
@@ -595,39 +622,66 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
         a_lds[j] = in_slice ? kk * LDA + m4 : BK * LDA + lane * 4;
     }
     const int a_step = BK * p.Mp;
-    floatx4 areg[AV];
-    float breg[EPT];
+    floatx4 areg[DIRECT ? 1 : AV];
+    float breg[DIRECT ? 1 : EPT];
 
-    auto load_a = [&](int step) {
+    // LDS-direct filter slice, as in conv_tap_kernel: a wavefront instruction moves RPI = 256 / BM
+    // whole rows; unit u belongs to wavefront u % 4; surplus rows of the last unit land in the
+    // parking area behind the slice.
+    constexpr int RPI = 256 / BM;
+    constexpr int A_UNITS = (BK + RPI - 1) / RPI;
+    constexpr int A_UPW = (A_UNITS + 3) / 4;
+    static_assert((RPI - 1) * BM <= 256, "the parking area holds the surplus rows of the last unit");
+    const int32x4 dma_w = make_rsrc_words(p.Wp, p.wp_bytes), dma_in = make_rsrc_words(p.I, p.in_bytes);
+    const int a_voff_direct = ((lane / (BM / 4)) * p.Mp + m0 + 4 * (lane % (BM / 4))) * 4;
+
+    auto load_a = [&](int step, lds_float *as) {
+        if constexpr (DIRECT) {
 #pragma unroll
-        for (int j = 0; j < AV; j++)
-            areg[j] = *reinterpret_cast<const floatx4 *>(a_ptr[j] + (size_t)step * a_step);
+            for (int j = 0; j < A_UPW; j++) {
+                const int u = wave + 4 * j;
+                if (A_UNITS % 4 == 0 || j < A_UPW - 1 || u < A_UNITS) {  // uniform in the wavefront
+                    const int kk = u * RPI;
+                    lds_dma_b128(dma_w, as + kk * LDA, a_voff_direct, (step * BK + kk) * p.Mp * 4);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < AV; j++) areg[j] = *reinterpret_cast<const floatx4 *>(a_ptr[j] + (size_t)step * a_step);
+        }
     };
-    auto load_b = [&](int step) {
-        const int i = step * BK + bg * EPT;  // uniform
-        int c = i / RS;
-        const int rem = i - c * RS;
-        int ky = rem / S, kx = rem - ky * S;
+    // the gather of one step: this wavefront's tap group, 64 pixels per tap row.  The table entries
+    // are read through the constant address space with a wavefront-uniform index: scalar loads.
+    typedef const __attribute__((address_space(4))) int32x4 *tap_table_ptr;
+    const tap_table_ptr taps = (tap_table_ptr)p.taps;
+    auto load_b = [&](int step, lds_float *bs) {
+        const int i = step * BK + bg * EPT;
+        int32x4 t[EPT];  // all entries first: the loads below are opaque to the compiler and would keep them apart
+#pragma unroll
+        for (int e = 0; e < EPT; e++) t[e] = taps[i + e];
 #pragma unroll
         for (int e = 0; e < EPT; e++) {
-            const bool ok = pvalid && c < p.C && (unsigned)(ih0 + ky) < (unsigned)p.H && (unsigned)(iw0 + kx) < (unsigned)p.W;
-            const int vo = ok ? (pix + ky * p.W + kx) * 4 : OOB;
-            breg[e] = buf_load(rsrc_in, vo, (c < p.C ? c : 0) * HW4);
-            if (++kx == S) {
-                kx = 0;
-                if (++ky == R) {
-                    ky = 0;
-                    ++c;
-                }
+            const bool ok = (unsigned)(ih0 + t[e].z) < (unsigned)p.H && (unsigned)(iw0 + t[e].w) < (unsigned)p.W;
+            const int vo = ok ? pix4 + t[e].x : OOB;
+            if constexpr (DIRECT) {
+                lds_dma_b32(dma_in, bs + (bg * EPT + e) * LDB + seg_off, vo, t[e].y);
+            } else {
+                breg[e] = buf_load(rsrc_in, vo, t[e].y);
             }
         }
     };
-    auto store_ab = [&](int buf) {
+    auto store_ab = [&](lds_float *as, lds_float *bs) {
+        if constexpr (!DIRECT) {
 #pragma unroll
-        for (int j = 0; j < AV; j++)
-            *reinterpret_cast<floatx4 *>(&As[buf][a_lds[j]]) = areg[j];
+            for (int j = 0; j < AV; j++) {
+                as[a_lds[j] + 0] = areg[j].x;
+                as[a_lds[j] + 1] = areg[j].y;
+                as[a_lds[j] + 2] = areg[j].z;
+                as[a_lds[j] + 3] = areg[j].w;
+            }
 #pragma unroll
-        for (int e = 0; e < EPT; e++) Bs[buf][(bg * EPT + e) * LDB + bn_l] = breg[e];
+            for (int e = 0; e < EPT; e++) bs[(bg * EPT + e) * LDB + bn_l] = breg[e];
+        }
     };
 
     floatx16 acc[TM][TN];
@@ -638,43 +692,53 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.0f;
 
-    load_a(step_lo);
-    load_b(step_lo);
-    store_ab(0);
-    __syncthreads();
-
     const int a_off = (lane >> 5) * LDA + wm * TM * 32 + (lane & 31);
     const int b_off = (lane >> 5) * LDB + wn * TN * 32 + (lane & 31);
+    auto as_of = [&](int buf) { return (lds_float *)&As[buf][0]; };
+    auto bs_of = [&](int buf) { return (lds_float *)&Bs[buf][0]; };
+
+    load_a(step_lo, as_of(0));
+    load_b(step_lo, bs_of(0));
+    store_ab(as_of(0), bs_of(0));
+    if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's LDS-direct loads have landed
+    __syncthreads();
 
     for (int step = step_lo; step < step_hi; step++) {
         const int buf = (step - step_lo) & 1;
         const bool more = step + 1 < step_hi;
+        const lds_float *__restrict__ a_cur = as_of(buf);
+        const lds_float *__restrict__ b_cur = bs_of(buf);
         if (more) {
-            load_a(step + 1);
-            load_b(step + 1);
+            load_a(step + 1, as_of(buf ^ 1));
+            load_b(step + 1, bs_of(buf ^ 1));
         }
         // operands of tap pair ks+1 are read from LDS while the MFMAs of pair ks run
         float a[2][TM], b[2][TN];
 #pragma unroll
-        for (int tm = 0; tm < TM; tm++) a[0][tm] = As[buf][a_off + tm * 32];
+        for (int tm = 0; tm < TM; tm++) a[0][tm] = a_cur[a_off + tm * 32];
 #pragma unroll
-        for (int tn = 0; tn < TN; tn++) b[0][tn] = Bs[buf][b_off + tn * 32];
+        for (int tn = 0; tn < TN; tn++) b[0][tn] = b_cur[b_off + tn * 32];
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
         for (int ks = 0; ks < BK / 2; ks++) {
             const int cur = ks & 1, nxt = cur ^ 1;
             if (ks + 1 < BK / 2) {
 #pragma unroll
-                for (int tm = 0; tm < TM; tm++) a[nxt][tm] = As[buf][(ks + 1) * 2 * LDA + a_off + tm * 32];
+                for (int tm = 0; tm < TM; tm++) a[nxt][tm] = a_cur[(ks + 1) * 2 * LDA + a_off + tm * 32];
 #pragma unroll
-                for (int tn = 0; tn < TN; tn++) b[nxt][tn] = Bs[buf][(ks + 1) * 2 * LDB + b_off + tn * 32];
+                for (int tn = 0; tn < TN; tn++) b[nxt][tn] = b_cur[(ks + 1) * 2 * LDB + b_off + tn * 32];
             }
 #pragma unroll
             for (int tm = 0; tm < TM; tm++)
 #pragma unroll
                 for (int tn = 0; tn < TN; tn++)
                     acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][tm], b[cur][tn], acc[tm][tn], 0, 0, 0);
+            if (ks + 1 < BK / 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
         }
-        if (more) store_ab(buf ^ 1);
+        if (more) store_ab(as_of(buf ^ 1), bs_of(buf ^ 1));
+        // the barrier publishes the next buffer: this wavefront's LDS-direct loads into it must be complete
+        if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
     }
 
@@ -795,9 +859,11 @@ struct Variant {
         "conv_tap_kernel<" #WM "," #WN "," #TM "," #TN "," #R "," #S "," #CPB "," #D ">", WM *TM * 32, WN *TN * 32, CPB,       \
             conv_tap_kernel<WM, WN, TM, TN, R, S, CPB, D>, conv_reduce_kernel<WM, WN, TM, TN>, 0                              \
     }
-#define GEN(WM, WN, TM, TN) \
-    { "conv_gen_kernel<" #WM "," #WN "," #TM "," #TN ">", WM *TM * 32, WN *TN * 32, 0, conv_gen_kernel<WM, WN, TM, TN>, \
-      conv_reduce_kernel<WM, WN, TM, TN>, 0 }
+#define GEN(WM, WN, TM, TN, D)                                                                                     \
+    {                                                                                                              \
+        "conv_gen_kernel<" #WM "," #WN "," #TM "," #TN "," #D ">", WM *TM * 32, WN *TN * 32, 0,                     \
+            conv_gen_kernel<WM, WN, TM, TN, D>, conv_reduce_kernel<WM, WN, TM, TN>, 0                              \
+    }
 
 // Per filter shape: [gather kind: register-staged, LDS-direct][tile: 128x128, 64x128, 64x64, 32x128]
 const Variant k3x3[2][4] = {
@@ -809,7 +875,8 @@ const Variant k1x1[2][4] = {
 const Variant k2x2[2][4] = {
     {TAP(2, 2, 2, 2, 2, 2, 4, false), TAP(1, 4, 2, 1, 2, 2, 4, false), TAP(2, 2, 1, 1, 2, 2, 4, false), TAP(1, 4, 1, 1, 2, 2, 4, false)},
     {TAP(2, 2, 2, 2, 2, 2, 4, true), TAP(1, 4, 2, 1, 2, 2, 4, true), TAP(2, 2, 1, 1, 2, 2, 4, true), TAP(1, 4, 1, 1, 2, 2, 4, true)}};
-const Variant kgen[4] = {GEN(2, 2, 2, 2), GEN(1, 4, 2, 1), GEN(2, 2, 1, 1), GEN(1, 4, 1, 1)};
+const Variant kgen[2][4] = {{GEN(2, 2, 2, 2, false), GEN(1, 4, 2, 1, false), GEN(2, 2, 1, 1, false), GEN(1, 4, 1, 1, false)},
+                            {GEN(2, 2, 2, 2, true), GEN(1, 4, 2, 1, true), GEN(2, 2, 1, 1, true), GEN(1, 4, 1, 1, true)}};
 
 // Launch plan: tile shape and, for the tiles that do not divide evenly over the CUs, the number
 // of K slices.  The MFMA pipe of a CU is shared by its resident workgroups, so a launch takes as
@@ -1104,7 +1171,7 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     if (R == 3 && S == 3) family = k3x3[direct];
     else if (R == 1 && S == 1) family = k1x1[direct];
     else if (R == 2 && S == 2) family = k2x2[direct];
-    else family = kgen;
+    else family = kgen[direct];
     for (int t = 0; t < 4; t++) {
         if (family[t].occupancy == 0) {
             int occ = 0;
@@ -1144,12 +1211,18 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
         }
     }
     const size_t wp_bytes = cached ? 0 : (((size_t)rows * p.Mp * sizeof(float) + 255) & ~(size_t)255);
+    const size_t taps_bytes = v->cpb ? 0 : (((size_t)rows * sizeof(int32x4) + 255) & ~(size_t)255);
     const size_t partial_bytes = (size_t)nslices * leftover * tile_floats * sizeof(float);
     void *ws = nullptr;
-    EH_TRY(get_workspace(dev, wp_bytes + partial_bytes, &ws));
+    EH_TRY(get_workspace(dev, wp_bytes + taps_bytes + partial_bytes, &ws));
     p.Wp = cached ? cached : (const float *)ws;
     p.wp_bytes = (unsigned)((size_t)rows * p.Mp * sizeof(float));
-    p.partial = (float *)((char *)ws + wp_bytes);
+    p.taps = (const int32x4 *)((char *)ws + wp_bytes);
+    p.partial = (float *)((char *)ws + wp_bytes + taps_bytes);
+    if (taps_bytes) {
+        hipLaunchKernelGGL(tap_table_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, (int32x4 *)((char *)ws + wp_bytes), rows, C, R, S, W, H * W);
+        EH_CHECK_LAUNCH();
+    }
     if (!cached) {
         hipLaunchKernelGGL(pack_filters_kernel, dim3((rows + 31) / 32, p.Mp / 32), dim3(256), 0, st, K, (float *)ws, Kf, p.CRS, p.Mp, rows);
         EH_CHECK_LAUNCH();
