@@ -224,6 +224,90 @@ __device__ __forceinline__ void stage_channel_constants(const ConvParams &p, flo
     put_channel_constants<BM>(epi, fetch_channel_constants<BM>(p, m0, tid), tid);
 }
 
+// The common case of store_tile below: every row and every pixel of the wavefront's blocks exists.
+// No per-value bounds tests; one 64-bit address per pixel column, advanced by whole channel planes;
+// the channel constants of four consecutive rows come from LDS in one read; which of batch norm,
+// affine, residual and ReLU apply is decided once per group of four rows (the flags are the same for
+// every lane) instead of once per value.  The arithmetic per value is that of store_tile, step by step.
+template <int TM, int TN, int BM>
+__device__ __forceinline__ void store_tile_inside(const ConvParams &p, floatx16 (&acc)[TM][TN], const float *epi, int m0, int m_local,
+                                                  int n_base, int lane) {
+    const int half = lane >> 5;
+    float *optr[TN];
+    const float *rptr[TN];
+    const size_t plane = (size_t)p.PQ;
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+        const unsigned n = (unsigned)(n_base + tn * 32 + (lane & 31));
+        const unsigned img = n / (unsigned)p.PQ;
+        const unsigned pq = n - img * (unsigned)p.PQ;
+        const size_t idx = ((size_t)img * p.Kf + (size_t)(m0 + m_local + 4 * half)) * plane + pq;
+        optr[tn] = p.O + idx;
+        rptr[tn] = p.residual + idx;  // not dereferenced without a residual
+    }
+    const bool has_bias = p.bias != nullptr, has_bn = p.bn_mean != nullptr, affine = p.bn_g != nullptr;
+    const bool has_res = p.residual != nullptr, relu = p.relu != 0;
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {  // rows 8*q4 + 4*half + 0..3 of the block: v = 4*q4 + j
+            const int row0 = m_local + tm * 32 + 8 * q4 + 4 * half;
+            const size_t roff = (size_t)(tm * 32 + 8 * q4) * plane;
+            float res[4][TN];
+            if (has_res) {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) res[j][tn] = rptr[tn][roff + (size_t)j * plane];
+            }
+            float x[4][TN];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) x[j][tn] = acc[tm][tn][4 * q4 + j];
+            if (has_bias) {
+                const floatx4 bias = *reinterpret_cast<const floatx4 *>(epi + row0);
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) x[j][tn] = __fadd_rn(x[j][tn], bias[j]);
+            }
+            if (has_bn) {
+                const floatx4 mean = *reinterpret_cast<const floatx4 *>(epi + BM + row0);
+                const floatx4 sd = *reinterpret_cast<const floatx4 *>(epi + 2 * BM + row0);
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) x[j][tn] = __fdiv_rn(__fsub_rn(x[j][tn], mean[j]), sd[j]);
+                if (affine) {
+                    const floatx4 g = *reinterpret_cast<const floatx4 *>(epi + 3 * BM + row0);
+                    const floatx4 b = *reinterpret_cast<const floatx4 *>(epi + 4 * BM + row0);
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int tn = 0; tn < TN; tn++) x[j][tn] = __fadd_rn(__fmul_rn(x[j][tn], g[j]), b[j]);
+                }
+            }
+            if (has_res) {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) x[j][tn] = __fadd_rn(x[j][tn], res[j][tn]);
+            }
+            if (relu) {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) x[j][tn] = x[j][tn] > 0.0f ? x[j][tn] : 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) optr[tn][roff + (size_t)j * plane] = x[j][tn];
+        }
+    }
+}
+
 // Writes a wavefront's TM x TN blocks.  A lane holds column (pixel) lane%32 and rows
 // 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 block: for a fixed v the 32 lanes of a half
 // wavefront store 32 consecutive pixels of one channel plane (128 contiguous bytes).
@@ -233,6 +317,10 @@ __device__ __forceinline__ void stage_channel_constants(const ConvParams &p, flo
 template <int TM, int TN, int BM>
 __device__ __forceinline__ void store_tile(const ConvParams &p, floatx16 (&acc)[TM][TN], const float *epi, int m0, int m_local, int n_base,
                                            int lane) {
+    if (m0 + m_local + TM * 32 <= p.Kf && (long long)n_base + TN * 32 <= p.npix) {
+        store_tile_inside<TM, TN, BM>(p, acc, epi, m0, m_local, n_base, lane);
+        return;
+    }
     size_t obase[TN];
     bool nok[TN];
 #pragma unroll
