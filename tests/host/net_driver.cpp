@@ -202,8 +202,38 @@ static int onnx(int argc, char **argv) {
     return 0;
 }
 
+// onnxinfo <file.onnx> [<re-export.onnx>]: imports the file on the host (no GPU is touched) and prints one line
+// per layer: kind, name, output shape, and per parameter its size and the sum of its values; with a second
+// argument the imported net is written back out as ONNX.
+static int onnxinfo(int argc, char **argv) {
+    if (argc < 3) {
+        fprintf(stderr, "usage: net_driver onnxinfo <file.onnx> [<re-export.onnx>]\n");
+        return 2;
+    }
+    try {
+        model m = eddl_hip::import_net_from_onnx_file(argv[2]);
+        for (Layer *l : m->layers) {
+            printf("layer %s %s", l->kind().c_str(), l->name.c_str());
+            for (int d : l->output->shape) printf(" %d", d);
+            for (Tensor *t : l->params) {
+                double sum = 0.0;
+                for (unsigned long i = 0; i < t->size; i++) sum += t->ptr[i];
+                printf(" | %lu %.9g", t->size, sum);
+            }
+            printf("\n");
+        }
+        if (argc > 3) eddl_hip::save_net_to_onnx_file(m, argv[3]);
+        delete m;
+    } catch (const std::exception &e) {
+        fprintf(stderr, "exception: %s\n", e.what());
+        return 1;
+    }
+    return 0;
+}
+
 int main(int argc, char **argv) {
     if (argc >= 2 && !strcmp(argv[1], "errors")) return errors();
+    if (argc >= 2 && !strcmp(argv[1], "onnxinfo")) return onnxinfo(argc, argv);
     if (argc >= 2 && !strcmp(argv[1], "onnx")) return onnx(argc, argv);
     if (argc < 7) {
         fprintf(stderr, "usage: net_driver <model> <params.bin|-> <input.raw> <output.raw> <batch> <size> [model arguments]\n");

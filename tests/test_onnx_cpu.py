@@ -223,3 +223,79 @@ def test_pools_refuse_asymmetric_paddings_like_the_reference():
     assert e.value.pads == [0, 1, 0, 1]
     with pytest.raises(N.AsymmetricPaddingException):
         N.AveragePool2D(x, [2, 2], [2, 2], [0, 1, 0, 1])
+
+
+# ---------------------------------------------------------------------------- the C++ importer / exporter (host only)
+NET_DRIVER = os.path.join(os.path.dirname(HERE), "eddl_amd", "host", "net_driver")
+
+
+def cpp_onnxinfo(path, back=None):
+    import subprocess
+    if not os.path.exists(NET_DRIVER):
+        subprocess.run(["make", "-C", os.path.dirname(NET_DRIVER), "all"], check=True, stdout=subprocess.DEVNULL)
+    res = subprocess.run([NET_DRIVER, "onnxinfo", str(path)] + ([str(back)] if back else []), stdout=subprocess.PIPE,
+                         stderr=subprocess.PIPE, text=True, timeout=120)
+    return res
+
+
+def layer_lines(net):
+    """What `net_driver onnxinfo` prints for a net, computed from the Python graph."""
+    out = []
+    for l in net.layers:
+        fields = ["layer", l.kind, l.name] + [str(d) for d in l.out_shape]
+        line = " ".join(fields)
+        for key, v in l.params.items():
+            if key == "bias" and l.kind == "dense" and not l.attrs["use_bias"]:
+                continue  # the C++ LDense owns no bias tensor then
+            line += " | %d %.9g" % (v.size, float(np.sum(v.astype(np.float64))))
+        out.append(line)
+    return out
+
+
+@pytest.mark.parametrize("name", sorted(EXPECTED_KINDS))
+def test_cpp_importer_builds_the_same_graph_as_the_python_importer(name, tmp_path):
+    path = os.path.join(FIX, name + ".onnx")
+    res = cpp_onnxinfo(path, tmp_path / "back.onnx")
+    assert res.returncode == 0, res.stderr[-2000:]
+    want = layer_lines(O.import_net_from_onnx_file(path))
+    got = [l for l in res.stdout.splitlines() if l.startswith("layer ")]
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        gk, wk = g.split(" | "), w.split(" | ")
+        assert gk[0] == wk[0] and len(gk) == len(wk), (g, w)
+        for a, b in zip(gk[1:], wk[1:]):  # parameter size exact, sum of values to float printing
+            assert a.split()[0] == b.split()[0] and abs(float(a.split()[1]) - float(b.split()[1])) <= 1e-6 * max(1.0, abs(float(b.split()[1]))), (g, w)
+    # what the C++ exporter wrote comes back through the Python importer with the same layers and parameters
+    net, back = O.import_net_from_onnx_file(path), O.import_net_from_onnx_file(str(tmp_path / "back.onnx"))
+    assert [(l.kind, l.name, l.out_shape) for l in back.layers] == [(l.kind, l.name, l.out_shape) for l in net.layers]
+    for a, b in zip(net.layers, back.layers):
+        for key in a.params:
+            if key == "bias" and not (a.attrs["cd"].use_bias if a.kind == "conv2d" else a.attrs.get("use_bias", True)):
+                continue
+            assert np.array_equal(a.params[key], b.params[key]), (a.name, key)
+
+
+def test_cpp_importer_repairs_and_errors(tmp_path):
+    rng = np.random.default_rng(6)
+    K = rng.standard_normal((4, 2, 2, 2)).astype(np.float32)
+    conv = O._node("Conv", "c", ["x", "c_W"], ["c"], [("kernel_shape", [2, 2]), ("pads", [0, 0, 1, 1]), ("strides", [1, 1])])
+    add = O._node("Add", "a", ["c", "b"], ["a"])
+    pool = O._node("AveragePool", "p", ["a"], ["p"], [("kernel_shape", [2, 2]), ("pads", [1, 0, 0, 1]), ("strides", [2, 2])])
+    data = tiny_model([conv, add, pool], [O._tensor("c_W", K), O._tensor("b", np.float32([1, 2, 3, 4]))], [2, 6, 6], "p", [4, 3, 3])
+    (tmp_path / "m.onnx").write_bytes(data)
+    res = cpp_onnxinfo(tmp_path / "m.onnx")
+    assert res.returncode == 0, res.stderr[-2000:]
+    want = layer_lines(O.import_net_from_onnx_bytes(data))
+    assert [l for l in res.stdout.splitlines() if l.startswith("layer ")] == want
+    assert [w.split()[1:3] for w in want] == [["input", "x"], ["pad", "c__asymmetric_padding"], ["conv2d", "c"],
+                                             ["pad", "p__asymmetric_padding"], ["avgpool2d", "p"]]
+    assert want[2].endswith("| 4 10")  # the added constant became the convolution's bias
+    # refused nodes and broken files raise the reference's error, not a crash
+    (tmp_path / "bad.onnx").write_bytes(tiny_model([O._node("LSTM", "r", ["x"], ["r"])], [], [4, 4], "r", [4]))
+    res = cpp_onnxinfo(tmp_path / "bad.onnx")
+    assert res.returncode == 1 and "ONNX::ImportNet" in res.stderr
+    (tmp_path / "cut.onnx").write_bytes(open(os.path.join(FIX, "vgg_like.onnx"), "rb").read()[:3000])
+    res = cpp_onnxinfo(tmp_path / "cut.onnx")
+    assert res.returncode == 1 and "ONNX::ImportNet" in res.stderr
+    res = cpp_onnxinfo(tmp_path / "absent.onnx")
+    assert res.returncode == 1 and "ONNX::ImportNet" in res.stderr
