@@ -624,8 +624,9 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
 }
 
 // ---------------------------------------------------------------- MFMA kernel, any filter shape
-// K-step = 16 taps.  Thread t gathers pixel t % BN for EPT consecutive taps of the step; the tap
-// walk (c, ky, kx) is uniform in a wavefront and advances with scalar arithmetic.
+// K-step = 16 taps.  Thread t gathers pixel t % BN for EPT consecutive taps of the step.  Which
+// channel, filter row and filter column a tap is does not depend on the pixel, so it is worked out
+// once per call, by tap_table_kernel, and the gather reads it back with scalar loads.
 // Tap table of conv_gen_kernel: entry k of the padded K range (k = (c*R + ky)*S + kx) holds
 // { byte offset of the tap relative to the window origin, byte offset of channel c, ky, kx }.
 // Taps past C*R*S get a row offset no image reaches, so their gathers read zeros.
