@@ -299,3 +299,67 @@ def test_cpp_importer_repairs_and_errors(tmp_path):
     assert res.returncode == 1 and "ONNX::ImportNet" in res.stderr
     res = cpp_onnxinfo(tmp_path / "absent.onnx")
     assert res.returncode == 1 and "ONNX::ImportNet" in res.stderr
+
+
+def random_net(rng):
+    """A small random graph over the layer set of the path (valid shapes by construction)."""
+    c, size = int(rng.integers(1, 5)), int(rng.integers(9, 17))
+    x = N.Input([c, size, size])
+    l, skips = x, []
+    for _ in range(int(rng.integers(2, 6))):
+        choice = rng.integers(0, 8)
+        h = l.out_shape[2]
+        if choice == 0 and h >= 6:
+            k = int(rng.integers(1, 4))
+            l = N.Conv2D(l, int(rng.integers(1, 7)), [k, k], [1, 1], "custom", bool(rng.integers(0, 2)), pads=[k // 2] * 4)
+        elif choice == 1 and h >= 6:
+            l = N.Conv2D(l, int(rng.integers(1, 7)), [3, 3], [2, 2], "custom", True, pads=[1, 1, 1, 1])
+        elif choice == 2:
+            l = N.BatchNormalization(l, True, 0.9, float(rng.choice([1e-5, 1e-3])))
+        elif choice == 3:
+            l = N.ReLu(l)
+        elif choice == 4 and h >= 4:
+            l = (N.MaxPool2D if rng.integers(0, 2) else N.AveragePool2D)(l, [2, 2], [2, 2], [0, 0, 0, 0])
+        elif choice == 5 and h <= 12:
+            l = N.UpSampling2D(l, [2, 2])
+        elif choice == 6:
+            l = N.Pad(l, [int(v) for v in rng.integers(0, 3, 4)], 0.0)
+        else:
+            same = [s for s in skips if s.out_shape == l.out_shape and s is not l]
+            if same:
+                l = N.Add(l, same[0]) if rng.integers(0, 2) else N.Concat([l, same[0]])
+            else:
+                l = N.Sigmoid(l)
+        skips.append(l)
+    l = N.Dense(N.Flatten(l), int(rng.integers(2, 6)), bool(rng.integers(0, 2)))
+    net = N.Net([x], [N.Softmax(l)])
+    for layer in net.layers:
+        for key, v in layer.params.items():
+            layer.params[key] = rng.standard_normal(v.shape).astype(np.float32) + (1.5 if key == "variance" else 0.0)
+    return net
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_graphs_through_both_codecs(seed, tmp_path):
+    """Python export -> C++ import -> C++ export -> Python import: the same layers, shapes and parameters all the way."""
+    net = random_net(np.random.default_rng(100 + seed))
+    data = O.export_net_to_onnx_bytes(net)
+    (tmp_path / "a.onnx").write_bytes(data)
+    res = cpp_onnxinfo(tmp_path / "a.onnx", tmp_path / "b.onnx")
+    assert res.returncode == 0, res.stderr[-2000:]
+    first = O.import_net_from_onnx_bytes(data)
+    assert [(l.kind, l.out_shape) for l in first.layers] == [(l.kind, l.out_shape) for l in net.layers]
+    got = [l for l in res.stdout.splitlines() if l.startswith("layer ")]
+    want = layer_lines(first)
+    assert [g.split(" | ")[0] for g in got] == [w.split(" | ")[0] for w in want]
+    second = O.import_net_from_onnx_file(str(tmp_path / "b.onnx"))
+    assert [(l.kind, l.name, l.out_shape) for l in second.layers] == [(l.kind, l.name, l.out_shape) for l in first.layers]
+    for a, b in zip(first.layers, second.layers):
+        for key in a.params:
+            if key == "bias" and not (a.attrs["cd"].use_bias if a.kind == "conv2d" else a.attrs.get("use_bias", True)):
+                continue
+            assert np.array_equal(a.params[key], b.params[key]), (a.name, key)
+        if a.kind == "conv2d":
+            assert (a.attrs["cd"].pads, a.attrs["cd"].sr) == (b.attrs["cd"].pads, b.attrs["cd"].sr)
+        if a.kind == "pad":
+            assert a.attrs["pads"] == b.attrs["pads"]
