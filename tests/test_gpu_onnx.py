@@ -49,3 +49,21 @@ def test_exported_network_comes_back_with_the_same_outputs(hip):
     back = O.import_net_from_onnx_bytes(O.export_net_to_onnx_bytes(m))
     back.build(hip)
     assert np.array_equal(back.predict([x])[0], want)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_graphs_on_the_device(hip, oracle, seed):
+    """Random small graphs over the whole layer set (tests/test_onnx_cpu.py:random_net), sent through the
+    exporter and the importer first: the layer walk agrees with the CPU oracle, the fused plan with the
+    layer walk bit for bit, whatever chains the graph happens to contain."""
+    from test_onnx_cpu import random_net
+    rng = np.random.default_rng(500 + seed)
+    net = O.import_net_from_onnx_bytes(O.export_net_to_onnx_bytes(random_net(rng)))
+    x = rng.standard_normal([3] + net.lin[0].out_shape[1:]).astype(np.float32)
+    want = net_oracle.forward(oracle, net, [x], conv_algo="direct")[0]
+    net.build(hip, fuse=False)
+    plain = net.predict([x])[0]
+    assert plain.shape == want.shape
+    assert np.all(np.abs(plain - want) <= 1e-5 * np.abs(want).max() + 2e-4 * np.abs(want)), np.abs(plain - want).max()
+    net.build(hip, fuse=True)
+    assert np.array_equal(net.predict([x])[0], plain)

@@ -306,8 +306,8 @@ def random_net(rng):
     c, size = int(rng.integers(1, 5)), int(rng.integers(9, 17))
     x = N.Input([c, size, size])
     l, skips = x, []
-    for _ in range(int(rng.integers(2, 6))):
-        choice = rng.integers(0, 8)
+    for _ in range(int(rng.integers(3, 9))):
+        choice = rng.integers(0, 10)
         h = l.out_shape[2]
         if choice == 0 and h >= 6:
             k = int(rng.integers(1, 4))
@@ -320,6 +320,8 @@ def random_net(rng):
             l = N.ReLu(l)
         elif choice == 4 and h >= 4:
             l = (N.MaxPool2D if rng.integers(0, 2) else N.AveragePool2D)(l, [2, 2], [2, 2], [0, 0, 0, 0])
+        elif choice == 7:
+            l = N.BatchNormalization(N.ReLu(l), True, 0.9, 1e-5)  # two shape-keeping layers: partners for a later add / concat
         elif choice == 5 and h <= 12:
             l = N.UpSampling2D(l, [2, 2])
         elif choice == 6:
@@ -339,7 +341,7 @@ def random_net(rng):
     return net
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(30))
 def test_random_graphs_through_both_codecs(seed, tmp_path):
     """Python export -> C++ import -> C++ export -> Python import: the same layers, shapes and parameters all the way."""
     net = random_net(np.random.default_rng(100 + seed))
