@@ -337,7 +337,8 @@ def random_net(rng):
     net = N.Net([x], [N.Softmax(l)])
     for layer in net.layers:
         for key, v in layer.params.items():
-            layer.params[key] = rng.standard_normal(v.shape).astype(np.float32) + (1.5 if key == "variance" else 0.0)
+            w = rng.standard_normal(v.shape).astype(np.float32)
+            layer.params[key] = np.abs(w) + 0.5 if key == "variance" else w * np.float32(0.5)
     return net
 
 
