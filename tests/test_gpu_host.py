@@ -209,3 +209,26 @@ def test_cpp_onnx_import_matches_pytorch_and_the_python_importer(hip, name, fuse
             if key == "bias" and not (a.attrs["cd"].use_bias if a.kind == "conv2d" else a.attrs.get("use_bias", True)):
                 continue
             assert np.array_equal(a.params[key], b.params[key]), (a.name, key)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_cpp_fused_plan_on_random_graphs(hip, seed, tmp_path):
+    """Random graphs (tests/test_onnx_cpu.py:random_net) written to ONNX, imported by the C++ host layer and
+    run through Net::fuse: bit for bit what the Python layer walk computes, so the C++ chain rules
+    (pad folding, batch norm, LSum / LAdd + ReLU, dense + ReLU) hold on graphs nobody wrote by hand."""
+    from eddl_amd import onnx_io
+    from test_onnx_cpu import random_net
+    rng = np.random.default_rng(900 + seed)
+    data = onnx_io.export_net_to_onnx_bytes(random_net(rng))
+    (tmp_path / "g.onnx").write_bytes(data)
+    net = onnx_io.import_net_from_onnx_bytes(data)
+    x = rng.standard_normal([3] + net.lin[0].out_shape[1:]).astype(np.float32)
+    x.tofile(tmp_path / "x.raw")
+    for fused in (0, 1):
+        out = run_net_driver(["onnx", tmp_path / "g.onnx", tmp_path / "x.raw", tmp_path / ("y%d.raw" % fused), 3, fused])
+        assert "FAILED" not in out, out
+    net.build(hip, fuse=False)
+    want = net.predict([x])[0]
+    for fused in (0, 1):
+        got = np.fromfile(tmp_path / ("y%d.raw" % fused), np.float32).reshape(want.shape)
+        assert np.array_equal(got, want), (fused, np.abs(got - want).max())

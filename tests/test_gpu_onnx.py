@@ -51,7 +51,7 @@ def test_exported_network_comes_back_with_the_same_outputs(hip):
     assert np.array_equal(back.predict([x])[0], want)
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(48))
 def test_random_graphs_on_the_device(hip, oracle, seed):
     """Random small graphs over the whole layer set (tests/test_onnx_cpu.py:random_net), sent through the
     exporter and the importer first: the layer walk agrees with the CPU oracle, the fused plan with the
