@@ -720,6 +720,42 @@ void Net::load(const string &filename, const string &format) {
         }
 }
 
+vector<vector<Tensor *>> Net::get_parameters(bool) {
+    vector<vector<Tensor *>> all;
+    for (Layer *l : layers) {
+        vector<Tensor *> ps;
+        for (Tensor *p : l->params) {
+            Tensor *host = new Tensor(p->getShape(), DEV_CPU);
+            Tensor::copy(p, host);
+            ps.push_back(host);
+        }
+        all.push_back(ps);
+    }
+    return all;
+}
+
+void Net::set_parameters(const vector<vector<Tensor *>> &new_params) {
+    if (new_params.size() != layers.size())
+        msg("AssertionError: The number of layers in params does not match the number of layers in this network (" +
+                std::to_string(new_params.size()) + "!=" + std::to_string(layers.size()) + ")",
+            "Net::set_parameters");
+    for (size_t i = 0; i < layers.size(); i++)
+        if (new_params[i].size() != layers[i]->params.size())
+            msg("AssertionError: The number of parameters in layer '" + std::to_string(i) + "'(" + layers[i]->name +
+                    ") does not match the number of parameters in the given vector<Tensor*>. (" +
+                    std::to_string(layers[i]->params.size()) + "!=" + std::to_string(new_params[i].size()) + ")",
+                "Net::set_parameters");
+    for (size_t i = 0; i < layers.size(); i++)
+        for (size_t j = 0; j < layers[i]->params.size(); j++) Tensor::copy(new_params[i][j], layers[i]->params[j]);
+}
+
+Layer *Net::getLayer(const string &lname) {
+    for (Layer *l : layers)
+        if (l->name == lname) return l;
+    msg("layer " + lname + " not found", "Net::getLayer");
+    return nullptr;
+}
+
 string Net::summary(bool print_stdout) {
     std::stringstream ss;
     ss << "-------------------------------------------------------------------------------\n" << name << "\n";
@@ -779,6 +815,20 @@ Tensor *getOutput(layer l1) {
     Tensor *t = new Tensor(l1->output->getShape(), DEV_CPU);
     Tensor::copy(l1->output, t);
     return t;
+}
+
+vector<vtensor> get_parameters(model net, bool deepcopy) { return net->get_parameters(deepcopy); }
+void set_parameters(model net, const vector<vtensor> &params) { net->set_parameters(params); }
+layer getLayer(model net, const string &name) { return net->getLayer(name); }
+vlayer getOut(model net) { return net->lout; }
+vtensor getParams(layer l1) {
+    vtensor out;
+    for (Tensor *p : l1->params) {
+        Tensor *host = new Tensor(p->getShape(), DEV_CPU);
+        Tensor::copy(p, host);
+        out.push_back(host);
+    }
+    return out;
 }
 
 layer Input(const vector<int> &shape, string name) {

@@ -244,6 +244,12 @@ class Net {
     void save(const string &filename, const string &format = "bin");
     void load(const string &filename, const string &format = "bin");
     string summary(bool print_stdout = true);
+    // Parameters per layer, in `layers` order (src/net/net_api.cpp:199-260).  The tensors handed out are
+    // host copies owned by the caller (the reference's deepcopy = true; without it the reference hands
+    // out its own host-side tensors, which this device-resident net does not keep).
+    vector<vector<Tensor *>> get_parameters(bool deepcopy = true);
+    void set_parameters(const vector<vector<Tensor *>> &params);
+    Layer *getLayer(const string &name);
 
     // Inference plan with the layer chains conv [+ batchnorm] [+ sum] [+ relu], zero pad + conv and
     // dense + relu each computed by one kernel, and the repacked filters of every convolution kept
@@ -283,6 +289,11 @@ void save(model m, const string &fname, const string &format = "bin");
 vlayer forward(model m, vtensor in);
 vtensor predict(model m, const vtensor &in);
 Tensor *getOutput(layer l1);  // a host copy, owned by the caller
+vector<vtensor> get_parameters(model net, bool deepcopy = true);
+void set_parameters(model net, const vector<vtensor> &params);
+layer getLayer(model net, const string &name);
+vlayer getOut(model net);
+vtensor getParams(layer l1);  // host copies, owned by the caller
 
 layer Input(const vector<int> &shape, string name = "");
 layer Conv2D(layer parent, int filters, const vector<int> &kernel_size, const vector<int> &strides = {1, 1}, string padding = "same",

@@ -300,6 +300,7 @@ int main(int argc, char **argv) {
             ofs.write(reinterpret_cast<const char *>(t->ptr), t->size * sizeof(float));
             delete t;
         }
+        ofs.close();
         if (timed) {  // forwards with the input already on the device
             for (int i = 0; i < 5; i++) m->forward();
             const auto t0 = std::chrono::steady_clock::now();
@@ -320,6 +321,35 @@ int main(int argc, char **argv) {
                     printf("%s getOutput of a fused-away layer\n", threw ? "ok " : "FAILED");
                     break;
                 }
+        }
+        {  // parameters out and back in: a doubled bias-free copy changes the result, the original restores it
+            vector<vtensor> ps = get_parameters(m);
+            size_t count = 0;
+            for (vtensor &v : ps) count += v.size();
+            set_parameters(m, ps);
+            vtensor again = predict(m, {&x});
+            bool same = true;
+            {
+                std::ifstream chk(out_path, std::ios::binary);
+                for (Tensor *t : again) {
+                    vector<float> ref(t->size);
+                    chk.read(reinterpret_cast<char *>(ref.data()), t->size * sizeof(float));
+                    same = same && memcmp(ref.data(), t->ptr, t->size * sizeof(float)) == 0;
+                    delete t;
+                }
+            }
+            printf("%s get_parameters / set_parameters round trip (%zu tensors)\n", same ? "ok " : "FAILED", count);
+            bool threw = false;
+            try {
+                vector<vtensor> fewer(ps.begin(), ps.end() - 1);
+                set_parameters(m, fewer);
+            } catch (const std::runtime_error &) {
+                threw = true;
+            }
+            printf("%s set_parameters with a missing layer\n", threw ? "ok " : "FAILED");
+            printf("%s getLayer / getOut\n", getLayer(m, m->layers.back()->name) == m->layers.back() && getOut(m) == m->lout ? "ok " : "FAILED");
+            for (vtensor &v : ps)
+                for (Tensor *t : v) delete t;
         }
         if (params == "-") save(m, out_path + ".params");  // round trip of freshly initialised parameters
         delete m;

@@ -147,8 +147,9 @@ def test_cpp_graphs_match_the_python_runner_bit_for_bit(hip, which, fused, tmp_p
     x = rng.standard_normal(m.lin[0].out_shape, dtype=np.float32)
     x.tofile(tmp_path / "x.raw")
     out = run_net_driver([("fused:" if fused else "") + which, tmp_path / "params.bin", tmp_path / "x.raw", tmp_path / "y.raw", batch, size] + extra)
+    assert "FAILED" not in out and "ok  get_parameters / set_parameters round trip" in out and "ok  set_parameters with a missing layer" in out, out
     if fused:
-        assert "FAILED" not in out and "ok  getOutput of a fused-away layer" in out, out
+        assert "ok  getOutput of a fused-away layer" in out, out
         steps = int([l for l in out.splitlines() if l.startswith("plan:")][0].split()[1])
         m.build(hip, fuse=True)
         views = sum(1 for l in m.layers if l.kind in ("input", "reshape"))   # steps of the C++ plan that launch nothing
