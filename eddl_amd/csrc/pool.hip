@@ -229,6 +229,24 @@ __global__ __launch_bounds__(TPB) void avgpool_kernel(const float *__restrict__ 
     }
 }
 
+// Window = the whole plane, no padding (GlobalAveragePool2D): one wavefront takes 64 planes, which
+// are contiguous in memory, reads them with coalesced loads into LDS (row stride odd: no bank
+// conflicts), and each lane then adds up its own plane in the same sequential order as above.
+__global__ __launch_bounds__(64) void avgpool_plane_kernel(const float *__restrict__ I, float *__restrict__ O, size_t planes, int hw) {
+    extern __shared__ float plane_tile[];
+    const int lane = threadIdx.x, row = hw | 1;
+    const size_t p0 = (size_t)blockIdx.x * 64;
+    const int here = (int)(planes - p0 < 64 ? planes - p0 : 64);
+    const float *src = I + p0 * hw;
+    for (int i = lane; i < here * hw; i += 64) plane_tile[(i / hw) * row + i % hw] = src[i];
+    __syncthreads();
+    if (lane < here) {
+        float sum = 0.0f;
+        for (int k = 0; k < hw; k++) sum = __fadd_rn(sum, plane_tile[lane * row + k]);
+        O[p0 + lane] = __fdiv_rn(sum, (float)hw);
+    }
+}
+
 int loop_count(int in, int k, int stride, int pad_lo, int pad_hi) {
     long long last = (long long)in + pad_hi - k, first = -(long long)pad_lo;
     if (last < first) return 0;
@@ -294,7 +312,14 @@ int eddlhip_avgpool2d(int dev, const float *I, float *O, int N, int C, int H, in
     if (total == 0) return 0;
     EH_REQUIRE(I && O, "avgpool2d: NULL tensor");
     EH_TRY(use_device(dev));
-    hipLaunchKernelGGL(avgpool_kernel, dim3(eh_blocks(total, TPB, 1u << 18)), dim3(TPB), 0, state(dev).stream, I, O, total, s);
+    const bool whole_plane = kr == H && kc == W && pad_top == 0 && pad_bottom == 0 && pad_left == 0 && pad_right == 0 && s.LP == 1 && s.LQ == 1;
+    if (whole_plane && H * W <= 255 && total <= 0x7fffffffULL * 64) {
+        const int hw = H * W;
+        hipLaunchKernelGGL(avgpool_plane_kernel, dim3((unsigned)((total + 63) / 64)), dim3(64), (size_t)64 * (hw | 1) * sizeof(float),
+                           state(dev).stream, I, O, total, hw);
+    } else {
+        hipLaunchKernelGGL(avgpool_kernel, dim3(eh_blocks(total, TPB, 1u << 18)), dim3(TPB), 0, state(dev).stream, I, O, total, s);
+    }
     EH_CHECK_LAUNCH();
     return 0;
 }

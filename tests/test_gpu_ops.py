@@ -332,7 +332,12 @@ def test_maxpool_bit_exact_with_indices(hip, oracle):
 def test_avgpool_bit_exact(hip, oracle):
     rng = np.random.default_rng(403)
     for shape, k, s, pads in [((4, 16, 56, 56), (2, 2), (2, 2), (0, 0, 0, 0)), ((2, 8, 28, 28), (3, 3), (2, 2), (1, 1, 1, 1)),
-                              ((2, 64, 7, 7), (7, 7), (1, 1), (0, 0, 0, 0)), ((2, 4, 13, 17), (3, 2), (1, 2), (1, 0, 0, 1))]:
+                              ((2, 64, 7, 7), (7, 7), (1, 1), (0, 0, 0, 0)), ((2, 4, 13, 17), (3, 2), (1, 2), (1, 0, 0, 1)),
+                              # whole-plane windows (global average pool): ragged plane counts, even and odd plane sizes,
+                              # the largest plane of the LDS kernel and one beyond it
+                              ((3, 67, 7, 7), (7, 7), (1, 1), (0, 0, 0, 0)), ((1, 5, 8, 8), (8, 8), (1, 1), (0, 0, 0, 0)),
+                              ((2, 130, 15, 17), (15, 17), (1, 1), (0, 0, 0, 0)), ((2, 9, 16, 16), (16, 16), (1, 1), (0, 0, 0, 0)),
+                              ((1, 3, 1, 1), (1, 1), (1, 1), (0, 0, 0, 0))]:
         x = rng.standard_normal(shape, dtype=np.float32)
         ref = oracle.avgpool2d(x, k, s, pads)
         O = hip.empty(ref.shape)
