@@ -856,17 +856,35 @@ __global__ __launch_bounds__(64) void conv_reduce_kernel(const ConvParams p) {
     const int m0 = (tile % p.gm) * BM + (wm * TM + tm) * 32;
     const long long n0 = (long long)(tile / p.gm) * BN + (wn * TN + tn) * 32;
     const size_t tiles = gridDim.x / UNITS;
+    // the channel constants are asked for first; four slices' loads are in flight at a time, and the
+    // additions keep the slice order (starting from slice 0's value, not from zero)
+    const ChannelEpilogue chan = fetch_channel_constants<32>(p, m0, lane);
+    const size_t slice_stride = tiles * 4 * (TM * TN) * (16 * 64);
+    const float *src = p.partial + (((size_t)local_tile * 4 + wave) * (TM * TN) + blk) * (16 * 64) + lane;
     floatx16 acc[1][1];
-    for (int sl = 0; sl < p.nslices; sl++) {
-        const float *src = p.partial + ((((size_t)sl * tiles + local_tile) * 4 + wave) * (TM * TN) + blk) * (16 * 64) + lane;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const float x = src[v * 64];
-            acc[0][0][v] = sl == 0 ? x : __fadd_rn(acc[0][0][v], x);
-        }
+    for (int v = 0; v < 16; v++) acc[0][0][v] = src[v * 64];
+    int sl = 1;
+    for (; sl + 4 <= p.nslices; sl += 4) {
+        float x[4][16];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) x[u][v] = src[(size_t)(sl + u) * slice_stride + v * 64];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[0][0][v] = __fadd_rn(acc[0][0][v], x[u][v]);
+    }
+    for (; sl < p.nslices; sl++) {
+        float x[16];
+#pragma unroll
+        for (int v = 0; v < 16; v++) x[v] = src[(size_t)sl * slice_stride + v * 64];
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[0][0][v] = __fadd_rn(acc[0][0][v], x[v]);
     }
     __shared__ float epi[5 * 32];
-    stage_channel_constants<32>(p, epi, m0, lane);
+    put_channel_constants<32>(epi, chan, lane);
     __syncthreads();
     store_tile<1, 1, 32>(p, acc, epi, m0, 0, (int)n0, lane);
 }
