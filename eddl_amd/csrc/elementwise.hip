@@ -117,6 +117,40 @@ __global__ __launch_bounds__(64) void softmax_kernel(const float *__restrict__ A
     if (si >= n_samples) return;
     const int lane = threadIdx.x;
     const size_t start = (size_t)(si % inner) + (size_t)(si / inner) * ((size_t)len * inner);
+    if (len <= 64 * 16) {
+        // lines of up to 1024 entries stay in registers: one read, one write, the same operations in the same order
+        float v[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const int i = lane + 64 * j;
+            v[j] = i < len ? A[start + (size_t)i * inner] : 0.0f;
+        }
+        float mx = -3.40282e+38f;
+        if (stable) {
+#pragma unroll
+            for (int j = 0; j < 16; j++)
+                if (lane + 64 * j < len && v[j] > mx) mx = v[j];
+            for (int off = 32; off > 0; off >>= 1) {
+                float o = __shfl_xor(mx, off, 64);
+                if (o > mx) mx = o;
+            }
+        }
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 16; j++)
+            if (lane + 64 * j < len) {
+                v[j] = expf(v[j] - mx);
+                sum += v[j];
+            }
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+        const float den = 1.19209e-07f + sum;
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const int i = lane + 64 * j;
+            if (i < len) B[start + (size_t)i * inner] = __fdiv_rn(v[j], den);
+        }
+        return;
+    }
     float mx = -3.40282e+38f;
     if (stable) {
         for (int i = lane; i < len; i += 64) {

@@ -413,11 +413,15 @@ def test_dense_sigmoid_softmax_within_tolerance(hip, oracle):
     B = hip.empty(x.shape)
     hip.sigmoid(hip.array(x), B)
     np.testing.assert_allclose(B.numpy(), oracle.sigmoid(x), rtol=1e-6, atol=1e-7)
-    for shape, axis in [((32, 1000), 1), ((3, 7, 5, 4), 1), ((6, 1), 1)]:
+    # line lengths on both sides of the 1024 entries the register path holds, axes with and without an inner stride
+    for shape, axis in [((32, 1000), 1), ((3, 7, 5, 4), 1), ((6, 1), 1), ((5, 1024), 1), ((5, 1025), 1), ((3, 4099), 1), ((2, 1500, 3), 1),
+                        ((2, 3, 70), 2)]:
         x = rng.standard_normal(shape, dtype=np.float32) * 3
         B = hip.empty(shape)
         hip.full_softmax(hip.array(x), B, axis)
-        np.testing.assert_allclose(B.numpy(), oracle.softmax(x, axis), rtol=2e-6, atol=1e-8)
+        # the denominator is summed per lane and then across the wavefront, the oracle's sequentially: the two
+        # orders drift apart with the length of the line (2e-6 up to 1024 entries, 5e-6 at 4099)
+        np.testing.assert_allclose(B.numpy(), oracle.softmax(x, axis), rtol=2e-6 if shape[axis] <= 1024 else 5e-6, atol=1e-8)
 
 
 def test_conv2d_cached_filters_follow_every_write(hip, oracle):
