@@ -7,7 +7,11 @@ headline metric is quoted on).  Prints ONE JSON line on stdout; the per-layer ta
 stderr with --layers and to DIR/bench_layers_<workload>.{json,txt} with --out DIR.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vgg16|block|resnet50|unet]
-                    [--no-cpu-baseline] [--layers] [--out DIR]
+                    [--no-cpu-baseline] [--layers] [--out DIR] [--unfused]
+
+--unfused runs the graph layer by layer (every BatchNorm, ReLU, Add and Pad as a launch of its own, as
+the reference walks it): not the headline figure, but the run whose per-op table gives the HBM rate of
+each bandwidth kernel at the workload's real tensor sizes.
 """
 import argparse
 import json
@@ -137,6 +141,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layers", action="store_true", help="print the per-op table to stderr")
     ap.add_argument("--out", default=None, metavar="DIR", help="also write the per-op table and the result into this directory")
+    ap.add_argument("--unfused", action="store_true",
+                    help="one launch per layer (no Conv+BN+Add+ReLU / Pad / Dense+ReLU fusion): measures the stand-alone bandwidth kernels")
     ap.add_argument("--conv-algo", default="auto", choices=["auto", "mfma_staged", "mfma_lds"], help="input gather of the convolution kernels")
     ap.add_argument("--no-device-probe", action="store_true",
                     help="skip the pure-MFMA probe of the device's sustained fp32 matrix rate (keeps kernel traces to the workload)")
@@ -151,7 +157,7 @@ def main():
     hip = eddl_amd.Backend(0)
     hip.set_conv_algo(args.conv_algo)
     model, x, desc = build_workload(args.workload)
-    model.build(hip, fuse=True)
+    model.build(hip, fuse=not args.unfused)
     batch = x.shape[0]
     model.input_tensor().copy_from(x)  # input resident in HBM before the timed region
     hip.synchronize()
@@ -203,7 +209,7 @@ def main():
     achieved = dom_flops / dom_ms / 1e9 if dom_ms > 0 else 0.0
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "traffic_%s.json" % args.workload)
-    if os.path.exists(tpath):
+    if os.path.exists(tpath) and not args.unfused:  # the committed counter runs are of the fused plan
         with open(tpath) as fh:
             traffic = json.load(fh).get("hbm_bytes_per_launch")
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
@@ -225,11 +231,11 @@ def main():
     conv_ms = sum(r["ms"] for r in conv_rows)
     conv_flops = sum(r["flops"] for r in conv_rows)
     result = {
-        "metric": "%s forward images/sec (fp32, 1 GPU)" % args.workload,
+        "metric": "%s forward images/sec (fp32, 1 GPU%s)" % (args.workload, ", layer by layer" if args.unfused else ""),
         "value": batch * args.steps / wall, "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (seeded He-normal weights, U(0,1)/N(0,1) inputs, resident in HBM)",
-        "config": {"workload": desc, "batch": batch, "fused_ops": len(model.ops), "device": hip.name},
+        "config": {"workload": desc, "batch": batch, "fused": not args.unfused, "fused_ops": len(model.ops), "device": hip.name},
         "roofline": roofline,
         "conv_total": {"tflops": conv_flops / conv_ms / 1e9 if conv_ms else 0.0, "ms": conv_ms, "gflop": conv_flops / 1e9,
                        "frac_fp32_mfma_peak": (conv_flops / conv_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS) if conv_ms else 0.0},
@@ -249,9 +255,10 @@ def main():
     out_dir = args.out
     if out_dir:
         os.makedirs(out_dir, exist_ok=True)
-        with open(os.path.join(out_dir, "bench_layers_%s.json" % args.workload), "w") as fh:
+        stem = "bench_layers_%s%s" % (args.workload, "_unfused" if args.unfused else "")
+        with open(os.path.join(out_dir, stem + ".json"), "w") as fh:
             json.dump({"result": result, "ops": rows}, fh, indent=1)
-        with open(os.path.join(out_dir, "bench_layers_%s.txt" % args.workload), "w") as fh:
+        with open(os.path.join(out_dir, stem + ".txt"), "w") as fh:
             fh.write("\n".join(table) + "\n")
     print(json.dumps(result))
 

@@ -254,6 +254,30 @@ __global__ __launch_bounds__(TPB) void pad_kernel(const float *__restrict__ A, f
     }
 }
 
+// Rows of at least 64 pixels: one wavefront per source row, lanes on consecutive pixels (256 contiguous
+// bytes per load and per store, whatever the destination row's alignment), four loads in flight per
+// lane, and one division per row instead of three per pixel.
+__global__ __launch_bounds__(TPB) void pad_rows_kernel(const float *__restrict__ A, float *__restrict__ B, size_t rows, int H,
+                                                       int W, int OH, int OW, int top, int left) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    constexpr int WAVES = TPB / 64;
+    for (size_t r = (size_t)blockIdx.x * WAVES + wv; r < rows; r += (size_t)gridDim.x * WAVES) {
+        const size_t plane = r / H;
+        const int h = (int)(r - plane * H);
+        const float *src = A + r * W;
+        float *dst = B + (plane * OH + (h + top)) * OW + left;
+        int j = lane;
+        for (; j + 192 < W; j += 256) {
+            const float v0 = src[j], v1 = src[j + 64], v2 = src[j + 128], v3 = src[j + 192];
+            dst[j] = v0;
+            dst[j + 64] = v1;
+            dst[j + 128] = v2;
+            dst[j + 192] = v3;
+        }
+        for (; j < W; j += 64) dst[j] = src[j];
+    }
+}
+
 __global__ __launch_bounds__(TPB) void sum2d_rowwise_kernel(const float *A, const float *__restrict__ B, float *C,
                                                             size_t total, int cols) {
     size_t i = (size_t)blockIdx.x * TPB + threadIdx.x, stride = (size_t)gridDim.x * TPB;
@@ -427,8 +451,14 @@ int eddlhip_pad(int dev, const float *A, float *B, int N, int C, int H, int W, i
     EH_REQUIRE(A && B, "pad: NULL tensor");
     EH_TRY(use_device(dev));
     size_t total = (size_t)N * C * H * W;
-    hipLaunchKernelGGL(pad_kernel, dim3(eh_blocks(total, TPB, 1u << 18)), dim3(TPB), 0, state(dev).stream, A, B, total, H, W,
-                       H + top + bottom, W + left + right, top, left);
+    if (W >= 64) {
+        size_t rows = (size_t)N * C * H;
+        hipLaunchKernelGGL(pad_rows_kernel, dim3(eh_blocks(rows, TPB / 64, 1u << 16)), dim3(TPB), 0, state(dev).stream, A, B, rows,
+                           H, W, H + top + bottom, W + left + right, top, left);
+    } else {
+        hipLaunchKernelGGL(pad_kernel, dim3(eh_blocks(total, TPB, 1u << 18)), dim3(TPB), 0, state(dev).stream, A, B, total, H, W,
+                           H + top + bottom, W + left + right, top, left);
+    }
     EH_CHECK_LAUNCH();
     return 0;
 }

@@ -385,6 +385,15 @@ def test_upsample_concat_pad_bit_exact(hip, oracle):
     B = hip.full(ref.shape, 7.0)
     hip.pad(hip.array(x), B, (1, 2, 3, 4))
     assert np.array_equal(B.numpy(), ref)
+    # rows of 64 pixels and more take the row-per-wavefront kernel: widths around its 256-pixel step and 64-pixel remainder
+    for shape, pads in [((2, 3, 5, 64), (0, 1, 1, 0)), ((1, 2, 7, 65), (2, 0, 0, 3)), ((1, 3, 4, 255), (1, 1, 1, 1)),
+                        ((2, 1, 3, 256), (0, 1, 1, 0)), ((1, 2, 6, 449), (3, 2, 1, 5)), ((1, 1, 9, 1030), (0, 0, 0, 1)),
+                        ((1, 5, 1100, 70), (1, 0, 0, 0))]:
+        y = rng.standard_normal(shape, dtype=np.float32)
+        ref = oracle.pad(y, pads, cval=-2.0)
+        B = hip.full(ref.shape, -2.0)
+        hip.pad(hip.array(y), B, pads)
+        assert np.array_equal(B.numpy(), ref), (shape, pads)
 
 
 def test_dense_sigmoid_softmax_within_tolerance(hip, oracle):
