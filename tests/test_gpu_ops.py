@@ -305,6 +305,14 @@ def test_maxpool_bit_exact_with_indices(hip, oracle):
         ((2, 3, 57, 55), (2, 2), (2, 2), (0, 0, 0, 0)),    # odd sizes: general path
         ((2, 8, 28, 28), (3, 3), (2, 2), (1, 1, 1, 1)),    # ResNet stem pool geometry
         ((2, 4, 13, 17), (3, 3), (1, 1), (1, 1, 1, 1)),
+        # 3x3 stride 2, two outputs per thread: left pad 1 and 0, rows that end inside a wavefront, a ragged last wavefront
+        ((2, 3, 112, 112), (3, 3), (2, 2), (1, 1, 1, 1)),
+        ((2, 4, 28, 28), (3, 3), (2, 2), (0, 1, 0, 1)),
+        ((2, 2, 30, 32), (3, 3), (2, 2), (0, 1, 1, 0)),
+        ((1, 2, 12, 264), (3, 3), (2, 2), (1, 1, 1, 1)),
+        ((1, 2, 11, 264), (3, 3), (2, 2), (2, 0, 0, 1)),
+        ((1, 1, 8, 12), (3, 3), (2, 2), (1, 1, 1, 1)),
+        ((1, 3, 20, 22), (3, 3), (2, 2), (1, 1, 1, 1)),    # width not a multiple of 4: one output per thread
         ((2, 4, 12, 12), (2, 2), (2, 2), (0, 1, 0, 1)),
         ((3, 5, 7, 7), (7, 7), (1, 1), (0, 0, 0, 0)),      # 49 taps, one thread per output
         ((3, 5, 9, 9), (9, 9), (1, 1), (0, 0, 0, 0)),      # 81 taps: one wavefront per output
@@ -326,6 +334,14 @@ def test_maxpool_bit_exact_with_indices(hip, oracle):
         O_ref, ix_ref, iy_ref = oracle.maxpool2d(x, k, k, (0, 0, 0, 0), fill=-5.0)
         O, ix, iy = hip.empty(O_ref.shape), hip.full(O_ref.shape, -5.0), hip.full(O_ref.shape, -5.0)
         hip.mpool2D(hip.array(x), O, ix, iy, k, k, (0, 0, 0, 0))
+        assert np.array_equal(O.numpy(), O_ref) and np.array_equal(ix.numpy(), ix_ref) and np.array_equal(iy.numpy(), iy_ref)
+    for pads in ((1, 1, 1, 1), (0, 1, 0, 1)):  # the same through the 3x3 stride-2 kernel, half of the plane finite
+        x = np.full((1, 2, 16, 16), -np.inf, np.float32)
+        x[0, 0, :4, :4] = np.nan
+        x[0, 1, 8:, :] = rng.standard_normal((8, 16), dtype=np.float32)
+        O_ref, ix_ref, iy_ref = oracle.maxpool2d(x, (3, 3), (2, 2), pads, fill=-5.0)
+        O, ix, iy = hip.empty(O_ref.shape), hip.full(O_ref.shape, -5.0), hip.full(O_ref.shape, -5.0)
+        hip.mpool2D(hip.array(x), O, ix, iy, (3, 3), (2, 2), pads)
         assert np.array_equal(O.numpy(), O_ref) and np.array_equal(ix.numpy(), ix_ref) and np.array_equal(iy.numpy(), iy_ref)
 
 
