@@ -22,7 +22,10 @@
  *  - The library never owns user-visible tensors.  It keeps one private, grow-only
  *    workspace per device (repacked filters); eddlhip_shutdown() releases it.
  *  - Calls on one device must not overlap from several threads (the reference drives one
- *    device from one thread: src/net/net_api.cpp:146-171).
+ *    device from one thread: src/net/net_api.cpp:146-171).  Different devices may be driven
+ *    from different threads.  The tuning and measurement switches (eddlhip_conv2d_set_algo,
+ *    _force_plan, _profile, _profile_read) act on the whole process: change them only while
+ *    no other thread is inside the library.
  */
 #ifndef EDDLHIP_H
 #define EDDLHIP_H
