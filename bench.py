@@ -7,7 +7,7 @@ headline metric is quoted on).  Prints ONE JSON line on stdout; the per-layer ta
 stderr with --layers and to DIR/bench_layers_<workload>.{json,txt} with --out DIR.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vgg16|block|resnet50|unet]
-                    [--no-cpu-baseline] [--layers] [--out DIR] [--unfused]
+                    [--no-cpu-baseline] [--layers] [--out DIR] [--unfused] [--graph]
 
 --unfused runs the graph layer by layer (every BatchNorm, ReLU, Add and Pad as a launch of its own, as
 the reference walks it): not the headline figure, but the run whose per-op table gives the HBM rate of
@@ -143,6 +143,8 @@ def main():
     ap.add_argument("--out", default=None, metavar="DIR", help="also write the per-op table and the result into this directory")
     ap.add_argument("--unfused", action="store_true",
                     help="one launch per layer (no Conv+BN+Add+ReLU / Pad / Dense+ReLU fusion): measures the stand-alone bandwidth kernels")
+    ap.add_argument("--graph", action="store_true",
+                    help="record the plan once as a graph and replay it with one call per step (for plans of short kernels)")
     ap.add_argument("--conv-algo", default="auto", choices=["auto", "mfma_staged", "mfma_lds"], help="input gather of the convolution kernels")
     ap.add_argument("--no-device-probe", action="store_true",
                     help="skip the pure-MFMA probe of the device's sustained fp32 matrix rate (keeps kernel traces to the workload)")
@@ -162,12 +164,16 @@ def main():
     model.input_tensor().copy_from(x)  # input resident in HBM before the timed region
     hip.synchronize()
 
+    step = model.run
+    if args.graph:
+        model.capture()
+        step = model.run_graph
     for _ in range(args.warmup):
-        model.run()
+        step()
     hip.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        model.run()
+        step()
     hip.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
@@ -235,7 +241,7 @@ def main():
         "value": batch * args.steps / wall, "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (seeded He-normal weights, U(0,1)/N(0,1) inputs, resident in HBM)",
-        "config": {"workload": desc, "batch": batch, "fused": not args.unfused, "fused_ops": len(model.ops), "device": hip.name},
+        "config": {"workload": desc, "batch": batch, "fused": not args.unfused, "fused_ops": len(model.ops), "graph_replay": bool(args.graph), "device": hip.name},
         "roofline": roofline,
         "conv_total": {"tflops": conv_flops / conv_ms / 1e9 if conv_ms else 0.0, "ms": conv_ms, "gflop": conv_flops / 1e9,
                        "frac_fp32_mfma_peak": (conv_flops / conv_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS) if conv_ms else 0.0},

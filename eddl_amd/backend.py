@@ -111,6 +111,24 @@ class Event:
             pass
 
 
+class Graph:
+    """A recorded sequence of launches (``Backend.record``); ``launch()`` replays it on the device's stream."""
+
+    def __init__(self, backend, handle):
+        self.backend, self.handle = backend, handle
+
+    def launch(self):
+        self.backend._check(self.backend.lib.eddlhip_graph_launch(self.backend.dev, self.handle))
+
+    def __del__(self):
+        try:
+            if self.handle:
+                self.backend.lib.eddlhip_graph_destroy(self.backend.dev, self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
 def _ptr(t):
     return None if t is None else t.ptr
 
@@ -135,6 +153,21 @@ class Backend:
 
     def _free(self, ptr):
         self.lib.eddlhip_free(self.dev, ptr)
+
+    def record(self, fn):
+        """Records the launches ``fn()`` makes into a Graph instead of running them.  ``fn`` must have
+        run once before (workspace at its final size) and may only launch kernels."""
+        self._check(self.lib.eddlhip_graph_begin(self.dev))
+        h = ctypes.c_void_p()
+        try:
+            fn()
+        except BaseException:
+            self.lib.eddlhip_graph_end(self.dev, ctypes.byref(h))  # leaves recording mode; the first error is the one to report
+            if h.value:
+                self.lib.eddlhip_graph_destroy(self.dev, h)
+            raise
+        self._check(self.lib.eddlhip_graph_end(self.dev, ctypes.byref(h)))
+        return Graph(self, h)
 
     @property
     def name(self):

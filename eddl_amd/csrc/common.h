@@ -19,6 +19,10 @@ struct DeviceState {
     size_t workspace_bytes = 0;
     void *flag = nullptr;  // one int of device memory for kernels that report a condition
     hipStream_t copy_stream[2] = {nullptr, nullptr};  // uploads, downloads: created on first use (non-blocking, default priority)
+    // eddlhip_graph_begin .. _end: launches go to capture_stream and are recorded, not run
+    bool capturing = false;
+    hipStream_t capture_stream = nullptr;  // created on first use (non-blocking, default priority)
+    hipStream_t stream_before_capture = nullptr;
 };
 
 DeviceState &state(int dev);
@@ -56,6 +60,10 @@ void conv_filters_released(int dev, const void *base, size_t bytes);
     } while (0)
 
 #define EH_CHECK_LAUNCH() EH_TRY_HIP(hipGetLastError())
+
+// For entry points that wait for the device, allocate or free: not possible while a graph is being recorded.
+#define EH_NOT_CAPTURING(dev, what)                                                                                   \
+    EH_REQUIRE(!eddlhip::state(dev).capturing, "%s is not possible between eddlhip_graph_begin and eddlhip_graph_end", what)
 
 static inline unsigned eh_blocks(size_t work, unsigned per_block, unsigned cap = 1u << 20) {
     size_t b = (work + per_block - 1) / per_block;

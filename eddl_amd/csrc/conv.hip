@@ -1144,6 +1144,7 @@ int eddlhip_conv2d_cache_filters(int dev, const float *K, int Kf, int C, int R, 
     EH_REQUIRE(K != nullptr && Kf > 0 && C > 0 && R > 0 && S > 0, "conv2d_cache_filters: bad filter tensor %dx%dx%dx%d", Kf, C, R, S);
     EH_REQUIRE((long long)C * R * S <= (1LL << 24), "conv2d_cache_filters: filter too large");
     EH_TRY(use_device(dev));
+    EH_NOT_CAPTURING(dev, "eddlhip_conv2d_cache_filters");
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     for (CachedFilters &e : g_cache[dev]) {
         if (e.K == K) {
@@ -1170,6 +1171,7 @@ int eddlhip_conv2d_cache_filters(int dev, const float *K, int Kf, int C, int R, 
 
 int eddlhip_conv2d_uncache_filters(int dev, const float *K) {
     EH_TRY(use_device(dev));
+    EH_NOT_CAPTURING(dev, "eddlhip_conv2d_uncache_filters");
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     std::vector<CachedFilters> &c = g_cache[dev];
     bool synced = false;
@@ -1245,6 +1247,7 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     if (N == 0) return 0;
     EH_REQUIRE(I && K && O, "conv2d: NULL tensor");
     EH_TRY(use_device(dev));
+    EH_REQUIRE(!(g_prof_on && state(dev).capturing), "conv2d: launches cannot be timed (eddlhip_conv2d_profile) while a graph is being recorded");
     hipStream_t st = state(dev).stream;
 
     ConvParams p;

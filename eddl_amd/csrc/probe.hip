@@ -59,6 +59,7 @@ extern "C" int eddlhip_probe_mfma_f32(int dev, int vary_operands, int launches, 
         x = x * 1664525u + 1013904223u;
         host[i] = ((x >> 8) * (1.0f / 16777216.0f) - 0.5f) * 6.0f;
     }
+    EH_NOT_CAPTURING(dev, "eddlhip_probe_mfma_f32");
     void *ws = nullptr;
     EH_TRY(get_workspace(dev, sizeof(host) + (size_t)blocks * 256 * sizeof(float), &ws));
     float *in = (float *)ws, *out = in + 16 * 256;

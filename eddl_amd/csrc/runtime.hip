@@ -47,6 +47,9 @@ int use_device(int dev) {
 int get_workspace(int dev, size_t bytes, void **ptr) {
     DeviceState &s = g_state[dev];
     if (bytes > s.workspace_bytes) {
+        if (s.capturing)
+            return set_error(EDDLHIP_EINVAL, "the workspace would have to grow to %zu bytes while a graph is being recorded: "
+                             "run the same calls once before recording them", bytes);
         if (s.workspace) {
             EH_TRY_HIP(hipStreamSynchronize(s.stream));
             EH_TRY_HIP(hipFree(s.workspace));
@@ -87,6 +90,7 @@ int eddlhip_shutdown(int dev) {
     if (dev < 0 || dev >= EDDLHIP_MAX_DEVICES) return set_error(EDDLHIP_ENODEV, "device index %d out of range", dev);
     DeviceState &s = g_state[dev];
     if (!s.inited) return 0;
+    EH_NOT_CAPTURING(dev, "eddlhip_shutdown");
     EH_TRY_HIP(hipSetDevice(dev));
     EH_TRY_HIP(hipDeviceSynchronize());
     EH_TRY(eddlhip_conv2d_uncache_filters(dev, nullptr));
@@ -94,6 +98,7 @@ int eddlhip_shutdown(int dev) {
     if (s.flag) EH_TRY_HIP(hipFree(s.flag));
     for (hipStream_t cs : s.copy_stream)
         if (cs) EH_TRY_HIP(hipStreamDestroy(cs));
+    if (s.capture_stream) EH_TRY_HIP(hipStreamDestroy(s.capture_stream));
     s = DeviceState();
     return 0;
 }
@@ -109,12 +114,14 @@ int eddlhip_device_name(int dev, char *buf, size_t buflen) {
 
 int eddlhip_set_stream(int dev, void *hip_stream) {
     EH_TRY(use_device(dev));
+    EH_NOT_CAPTURING(dev, "eddlhip_set_stream");
     state(dev).stream = (hipStream_t)hip_stream;
     return 0;
 }
 
 int eddlhip_synchronize(int dev) {
     EH_TRY(use_device(dev));
+    EH_NOT_CAPTURING(dev, "eddlhip_synchronize");
     EH_TRY_HIP(hipStreamSynchronize(state(dev).stream));
     return 0;
 }
@@ -122,6 +129,7 @@ int eddlhip_synchronize(int dev) {
 int eddlhip_malloc(int dev, size_t bytes, void **dev_ptr) {
     EH_REQUIRE(dev_ptr != nullptr, "dev_ptr is NULL");
     EH_TRY(use_device(dev));
+    EH_NOT_CAPTURING(dev, "eddlhip_malloc");
     *dev_ptr = nullptr;
     if (bytes == 0) return 0;
     hipError_t e = hipMalloc(dev_ptr, bytes);
@@ -136,6 +144,7 @@ int eddlhip_malloc(int dev, size_t bytes, void **dev_ptr) {
 int eddlhip_free(int dev, void *dev_ptr) {
     if (!dev_ptr) return 0;
     EH_TRY(use_device(dev));
+    EH_NOT_CAPTURING(dev, "eddlhip_free");
     void *base = nullptr;
     size_t size = 0;
     if (hipMemGetAddressRange(&base, &size, dev_ptr) == hipSuccess) conv_filters_released(dev, base, size);
@@ -150,6 +159,7 @@ int eddlhip_memcpy_h2d(int dev, void *dev_dst, const void *host_src, size_t byte
     if (bytes == 0) return 0;
     EH_REQUIRE(dev_dst && host_src, "NULL pointer in h2d copy");
     EH_TRY(use_device(dev));
+    EH_NOT_CAPTURING(dev, "eddlhip_memcpy_h2d");
     conv_filters_written(dev, dev_dst, bytes);
     EH_TRY_HIP(hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice, state(dev).stream));
     EH_TRY_HIP(hipStreamSynchronize(state(dev).stream));
@@ -160,6 +170,7 @@ int eddlhip_memcpy_d2h(int dev, void *host_dst, const void *dev_src, size_t byte
     if (bytes == 0) return 0;
     EH_REQUIRE(host_dst && dev_src, "NULL pointer in d2h copy");
     EH_TRY(use_device(dev));
+    EH_NOT_CAPTURING(dev, "eddlhip_memcpy_d2h");
     EH_TRY_HIP(hipMemcpyAsync(host_dst, dev_src, bytes, hipMemcpyDeviceToHost, state(dev).stream));
     EH_TRY_HIP(hipStreamSynchronize(state(dev).stream));
     return 0;
@@ -251,6 +262,62 @@ int eddlhip_download_wait_event(int dev, void *event) {
     hipStream_t cs;
     EH_TRY(copy_stream_of(dev, 1, &cs));
     EH_TRY_HIP(hipStreamWaitEvent(cs, (hipEvent_t)event, 0));
+    return 0;
+}
+
+// ---- graphs: a fixed sequence of launches recorded once and replayed with one call, for plans whose
+// kernels are so short that queueing them one by one takes longer than running them
+int eddlhip_graph_begin(int dev) {
+    EH_TRY(use_device(dev));
+    DeviceState &s = state(dev);
+    EH_REQUIRE(!s.capturing, "graph_begin: a graph is already being recorded on device %d", dev);
+    if (!s.capture_stream) EH_TRY_HIP(hipStreamCreateWithFlags(&s.capture_stream, hipStreamNonBlocking));
+    EH_TRY_HIP(hipStreamBeginCapture(s.capture_stream, hipStreamCaptureModeThreadLocal));
+    s.stream_before_capture = s.stream;
+    s.stream = s.capture_stream;
+    s.capturing = true;
+    return 0;
+}
+
+int eddlhip_graph_end(int dev, void **graph) {
+    EH_REQUIRE(graph != nullptr, "graph_end: graph is NULL");
+    EH_TRY(use_device(dev));
+    DeviceState &s = state(dev);
+    EH_REQUIRE(s.capturing, "graph_end: no graph is being recorded on device %d", dev);
+    *graph = nullptr;
+    hipGraph_t g = nullptr;
+    const hipError_t e = hipStreamEndCapture(s.capture_stream, &g);
+    s.stream = s.stream_before_capture;
+    s.capturing = false;
+    if (e != hipSuccess || g == nullptr) {
+        (void)hipGetLastError();
+        if (g) (void)hipGraphDestroy(g);
+        return set_error(EDDLHIP_EHIP, "graph_end: the recording is not valid (%s); a call that waits, copies to or from the host, "
+                         "allocates or fails ends it", hipGetErrorString(e));
+    }
+    hipGraphExec_t exec = nullptr;
+    const hipError_t ei = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (ei != hipSuccess) {
+        (void)hipGetLastError();
+        return set_error(EDDLHIP_EHIP, "graph_end: hipGraphInstantiate: %s", hipGetErrorString(ei));
+    }
+    *graph = (void *)exec;
+    return 0;
+}
+
+int eddlhip_graph_launch(int dev, void *graph) {
+    EH_REQUIRE(graph != nullptr, "graph_launch: graph is NULL");
+    EH_TRY(use_device(dev));
+    EH_NOT_CAPTURING(dev, "eddlhip_graph_launch");
+    EH_TRY_HIP(hipGraphLaunch((hipGraphExec_t)graph, state(dev).stream));
+    return 0;
+}
+
+int eddlhip_graph_destroy(int dev, void *graph) {
+    if (!graph) return 0;
+    EH_TRY(use_device(dev));
+    EH_TRY_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
     return 0;
 }
 

@@ -352,6 +352,7 @@ class Net:
         self.out = {}   # id(layer) -> DeviceTensor holding its output (absent for layers folded into a fused op)
         self.aux = {}   # id(layer) -> extra tensors (pool indices, bn side outputs)
         self.ops = []
+        self.graph = None  # a captured plan names the tensors of the build it was recorded on
         absorbed = set()
         sole_child = lambda l: l.children[0] if len(l.children) == 1 and l not in self.lout else None
 
@@ -559,6 +560,21 @@ class Net:
         """Queue every op of the plan on the device's stream (inputs already resident)."""
         for op in self.ops:
             op.run()
+
+    def capture(self):
+        """Records the plan as a graph (one call replays every launch): for plans whose kernels are so short
+        that queueing them one at a time takes longer than running them.  Runs the plan once first, so that
+        the library's workspace has its final size.  The graph names this net's tensors: capture again after
+        ``resize``."""
+        self.run()
+        self.graph = self.backend.record(self.run)
+        return self.graph
+
+    def run_graph(self):
+        """Replays the captured plan on the device's stream (``capture`` first)."""
+        if self.graph is None:
+            msg("no captured plan: call capture() after build or resize", "Net::run_graph")
+        self.graph.launch()
 
     def predict(self, xs):
         """Inference forward; returns host arrays (the reference's predict collects outputs to the CPU)."""

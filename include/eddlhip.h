@@ -84,6 +84,22 @@ int eddlhip_upload_wait_event(int dev, void *event);
 int eddlhip_download_wait_event(int dev, void *event);
 int eddlhip_event_synchronize(int dev, void *event);
 
+/* Graphs.  A plan of short kernels (a small network, a small batch) can take longer to queue launch by
+ * launch than to run.  Between eddlhip_graph_begin and eddlhip_graph_end the library's launches on the
+ * device are recorded instead of run (stream capture on a stream of the library's own, default priority);
+ * eddlhip_graph_end returns the recorded sequence as a graph that eddlhip_graph_launch replays, in one
+ * call, on the device's stream - same kernels, same arguments, same order, hence the same results bit for
+ * bit.  Pointers and shapes are frozen into the graph: replay only while the tensors it names are alive,
+ * and record again after a resize.  Run the same calls once BEFORE recording, so that the workspace has
+ * its final size and registered filters are repacked; calls that wait for the device, copy from or to the
+ * host, allocate or free are refused while recording.  A call that fails while recording leaves the
+ * recording open: close it with eddlhip_graph_end (which then reports the failure too).
+ * No counterpart in the reference, which synchronises after every kernel. */
+int eddlhip_graph_begin(int dev);
+int eddlhip_graph_end(int dev, void **graph);
+int eddlhip_graph_launch(int dev, void *graph);
+int eddlhip_graph_destroy(int dev, void *graph);
+
 /* Events on the device's stream, for timing kernels where they run.  No counterpart in the
  * reference (its profiling is host wall-clock, include/eddl/profiling.h:27-66). */
 int eddlhip_event_create(int dev, void **event);

@@ -163,3 +163,46 @@ def test_predict_batches_overlapped_staging_matches_predict(hip, oracle):
         assert np.array_equal(a, b)
     assert [o[0].shape for o in m.predict_batches([batches[0]])] == [want[0].shape]
     assert list(m.predict_batches([])) == []
+
+
+def test_captured_plan_replays_bit_for_bit(hip, oracle):
+    """The plan recorded once as a graph gives, on every replay, what queueing the launches one by one gives:
+    several replays, each on a new input, with eager work of the same net and waits between them."""
+    from eddl_amd import EddlHipError, models
+    nets = [
+        (models.conv_bn_relu_pool_block(batch=3, channels=16, size=20, filters=24), (3, 16, 20, 20)),
+        (models.resnet50(batch=2, size=64, num_classes=10, base=16), (2, 3, 64, 64)),   # K-split launches, residual epilogues, dense
+        (models.unet(batch=1, size=64, widths=(8, 16, 32, 64), bottleneck=128), (1, 1, 64, 64)),  # concat, upsampling, folded pads
+        (models.vgg16(batch=2, size=32, num_classes=10, dense=128), (2, 3, 32, 32)),
+    ]
+    rng = np.random.default_rng(77)
+    for i, (m, shape) in enumerate(nets):
+        models.init_he_normal(m, 70 + i)
+        for fuse in (True, False):
+            m.build(hip, fuse=fuse)
+            with pytest.raises(RuntimeError):
+                m.run_graph()                # nothing captured yet
+            m.capture()
+            for _ in range(4):
+                x = rng.standard_normal(shape, dtype=np.float32)
+                want = m.predict([x])[0].copy()          # eager, with its waits and copies
+                m.input_tensor().copy_from(rng.standard_normal(shape, dtype=np.float32))
+                m.run()                                   # eager work on another input in between
+                hip.synchronize()
+                m.input_tensor().copy_from(x)
+                m.run_graph()
+                got = m.out[id(m.lout[0])].numpy()
+                assert np.array_equal(got, want), (i, fuse)
+    # a call that waits is refused while recording, and the recording can still be closed
+    m = nets[0][0]
+
+    def bad():
+        m.run()
+        hip.synchronize()
+    with pytest.raises(EddlHipError, match="graph_begin and eddlhip_graph_end"):
+        hip.record(bad)
+    m.run()            # the device and the library are usable afterwards
+    hip.synchronize()
+    g = hip.record(m.run)
+    g.launch()
+    hip.synchronize()
