@@ -233,6 +233,9 @@ def main():
                                     "pure_mfma_varying_operands_mean": vary_mean, "varying_best_launch": vary_best,
                                     "varying_worst_launch": vary_worst,
                                     "frac_of_varying_mean": achieved / vary_mean if vary_mean > 0 else None}
+        # and what plain read / write / copy streams over 1 GiB buffers sustain, beside the 8 TB/s HBM peak
+        rd, wr, cp = hip.probe_hbm(1 << 30)
+        roofline["device_probe"].update(hbm_unit="GB/s", hbm_read_stream=rd, hbm_write_stream=wr, hbm_copy_stream=cp)
 
     conv_ms = sum(r["ms"] for r in conv_rows)
     conv_flops = sum(r["flops"] for r in conv_rows)

@@ -46,6 +46,7 @@ PROTOTYPES = {
     "eddlhip_graph_launch": [c_int, c_void_p],
     "eddlhip_graph_destroy": [c_int, c_void_p],
     "eddlhip_probe_mfma_f32": [c_int, c_int, c_int, ctypes.POINTER(c_float), ctypes.POINTER(c_float), ctypes.POINTER(c_float)],
+    "eddlhip_probe_hbm": [c_int, c_size_t, ctypes.POINTER(c_float), ctypes.POINTER(c_float), ctypes.POINTER(c_float)],
     "eddlhip_conv2d_fwd": [c_int, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_cache_filters": [c_int, P, c_int, c_int, c_int, c_int],
     "eddlhip_conv2d_uncache_filters": [c_int, P],

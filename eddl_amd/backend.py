@@ -207,6 +207,13 @@ class Backend:
                                                     ctypes.byref(worst)))
         return mean.value, best.value, worst.value
 
+    def probe_hbm(self, nbytes=1 << 30):
+        """What plain streams over device memory sustain with nothing else running: (read, write, copy) GB/s over
+        two buffers of ``nbytes`` each; copy counts bytes read plus bytes written."""
+        r, w, c = ctypes.c_float(), ctypes.c_float(), ctypes.c_float()
+        self._check(self.lib.eddlhip_probe_hbm(self.dev, int(nbytes), ctypes.byref(r), ctypes.byref(w), ctypes.byref(c)))
+        return r.value, w.value, c.value
+
     def empty(self, shape):
         return DeviceTensor(self, shape)
 

@@ -114,6 +114,13 @@ int eddlhip_event_elapsed_ms(int dev, void *start, void *stop, float *ms);
  * No counterpart in the reference; the benchmark reports the result beside the published peak. */
 int eddlhip_probe_mfma_f32(int dev, int vary_operands, int launches, float *tflops_mean, float *tflops_best,
                            float *tflops_worst);
+/* Device probe: GB/s that plain streams over device memory sustain with nothing else running - read only,
+ * write only, and copy (bytes read + bytes written) - over two buffers of `bytes` each that the call
+ * allocates and frees (choose them larger than the device's caches: 1 GiB).  16-byte accesses, four in
+ * flight per thread or one, with and without the streaming (non-temporal) hint, several grid sizes; the best rate
+ * of each kind is returned.  It is what the bandwidth-bound kernels can be measured against beside the
+ * published 8 TB/s.  No counterpart in the reference. */
+int eddlhip_probe_hbm(int dev, size_t bytes, float *read_gbs, float *write_gbs, float *copy_gbs);
 
 /* ------------------------------------------------------------------ convolution
  * Replaces gpu_conv2D(ConvolDescriptor*) (src/hardware/gpu/nn/gpu_conv.cu:159-233; CPU

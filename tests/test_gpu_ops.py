@@ -544,3 +544,14 @@ def test_conv2d_input_beyond_2gib_runs_in_batch_chunks(hip, oracle):
     pts = got[idx[:, 0], idx[:, 1], idx[:, 2], idx[:, 3]]
     tol = 1e-5 * float(np.abs(got).max()) + 1e-4 * np.abs(ref)
     assert np.all(np.abs(ref - pts) <= tol), np.abs(ref - pts).max()
+
+
+def test_device_probes_report_plausible_rates(hip):
+    from eddl_amd import EddlHipError
+    rd, wr, cp = hip.probe_hbm(1 << 28)
+    for v in (rd, wr, cp):
+        assert 500.0 < v < 16000.0, (rd, wr, cp)   # GB/s: far above PCIe, below twice the published HBM peak
+    with pytest.raises(EddlHipError, match="buffer size"):
+        hip.probe_hbm(1000)
+    mean, best, worst = hip.probe_mfma_f32(vary_operands=True, launches=3)
+    assert 50.0 < worst <= mean <= best < 200.0
