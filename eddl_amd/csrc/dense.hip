@@ -41,7 +41,9 @@ __global__ __launch_bounds__(256) void dense_transpose_kernel(const float *__res
 
 // grid: (column tiles of 128, k slices, row tiles of 32); block: one wavefront.
 // VEC: n is a multiple of 4 and B is 16-byte aligned, so a lane's four columns are one float4.
-template <bool VEC>
+// STREAM (with VEC): the weights are read with the streaming (non-temporal) hint - for matrices larger than
+// the device's caches, which no later kernel finds there anyway (25088 x 4096: 96 -> 88 us).
+template <bool VEC, bool STREAM>
 __global__ __launch_bounds__(64) void dense_partial_kernel(const float *__restrict__ At, const float *__restrict__ B,
                                                            float *__restrict__ part, int m, int k, int n, int kslice) {
     const int lane = threadIdx.x, half = lane >> 5, l = lane & 31;
@@ -82,7 +84,8 @@ __global__ __launch_bounds__(64) void dense_partial_kernel(const float *__restri
             a[u] = ap[(size_t)ki * 32];
             const float *row = B + (size_t)ki * n;
             if (VEC) {
-                b[u] = col0 < n ? *reinterpret_cast<const floatx4 *>(row + col0) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+                const floatx4 *src = reinterpret_cast<const floatx4 *>(row + col0);
+                b[u] = col0 < n ? (STREAM ? __builtin_nontemporal_load(src) : *src) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
             } else {
                 b[u] = load_b(ki);
             }
@@ -177,8 +180,9 @@ int dense_impl(int dev, const float *A, const float *B, float *C, int m, int k, 
     hipLaunchKernelGGL(dense_transpose_kernel, dim3((k + 31) / 32, mt), dim3(256), 0, st, A, At, m, k);
     EH_CHECK_LAUNCH();
     const bool vec = (n % 4 == 0) && (((uintptr_t)B & 15u) == 0);
-    if (vec) hipLaunchKernelGGL(dense_partial_kernel<true>, dim3(nt, nslices, mt), dim3(64), 0, st, At, B, part, m, k, n, kslice);
-    else hipLaunchKernelGGL(dense_partial_kernel<false>, dim3(nt, nslices, mt), dim3(64), 0, st, At, B, part, m, k, n, kslice);
+    const bool stream = vec && (size_t)k * n * sizeof(float) > ((size_t)256 << 20);  // beyond the 256 MB last-level cache
+    auto kern = !vec ? dense_partial_kernel<false, false> : (stream ? dense_partial_kernel<true, true> : dense_partial_kernel<true, false>);
+    hipLaunchKernelGGL(kern, dim3(nt, nslices, mt), dim3(64), 0, st, At, B, part, m, k, n, kslice);
     EH_CHECK_LAUNCH();
     size_t mn = (size_t)m * n;
     hipLaunchKernelGGL(dense_reduce_kernel, dim3(eh_blocks(mn, 256, 65536)), dim3(256), 0, st, (const float *)part, C, mn, nslices, incC,
