@@ -11,6 +11,7 @@ using namespace eddlhip;
 namespace {
 
 constexpr int TPB = 256;
+constexpr int kBnFlatBelow = 4096;  // planes shorter than this take the flat batch-norm kernel
 
 __device__ __forceinline__ float relu_f(float x) { return x > 0.0f ? x : 0.0f; }
 
@@ -104,6 +105,58 @@ __global__ __launch_bounds__(TPB) void bn_inference_kernel(int plane0, int z, in
             o = aff(o);
         }
         out[base + j] = o;
+    }
+}
+
+// Small planes (a 7x7 plane would leave most of a workgroup idle above): one float4 of the whole tensor per
+// thread, whatever plane it falls into.  A float4 may cross from one plane into the next (planes of at
+// least 4 elements: at most one crossing), so the constants of both channels are at hand.  Same operations
+// per element as above.  IDX: 32-bit element arithmetic when the tensor allows it.
+template <typename IDX>
+__global__ __launch_bounds__(TPB) void bn_inference_flat_kernel(IDX total, int z, int rc, const float *__restrict__ in,
+                                                                float *__restrict__ out, float *__restrict__ opa,
+                                                                const float *__restrict__ gmean, const float *__restrict__ gvar,
+                                                                const float *__restrict__ g, const float *__restrict__ bb,
+                                                                float *__restrict__ variance, float eps) {
+    const bool affine = g != nullptr;
+    const IDX n4 = total / 4;
+    const IDX i0 = (IDX)blockIdx.x * TPB + threadIdx.x, stride = (IDX)gridDim.x * TPB;
+    for (IDX j = i0; j < n4; j += stride) {
+        const IDX e0 = j * 4;
+        const IDX plane = e0 / (IDX)rc;
+        const int r0 = (int)(e0 - plane * (IDX)rc);
+        const int c0 = (int)(plane % (IDX)z);
+        const bool crosses = r0 + 3 >= rc;  // components from rc - r0 on belong to the next plane
+        const int c1 = crosses ? (c0 + 1 == z ? 0 : c0 + 1) : c0;
+        const float sd0 = sqrtf(__fadd_rn(gvar[c0], eps)), sd1 = sqrtf(__fadd_rn(gvar[c1], eps));
+        const float m0 = gmean[c0], m1 = gmean[c1];
+        const float g0 = affine ? g[c0] : 1.0f, g1 = affine ? g[c1] : 1.0f;
+        const float b0 = affine ? bb[c0] : 0.0f, b1 = affine ? bb[c1] : 0.0f;
+        if (r0 == 0 && plane < (IDX)z) variance[c0] = sd0;
+        if (crosses && plane + 1 < (IDX)z) variance[c1] = sd1;
+        const float4 x = reinterpret_cast<const float4 *>(in)[j];
+        const float xs[4] = {x.x, x.y, x.z, x.w};
+        float o[4], y[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const bool first = r0 + k < rc;
+            o[k] = __fdiv_rn(__fsub_rn(xs[k], first ? m0 : m1), first ? sd0 : sd1);
+            y[k] = affine ? __fadd_rn(__fmul_rn(o[k], first ? g0 : g1), first ? b0 : b1) : o[k];
+        }
+        if (affine && opa) reinterpret_cast<float4 *>(opa)[j] = make_float4(o[0], o[1], o[2], o[3]);
+        reinterpret_cast<float4 *>(out)[j] = make_float4(y[0], y[1], y[2], y[3]);
+    }
+    for (IDX e = n4 * 4 + i0; e < total; e += stride) {  // the last total % 4 elements
+        const IDX plane = e / (IDX)rc;
+        const int c = (int)(plane % (IDX)z);
+        const float sd = sqrtf(__fadd_rn(gvar[c], eps));
+        if (e == plane * (IDX)rc && plane < (IDX)z) variance[c] = sd;
+        float o = __fdiv_rn(__fsub_rn(in[e], gmean[c]), sd);
+        if (affine) {
+            if (opa) opa[e] = o;
+            o = __fadd_rn(__fmul_rn(o, g[c]), bb[c]);
+        }
+        out[e] = o;
     }
 }
 
@@ -343,8 +396,21 @@ int eddlhip_batchnorm_inference(int dev, int b, int z, int rc, const float *inpu
     EH_REQUIRE(input && output, "batchnorm: NULL tensor");
     EH_REQUIRE((long long)b * z <= 0x7fffffffLL, "batchnorm: too many planes");
     EH_TRY(use_device(dev));
-    int vec = (rc % 4 == 0) && aligned16(input) && aligned16(output) && (!opa || aligned16(opa));
+    const bool all_aligned = aligned16(input) && aligned16(output) && (!opa || aligned16(opa));
     long long planes = (long long)b * z;
+    if (rc >= 4 && rc < kBnFlatBelow && all_aligned) {
+        const size_t total = (size_t)planes * rc;
+        const unsigned grid = eh_blocks(total / 4 + 1, TPB, 1u << 20);
+        if (total < 0x7fffffffULL)
+            hipLaunchKernelGGL(bn_inference_flat_kernel<unsigned>, dim3(grid), dim3(TPB), 0, state(dev).stream, (unsigned)total, z, rc,
+                               input, output, opa, global_mean, global_variance, affine_g, affine_b, variance, epsilon);
+        else
+            hipLaunchKernelGGL(bn_inference_flat_kernel<size_t>, dim3(grid), dim3(TPB), 0, state(dev).stream, total, z, rc, input,
+                               output, opa, global_mean, global_variance, affine_g, affine_b, variance, epsilon);
+        EH_CHECK_LAUNCH();
+        return 0;
+    }
+    int vec = (rc % 4 == 0) && all_aligned;
     // grid.y is limited to 65535: fold the rest into a loop of launches
     int gx = (int)eh_blocks((size_t)rc / 4 + 1, TPB, 64);
     for (long long p0 = 0; p0 < planes; p0 += 65535) {
