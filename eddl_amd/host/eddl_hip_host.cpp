@@ -107,6 +107,8 @@ void Tensor::allocate() {
     } else if (isGPU()) {
         gpu_device = device - DEV_GPU;
         gpu_init(gpu_device);  // once per device, on the first tensor (src/tensor/tensor.cpp:190-202)
+        // gpu_create_tensor keeps the reference's signature, whose element count is an int
+        if (size > 0x7fffffffUL) msg("A tensor of more than 2^31 - 1 elements does not fit gpu_create_tensor's int size", "Tensor::updateData");
         ptr = gpu_create_tensor(gpu_device, (int)size);
     } else {
         msg("Unsupported device", "Tensor::updateData");
