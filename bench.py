@@ -6,7 +6,7 @@ resident in HBM (default workload: VGG-16, batch 32, fp32, 3x224x224 - the confi
 headline metric is quoted on).  Prints ONE JSON line on stdout; the per-layer table goes to
 stderr with --layers and to DIR/bench_layers_<workload>.{json,txt} with --out DIR.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vgg16|block|resnet50|unet]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vgg16|block|resnet50|unet|conv]
                     [--no-cpu-baseline] [--layers] [--out DIR] [--unfused] [--graph]
 
 --unfused runs the graph layer by layer (every BatchNorm, ReLU, Add and Pad as a launch of its own, as
@@ -30,16 +30,23 @@ PEAK_HBM_GBS = 8000.0
 WORKLOADS = {
     # name -> (builder kwargs, seed, input distribution, description)
     "vgg16": (dict(batch=32), 3, "uniform", "VGG-16 forward, batch 32, 3x224x224, fp32 (13 conv3x3+ReLU, 5 maxpool, 3 dense, softmax)"),
+    "conv": (dict(batch=8), 1, "normal", "single Conv2D 3->32, 3x3 same, bias, batch 8, 3x32x32, fp32 (14 MFLOP: bound by launch latency)"),
     "block": (dict(batch=64), 2, "normal", "Conv3x3(64->64)-BN-ReLU-MaxPool2x2 block, batch 64, 64x56x56, fp32"),
     "resnet50": (dict(batch=64), 4, "normal", "ResNet-50 forward, batch 64, 3x224x224, fp32, inference BN"),
     "unet": (dict(batch=4), 5, "uniform", "U-Net forward, batch 4, 1x512x512, fp32"),
 }
 
 
+def builder_of(name):
+    from eddl_amd import models
+    return {"vgg16": models.vgg16, "block": models.conv_bn_relu_pool_block, "resnet50": models.resnet50, "unet": models.unet,
+            "conv": models.single_conv}[name]
+
+
 def build_workload(name):
     from eddl_amd import models
     kwargs, seed, dist, desc = WORKLOADS[name]
-    builder = {"vgg16": models.vgg16, "block": models.conv_bn_relu_pool_block, "resnet50": models.resnet50, "unet": models.unet}[name]
+    builder = builder_of(name)
     model = builder(**kwargs)
     models.init_he_normal(model, seed)
     rng = np.random.default_rng(seed + 1000)
@@ -95,7 +102,7 @@ def cpu_baseline(workload, want_seconds=20.0):
     if env_threads:
         cores = min(cores, int(env_threads))
     kwargs, seed, dist, _ = WORKLOADS[workload]
-    builder = {"vgg16": models.vgg16, "block": models.conv_bn_relu_pool_block, "resnet50": models.resnet50, "unet": models.unet}[workload]
+    builder = builder_of(workload)
     full_batch = kwargs["batch"]
     sample_batch = min(full_batch, max(1, cores))  # one image per thread: the reference parallelises over the batch
     result = {"unit": "images/sec", "cores": cores, "kind": "port"}

@@ -51,6 +51,12 @@ def conv_bn_relu_pool_block(batch=64, channels=64, size=56, filters=64):
     return L.Net([x], [l])
 
 
+def single_conv(batch=8, channels=3, size=32, filters=32):
+    """One Conv2D 3x3, stride 1, "same", with bias: the smallest configuration (the one the reference's CPU path runs today)."""
+    x = L.Input([channels, size, size], batch)
+    return L.Net([x], [L.Conv2D(x, filters, [3, 3], [1, 1], "same", use_bias=True)])
+
+
 def vgg16(batch=32, size=224, num_classes=1000, widths=(64, 128, 256, 512, 512), dense=4096):
     """VGG-16, all 3x3 convolutions with bias and ReLU, five 2x2 max-pools, three dense layers, softmax."""
     x = L.Input([3, size, size], batch)

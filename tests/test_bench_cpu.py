@@ -1,5 +1,5 @@
 """bench.py pieces that need no GPU: the refusal of more than one GPU, the workload table (FLOP
-counts of the four configurations against the figures the survey of the reference gives), and
+counts of the five configurations against the figures the survey of the reference gives), and
 the CPU-baseline leg on a tiny sample."""
 import json
 import os
@@ -20,11 +20,9 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 def test_workload_flops_match_the_configurations():
     sys.path.insert(0, ROOT)
     import bench
-    from eddl_amd import models
-    want = {"vgg16": 982.18e9, "resnet50": 523.15e9, "unet": 1745.1e9, "block": 14.797e9}
-    builders = {"vgg16": models.vgg16, "block": models.conv_bn_relu_pool_block, "resnet50": models.resnet50, "unet": models.unet}
+    want = {"vgg16": 982.18e9, "resnet50": 523.15e9, "unet": 1745.1e9, "block": 14.797e9, "conv": 14155776.0}
     for name, (kwargs, seed, dist, desc) in bench.WORKLOADS.items():
-        m = builders[name](**kwargs)
+        m = bench.builder_of(name)(**kwargs)
         flops = 0
         for l in m.layers:
             if l.kind == "conv2d":
