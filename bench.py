@@ -86,10 +86,15 @@ def time_ops(hip, model, reps):
     return op_ms, kernels, kern_ms, kern_launches
 
 
-def cpu_baseline(workload, want_seconds=20.0):
+PARITY_BOUND = 1e-4  # largest |device - oracle| over the sample's outputs, relative to the largest |oracle| output
+
+
+def cpu_baseline(workload, want_seconds=20.0, device_output=None):
     """The CPU oracle (a port of the reference's CPU algorithm: per-image im2col + one
     single-threaded GEMM, OpenMP over the batch, separate bias/ReLU/pool passes) timed on this
-    host on a bounded sample of the same workload."""
+    host on a bounded sample of the same workload.  The sample is the first images of the
+    benchmark's own batch (same seeds), so with ``device_output`` (the device's output for the
+    whole batch) the oracle's outputs also check the timed device run end to end: ``parity``."""
     from eddl_amd import models
     from oracle import net_oracle
     from oracle.oracle import Oracle
@@ -123,8 +128,15 @@ def cpu_baseline(workload, want_seconds=20.0):
         times = []
         while not times or (sum(times) < budget and len(times) < 200):
             t0 = time.perf_counter()
-            net_oracle.forward(ora, model, [x], conv_algo="im2col")
+            ref = net_oracle.forward(ora, model, [x], conv_algo="im2col")[0]
             times.append(time.perf_counter() - t0)
+        if not hpc and device_output is not None:  # the strict build is the parity oracle
+            got = np.asarray(device_output)[:sample_batch].reshape(ref.shape)
+            scale = float(np.abs(ref).max())
+            err = float(np.abs(got - ref).max())
+            result["parity"] = {"images": sample_batch, "max_abs_err": err, "max_abs_ref": scale,
+                                "err_over_max_ref": err / scale if scale > 0 else err, "bound": PARITY_BOUND,
+                                "ok": bool(err <= PARITY_BOUND * scale)}
         # the first forward pays for page faults of the lowered-matrix buffers: drop it when there are others
         timed = times[1:] if len(times) > 1 else times
         dt = sum(timed) / len(timed)
@@ -258,7 +270,12 @@ def main():
         "device_ms_sum_of_ops": sum(op_ms),
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(args.workload)
+        result["cpu_baseline"] = cpu_baseline(args.workload, device_output=out_host)
+        parity = result["cpu_baseline"].get("parity")
+        if parity is not None and not parity["ok"]:
+            print(json.dumps(result))
+            sys.exit("bench.py: the device's output differs from the CPU oracle's by %.3g of the largest output (bound %.0e)"
+                     % (parity["err_over_max_ref"], PARITY_BOUND))
 
     table = ["%-44s %9s %9s %8s %9s %7s" % ("op", "ms", "TFLOP/s", "%mfma", "GB/s", "%hbm")]
     for r in rows:

@@ -40,3 +40,25 @@ def test_cpu_baseline_leg_runs_on_a_small_sample(monkeypatch):
     assert out["kind"] == "port" and out["unit"] == "images/sec" and out["cores"] >= 1
     assert out["value"] > 0 and out["value_strict"] > 0 and "sample" in out
     json.dumps(out)
+
+
+def test_cpu_baseline_leg_checks_a_device_output_against_the_oracle(monkeypatch):
+    """The parity gate of the benchmark: an output equal to the oracle's passes, one that is off by 1e-3 of the
+    output scale does not; a larger batch than the sample is compared on its first images."""
+    sys.path.insert(0, ROOT)
+    import bench
+    from eddl_amd import models
+    from oracle import net_oracle
+    from oracle.oracle import Oracle
+    kwargs = {"batch": 2, "channels": 4, "size": 8, "filters": 4}
+    monkeypatch.setitem(bench.WORKLOADS, "block", (kwargs, 2, "normal", "tiny block"))
+    monkeypatch.setattr(os, "cpu_count", lambda: 1)   # a sample of one image out of the batch of two
+    monkeypatch.setattr(os, "sched_getaffinity", lambda pid: {0}, raising=False)
+    model = models.conv_bn_relu_pool_block(**kwargs)
+    models.init_he_normal(model, 2)
+    x = np.random.default_rng(1002).standard_normal(model.lin[0].out_shape, dtype=np.float32)
+    full = net_oracle.forward(Oracle(hpc=False), model, [x])[0]
+    good = bench.cpu_baseline("block", want_seconds=0.1, device_output=full)["parity"]
+    assert good["ok"] and good["images"] == 1 and good["max_abs_err"] == 0.0
+    bad = bench.cpu_baseline("block", want_seconds=0.1, device_output=full + 1e-3 * np.abs(full).max())["parity"]
+    assert not bad["ok"] and bad["err_over_max_ref"] > bench.PARITY_BOUND
