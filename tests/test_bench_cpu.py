@@ -1,5 +1,5 @@
 """bench.py pieces that need no GPU: the refusal of more than one GPU, the workload table (FLOP
-counts of the five configurations against the figures the survey of the reference gives), and
+counts of the five configurations against figures worked out by hand from their layer shapes), and
 the CPU-baseline leg on a tiny sample."""
 import json
 import os

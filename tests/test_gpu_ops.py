@@ -105,7 +105,7 @@ def test_pad_and_softmax_reference_vectors(hip, golden):
 # ------------------------------------------------------------------ convolution
 CONV_SHAPES = [
     # N, C, H, W, Kf, R, S, sr, sc, padding, pads, bias
-    (8, 3, 32, 32, 32, 3, 3, 1, 1, "same", None, True),        # BASELINE config 1 shape
+    (8, 3, 32, 32, 32, 3, 3, 1, 1, "same", None, True),        # the single-convolution configuration
     (2, 64, 28, 28, 64, 3, 3, 1, 1, "same", None, False),
     (2, 16, 19, 23, 130, 3, 3, 1, 1, "same", None, True),      # ragged: channels and pixels not tile multiples
     (3, 5, 17, 13, 7, 3, 3, 2, 2, "same", None, True),         # asymmetric same pads
