@@ -209,6 +209,16 @@ def main():
     # ---- per-op device times (events on the kernels' stream), same resident input
     reps = max(3, min(args.steps, 10))
     op_ms, op_kernels, kern_ms, kern_launches = time_ops(hip, model, reps)
+    # what an event pair reads around a kernel that does next to nothing (one float filled): the part of every
+    # per-op figure below that is not the op
+    tiny = hip.empty((1,))
+    pairs = [(hip.event(), hip.event()) for _ in range(50)]
+    for s, e in pairs:
+        s.record()
+        hip.fill_(tiny, 0.0)
+        e.record()
+    hip.synchronize()
+    event_floor_ms = float(np.median([s.elapsed_ms(e) for s, e in pairs]))
     rows = []
     for op, ms, kern, kms, kl in zip(model.ops, op_ms, op_kernels, kern_ms, kern_launches):
         row = {"op": op.kind, "name": op.name, "ms": ms, "flops": op.flops, "bytes": op.bytes}
@@ -268,6 +278,7 @@ def main():
         "conv_total": {"tflops": conv_flops / conv_ms / 1e9 if conv_ms else 0.0, "ms": conv_ms, "gflop": conv_flops / 1e9,
                        "frac_fp32_mfma_peak": (conv_flops / conv_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS) if conv_ms else 0.0},
         "device_ms_sum_of_ops": sum(op_ms),
+        "event_pair_floor_ms": event_floor_ms,
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.workload, device_output=out_host)
@@ -277,7 +288,9 @@ def main():
             sys.exit("bench.py: the device's output differs from the CPU oracle's by %.3g of the largest output (bound %.0e)"
                      % (parity["err_over_max_ref"], PARITY_BOUND))
 
-    table = ["%-44s %9s %9s %8s %9s %7s" % ("op", "ms", "TFLOP/s", "%mfma", "GB/s", "%hbm")]
+    table = ["# ms = device time between two events around the op; an event pair around a one-element fill reads %.4f ms"
+             % event_floor_ms,
+             "%-44s %9s %9s %8s %9s %7s" % ("op", "ms", "TFLOP/s", "%mfma", "GB/s", "%hbm")]
     for r in rows:
         table.append("%-44s %9.4f %9s %8s %9.1f %7.2f  %s" % (
             r["name"][:44], r["ms"], "%.2f" % r["tflops"] if "tflops" in r else "-",
