@@ -250,10 +250,15 @@ class Backend:
     def fill_(self, A, v):
         self._check(self.lib.eddlhip_fill(self.dev, A.ptr, A.size, v))
 
-    def conv2D(self, I, K, bias, O, sr, sc, padrt, padcl, bn=None, residual=None, relu=False):
-        """``bn`` = (g, b, mean, var, eps) device tensors (g, b may be None) or None."""
+    def conv2D(self, I, K, bias, O, sr, sc, padrt, padcl, bn=None, residual=None, relu=False, second=None):
+        """``bn`` = (g, b, mean, var, eps) device tensors (g, b may be None) or None.  ``second``: the other half
+        of the input channels as a tensor of its own (a channel Concat of ``I`` and ``second`` folded into the call)."""
         N, C, H, W = I.shape
         Kf, C2, R, S = K.shape
+        if second is not None:
+            if tuple(second.shape) != tuple(I.shape):
+                raise ValueError("the two input tensors differ in shape: %s, %s" % (I.shape, second.shape))
+            C = 2 * C
         if C2 != C:
             raise ValueError("filter depth %d != input channels %d" % (C2, C))
         if O.shape[0] != N or O.shape[1] != Kf:
@@ -262,9 +267,12 @@ class Backend:
         eps = 0.0
         if bn is not None:
             g, b, mean, var, eps = bn
-        self._check(self.lib.eddlhip_conv2d_fwd(self.dev, I.ptr, K.ptr, _ptr(bias), O.ptr, N, C, H, W, Kf, R, S, sr, sc, padrt,
-                                                padcl, O.shape[2], O.shape[3], _ptr(g), _ptr(b), _ptr(mean), _ptr(var), eps,
-                                                _ptr(residual), int(relu)))
+        tail = (K.ptr, _ptr(bias), O.ptr, N, C, H, W, Kf, R, S, sr, sc, padrt, padcl, O.shape[2], O.shape[3], _ptr(g), _ptr(b),
+                _ptr(mean), _ptr(var), eps, _ptr(residual), int(relu))
+        if second is None:
+            self._check(self.lib.eddlhip_conv2d_fwd(self.dev, I.ptr, *tail))
+        else:
+            self._check(self.lib.eddlhip_conv2d_fwd_concat(self.dev, I.ptr, second.ptr, *tail))
 
     def cache_conv_filters(self, K):
         """Keep the kernels' repacked copy of filter tensor ``K`` (fixed between calls) in the library."""

@@ -65,6 +65,11 @@ typedef int int32x4 __attribute__((ext_vector_type(4)));
 
 struct ConvParams {
     const float *I;
+    // Two-tensor input (a channel Concat folded into the convolution): channels [0, Csplit) come from I,
+    // channels [Csplit, C) from I2, both tensors holding Cimg = Csplit = C - Csplit channels per image.
+    // One tensor: I2 == I, Csplit == C, Cimg == C.
+    const float *I2;
+    int Csplit, Cimg;
     const float *Wp;  // packed filters [rows][Mp]
     const float *K;   // original OIHW filters (scalar kernel only)
     float *O;
@@ -435,6 +440,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     if (!split) chan = fetch_channel_constants<BM>(p, m0, tid);
 
     const __amdgpu_buffer_rsrc_t rsrc_in = __builtin_amdgcn_make_buffer_rsrc((void *)p.I, 0, p.in_bytes, RSRC_WORD3);
+    const __amdgpu_buffer_rsrc_t rsrc_in2 = __builtin_amdgcn_make_buffer_rsrc((void *)p.I2, 0, p.in_bytes, RSRC_WORD3);
 
     // ---- this thread's gathered pixel and its R*S tap offsets (bytes; OOB where the tap leaves the image)
     const int seg = wave % NS, cg = wave / NS;
@@ -447,7 +453,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         const int pq = (int)(ngc - (unsigned)img * (unsigned)p.PQ);
         const int op = (int)((unsigned)pq / (unsigned)p.Q), oq = pq - op * p.Q;
         const int ih0 = op * p.sr - p.pt, iw0 = oq * p.sc - p.pl;
-        const int pix = img * (p.C * p.H * p.W) + ih0 * p.W + iw0;
+        const int pix = img * (p.Cimg * p.H * p.W) + ih0 * p.W + iw0;
 #pragma unroll
         for (int t = 0; t < RS; t++) {
             const int ky = t / S, kx = t % S;
@@ -487,6 +493,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     constexpr int A_UPW = (A_UNITS + 3) / 4;
     static_assert((RPI - 1) * BM <= 256, "the parking area holds the surplus rows of the last unit");
     const int32x4 dma_w = make_rsrc_words(p.Wp, p.wp_bytes), dma_in = make_rsrc_words(p.I, p.in_bytes);
+    const int32x4 dma_in2 = make_rsrc_words(p.I2, p.in_bytes);
     const int a_voff_direct = ((lane / (BM / 4)) * p.Mp + m0 + 4 * (lane % (BM / 4))) * 4;
 
     auto load_a = [&](int step, lds_float *as) {
@@ -522,14 +529,15 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
             const int cl = cg * CPW + jc;
             const int c = step * CPB + cl;
             const bool cok = !checked || c < p.C;
-            const int soff = (cok ? c : 0) * HW4;
+            const bool second = c >= p.Csplit;  // uniform in the wavefront: the channel comes from the second tensor
+            const int soff = (cok ? (second ? c - p.Csplit : c) : 0) * HW4;
 #pragma unroll
             for (int t = 0; t < RS; t++) {
                 const int vo = cok ? voff[t] : OOB;
                 if constexpr (DIRECT) {
-                    lds_dma_b32(dma_in, bs + (cl * RS + t) * LDB + seg * 64, vo, soff);
+                    lds_dma_b32(second ? dma_in2 : dma_in, bs + (cl * RS + t) * LDB + seg * 64, vo, soff);
                 } else {
-                    breg[jc * RS + t] = buf_load(rsrc_in, vo, soff);
+                    breg[jc * RS + t] = second ? buf_load(rsrc_in2, vo, soff) : buf_load(rsrc_in, vo, soff);
                 }
             }
         }
@@ -903,7 +911,7 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvParams p) {
         r /= p.P;
         const int k = (int)(r % p.Kf);
         const int b = (int)(r / p.Kf);
-        const float *img = p.I + (size_t)b * p.C * p.H * p.W;
+        const float *img = p.I + (size_t)b * p.Cimg * p.H * p.W, *img2 = p.I2 + (size_t)b * p.Cimg * p.H * p.W;
         const float *flt = p.K + (size_t)k * p.C * p.R * p.S;
         float s = 0.0f;
         for (int x = 0; x < p.R; x++) {
@@ -912,8 +920,10 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvParams p) {
             for (int y = 0; y < p.S; y++) {
                 const int py = q * p.sc + y - p.pl;
                 if (py < 0 || py >= p.W) continue;
-                for (int c = 0; c < p.C; c++)
-                    s = __fadd_rn(s, __fmul_rn(flt[((size_t)c * p.R + x) * p.S + y], img[((size_t)c * p.H + px) * p.W + py]));
+                for (int c = 0; c < p.C; c++) {
+                    const float v = c < p.Csplit ? img[((size_t)c * p.H + px) * p.W + py] : img2[((size_t)(c - p.Csplit) * p.H + px) * p.W + py];
+                    s = __fadd_rn(s, __fmul_rn(flt[((size_t)c * p.R + x) * p.S + y], v));
+                }
             }
         }
         const ChannelEpilogue e = load_channel(p, k);
@@ -1229,9 +1239,15 @@ int eddlhip_conv2d_profile_read(int *launches, float *total_ms) {
 
 const char *eddlhip_conv2d_last_kernel(void) { return g_last_kernel; }
 
-int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bias, float *O, int N, int C, int H, int W, int Kf,
-                       int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b,
-                       const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu) {
+}  // extern "C"
+
+namespace {
+
+// I2 == nullptr: the input is the one tensor I[N,C,H,W].  Otherwise channels [0, C/2) are I[N,C/2,H,W] and
+// channels [C/2, C) are I2[N,C/2,H,W].
+int conv2d_fwd_impl(int dev, const float *I, const float *I2, const float *K, const float *bias, float *O, int N, int C, int H, int W,
+                    int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g,
+                    const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu) {
     EH_REQUIRE(N >= 0 && C > 0 && H > 0 && W > 0, "conv2d: bad input shape %dx%dx%dx%d", N, C, H, W);
     EH_REQUIRE(Kf > 0 && R > 0 && S > 0, "conv2d: bad filter shape %dx%dx%dx%d", Kf, C, R, S);
     EH_REQUIRE(sr > 0 && sc > 0, "conv2d: strides must be positive");
@@ -1240,7 +1256,14 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     EH_REQUIRE((bn_mean == nullptr) == (bn_var == nullptr), "conv2d: bn_mean and bn_var must come together");
     EH_REQUIRE((bn_g == nullptr) == (bn_b == nullptr), "conv2d: bn_g and bn_b must come together");
     EH_REQUIRE(bn_g == nullptr || bn_mean != nullptr, "conv2d: affine parameters without statistics");
-    const long long img_elems = (long long)C * H * W;
+    const bool two = I2 != nullptr;
+    const int Cimg = two ? C / 2 : C;  // channels per image in each input tensor
+    if (two) {
+        EH_REQUIRE(C % 2 == 0, "conv2d: a two-tensor input needs an even channel count, got %d", C);
+        EH_REQUIRE(g_algo == 2 || (R == S && (R == 1 || R == 2 || R == 3)),
+                   "conv2d: a two-tensor input is taken by the 1x1, 2x2 and 3x3 kernels only (filter %dx%d): concatenate first", R, S);
+    }
+    const long long img_elems = (long long)Cimg * H * W;
     EH_REQUIRE(img_elems <= (1LL << 28), "conv2d: one image of %lld elements exceeds the 1 GiB a buffer descriptor may cover", img_elems);
     EH_REQUIRE((long long)C * R * S <= (1LL << 24), "conv2d: filter too large");
     EH_REQUIRE((long long)P * Q <= 0x7fffffffLL, "conv2d: output plane too large");
@@ -1251,7 +1274,8 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     hipStream_t st = state(dev).stream;
 
     ConvParams p;
-    p.I = I; p.K = K; p.O = O; p.Wp = nullptr;
+    p.I = I; p.I2 = two ? I2 : I; p.Csplit = two ? C / 2 : C; p.Cimg = Cimg;
+    p.K = K; p.O = O; p.Wp = nullptr;
     p.bias = bias; p.bn_g = bn_g; p.bn_b = bn_b; p.bn_mean = bn_mean; p.bn_var = bn_var; p.residual = residual;
     p.bn_eps = bn_eps; p.relu = relu;
     p.N = N; p.C = C; p.H = H; p.W = W; p.Kf = Kf; p.R = R; p.S = S; p.sr = sr; p.sc = sc; p.pt = pad_top; p.pl = pad_left;
@@ -1343,6 +1367,7 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
         ConvParams q = p;
         q.N = nb;
         q.I = I + (size_t)b0 * img_elems;
+        q.I2 = p.I2 + (size_t)b0 * img_elems;
         q.O = O + (size_t)b0 * Kf * p.PQ;
         if (residual) q.residual = residual + (size_t)b0 * Kf * p.PQ;
         q.npix = (long long)nb * p.PQ;
@@ -1368,6 +1393,27 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
     if (leftover > 0) snprintf(g_last_kernel, sizeof(g_last_kernel), "%s +ksplit(%lld tiles x %d)", v->name, leftover, nslices);
     else snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", v->name);
     return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bias, float *O, int N, int C, int H, int W, int Kf,
+                       int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b,
+                       const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu) {
+    return conv2d_fwd_impl(dev, I, nullptr, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean,
+                           bn_var, bn_eps, residual, relu);
+}
+
+int eddlhip_conv2d_fwd_concat(int dev, const float *I_first, const float *I_second, const float *K, const float *bias, float *O,
+                              int N, int C, int H, int W, int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P,
+                              int Q, const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps,
+                              const float *residual, int relu) {
+    EH_REQUIRE(N == 0 || (I_first && I_second), "conv2d_fwd_concat: NULL input tensor");
+    if (N == 0) return 0;
+    return conv2d_fwd_impl(dev, I_first, I_second, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
+                           bn_mean, bn_var, bn_eps, residual, relu);
 }
 
 }  // extern "C"

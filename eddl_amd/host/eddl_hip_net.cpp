@@ -567,6 +567,17 @@ void Net::fuse() {
                 continue;
             }
         }
+        if (LConcat *cat = dynamic_cast<LConcat *>(l)) {
+            // a channel Concat of two equal-shaped 4-D tensors read only by a 1x1, 2x2 or 3x3 convolution: that
+            // convolution takes the two halves of its channels from the two tensors (eddlhip_conv2d_fwd_concat)
+            LConv *cv = dynamic_cast<LConv *>(sole_child(l));
+            if (cv != nullptr && cat->axis == 0 && cat->parent.size() == 2 && cat->parent[0] != cat->parent[1] &&
+                cat->output->ndim == 4 && cat->parent[0]->output->shape == cat->parent[1]->output->shape &&
+                cv->cd->kernel_size[0] == cv->cd->kernel_size[1] && cv->cd->kernel_size[0] >= 1 && cv->cd->kernel_size[0] <= 3) {
+                fused_away.push_back(l);
+                continue;
+            }
+        }
         if (LConv *conv = dynamic_cast<LConv *>(l)) {
             s.chain = true;
             s.src = l->parent[0];
@@ -577,6 +588,12 @@ void Net::fuse() {
                     s.pad_top += pad->padding[0];   // (top, right, bottom, left)
                     s.pad_left += pad->padding[3];
                     s.src = pad->parent[0];
+                }
+            }
+            if (LConcat *cat = dynamic_cast<LConcat *>(s.src)) {
+                if (is_fused_away(cat)) {
+                    s.src = cat->parent[0];
+                    s.src2 = cat->parent[1];
                 }
             }
             Layer *c = sole_child(s.last);
@@ -647,12 +664,21 @@ void Net::run_step(const FusedStep &s) {
         const Tensor *I = s.src->output;
         Tensor *O = s.last->output;
         const LBatchNorm *bn = s.bn;
-        gpu_check(eddlhip_conv2d_fwd(device, I->ptr, D->K->ptr, D->use_bias ? D->bias->ptr : nullptr, O->ptr, I->shape[0], I->shape[1],
-                                     I->shape[2], I->shape[3], D->nk, D->kr, D->kc, D->sr, D->sc, s.pad_top, s.pad_left, D->r, D->c,
-                                     bn && bn->affine ? bn->bn_g->ptr : nullptr, bn && bn->affine ? bn->bn_b->ptr : nullptr,
-                                     bn ? bn->mean->ptr : nullptr, bn ? bn->variance->ptr : nullptr, bn ? bn->epsilon : 0.0f,
-                                     s.res ? s.res->output->ptr : nullptr, s.relu ? 1 : 0),
-                  "Net::forward (fused convolution)");
+        const float *bias = D->use_bias ? D->bias->ptr : nullptr;
+        const float *g = bn && bn->affine ? bn->bn_g->ptr : nullptr, *b = bn && bn->affine ? bn->bn_b->ptr : nullptr;
+        const float *mean = bn ? bn->mean->ptr : nullptr, *var = bn ? bn->variance->ptr : nullptr;
+        const float eps = bn ? bn->epsilon : 0.0f;
+        const float *res = s.res ? s.res->output->ptr : nullptr;
+        if (s.src2 != nullptr)
+            gpu_check(eddlhip_conv2d_fwd_concat(device, I->ptr, s.src2->output->ptr, D->K->ptr, bias, O->ptr, I->shape[0], 2 * I->shape[1],
+                                                I->shape[2], I->shape[3], D->nk, D->kr, D->kc, D->sr, D->sc, s.pad_top, s.pad_left, D->r,
+                                                D->c, g, b, mean, var, eps, res, s.relu ? 1 : 0),
+                      "Net::forward (fused convolution over two tensors)");
+        else
+            gpu_check(eddlhip_conv2d_fwd(device, I->ptr, D->K->ptr, bias, O->ptr, I->shape[0], I->shape[1], I->shape[2], I->shape[3], D->nk,
+                                         D->kr, D->kc, D->sr, D->sc, s.pad_top, s.pad_left, D->r, D->c, g, b, mean, var, eps, res,
+                                         s.relu ? 1 : 0),
+                      "Net::forward (fused convolution)");
         return;
     }
     LDense *dense = static_cast<LDense *>(s.first);

@@ -218,6 +218,7 @@ struct FusedStep {
     Layer *first = nullptr;     // the layer the step starts at
     Layer *last = nullptr;      // the layer whose output tensor the step writes
     Layer *src = nullptr;       // conv chains: the layer whose output is read (a folded zero pad's parent)
+    Layer *src2 = nullptr;      // conv chains: a folded channel Concat's second parent (src is then its first)
     LBatchNorm *bn = nullptr;   // conv chains: inference batch norm applied to the sums
     Layer *res = nullptr;       // conv chains: the other operand of a residual LSum
     bool relu = false;

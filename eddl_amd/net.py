@@ -366,6 +366,8 @@ class Net:
                 c = sole_child(l)
                 if c is not None and c.kind == "conv2d":
                     continue  # folded into the convolution below (its op is emitted when the conv is reached)
+            if fuse and self._concat_folds(l, sole_child):
+                continue  # the convolution below reads the two tensors itself; no concatenated copy is made
             if l.kind == "conv2d":
                 self._emit_conv(l, fuse, absorbed, sole_child)
                 continue
@@ -382,6 +384,21 @@ class Net:
                     hip.cache_conv_filters(self.dparams[id(l)]["K"])
         return self
 
+    @staticmethod
+    def _concat_folds(l, sole_child):
+        """A channel Concat of two equal-shaped 4-D tensors whose only consumer is a 1x1, 2x2 or 3x3 convolution is
+        folded into that convolution, which then takes its first and second half of the channels from the two
+        tensors (``eddlhip_conv2d_fwd_concat``): the same taps in the same order, so the same result bit for bit."""
+        if l.kind != "concat" or l.attrs["axis"] != 1 or len(l.parents) != 2 or len(l.out_shape) != 4:
+            return False
+        if list(l.parents[0].out_shape) != list(l.parents[1].out_shape) or l.parents[0] is l.parents[1]:
+            return False
+        c = sole_child(l)
+        if c is None or c.kind != "conv2d":
+            return False
+        cd = c.attrs["cd"]
+        return cd.kr == cd.kc and cd.kr in (1, 2, 3)
+
     def _emit_conv(self, l, fuse, absorbed, sole_child):
         hip, cd = self.backend, l.attrs["cd"]
         src = l.parents[0]
@@ -389,6 +406,10 @@ class Net:
         if fuse and src.kind == "pad" and id(src) not in self.out:
             t, r, b, le = src.attrs["pads"]  # (top, right, bottom, left) -> added to the conv's top/left
             pt, pl = pt + t, pl + le
+            src = src.parents[0]
+        second = None
+        if fuse and src.kind == "concat" and id(src) not in self.out:
+            second = self.out[id(src.parents[1])]
             src = src.parents[0]
         bn = res = None
         relu = False
@@ -433,12 +454,15 @@ class Net:
         R = self.out[id(res)] if res is not None else None
         N, Kf, P, Q = cd.out_shape
         _, C, H, W = src.out_shape
+        if second is not None:
+            C = 2 * C
         flops = 2 * N * Kf * cd.kz * cd.kr * cd.kc * P * Q
         nbytes = 4 * (N * C * H * W + Kf * cd.kz * cd.kr * cd.kc + N * Kf * P * Q)
         name = "+".join(m.name for m in ([l] if not chain else [l] + chain))
         if src is not l.parents[0]:
             name = l.parents[0].name + "+" + name
-        self.ops.append(Op("conv2d", name, lambda: hip.conv2D(I, dp["K"], bias, O, cd.sr, cd.sc, pt, pl, bn=dbn, residual=R, relu=relu),
+        self.ops.append(Op("conv2d", name,
+                           lambda: hip.conv2D(I, dp["K"], bias, O, cd.sr, cd.sc, pt, pl, bn=dbn, residual=R, relu=relu, second=second),
                            flops, nbytes, [l] + chain))
 
     def _emit_dense(self, l, fuse, absorbed, sole_child):

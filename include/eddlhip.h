@@ -147,6 +147,19 @@ int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bia
                        const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var,
                        float bn_eps, const float *residual, int relu);
 
+/* A channel Concat of two tensors folded into the convolution that consumes it (no counterpart in the
+ * reference, which materialises the concatenation: src/layers/merge/layer_concat.cpp:87-94 followed by
+ * LConv::forward).  The input is I_first[N,C/2,H,W] for channels [0, C/2) and I_second[N,C/2,H,W] for
+ * channels [C/2, C); C is the filters' channel count.  Every other argument, the fused epilogue and the
+ * result are those of eddlhip_conv2d_fwd on the concatenated tensor, bit for bit (same taps in the same
+ * order).  Taken by the 1x1, 2x2 and 3x3 kernels; other filter shapes are refused with EDDLHIP_EINVAL and
+ * the caller concatenates first. */
+int eddlhip_conv2d_fwd_concat(int dev, const float *I_first, const float *I_second, const float *K, const float *bias,
+                              float *O, int N, int C, int H, int W, int Kf, int R, int S, int sr, int sc,
+                              int pad_top, int pad_left, int P, int Q,
+                              const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var,
+                              float bn_eps, const float *residual, int relu);
+
 /* Selects the convolution kernel: 0 = automatic; 1 = matrix-core (MFMA) implicit GEMM;
  * 2 = the scalar direct kernel (one thread per output; taps summed in the reference's ky,kx,c
  * order with its rounding - used to cross-check the MFMA kernels on the device);

@@ -110,7 +110,7 @@ def test_unet_small(hip, oracle):
     x = np.random.default_rng(5).uniform(0, 1, (1, 1, 64, 64)).astype(np.float32)
     check_model(hip, oracle, m, x, 5)
     kinds = [op.kind for op in m.ops]
-    assert "pad" not in kinds and "batchnorm" not in kinds and kinds.count("conv2d") == 23
+    assert "pad" not in kinds and "batchnorm" not in kinds and "concat" not in kinds and kinds.count("conv2d") == 23
 
 
 def test_batch_resize_and_asymmetric_padding_exception(hip, oracle):

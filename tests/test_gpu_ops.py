@@ -229,6 +229,52 @@ def test_conv2d_every_tile_shape_and_slice_count(hip, oracle, algo):
                 assert_conv_close(ref, out, "%s tile %d slices %d: %s" % ((N, C, H, W, Kf, R, S), tile, slices, name))
 
 
+@pytest.mark.parametrize("algo", ["mfma_staged", "mfma_lds", "direct"])
+def test_conv2d_two_tensor_input_equals_conv_of_the_concatenation(hip, oracle, algo):
+    """A channel Concat folded into the convolution: channels from two tensors give, bit for bit, what the same
+    kernel gives on the concatenated tensor - 3x3, 1x1 and 2x2 filters, every tile shape, divided along K and not,
+    odd half-channel counts (a K-step that takes channels from both tensors), strides, padding, the fused epilogue."""
+    from eddl_amd import EddlHipError
+    rng = np.random.default_rng(305)
+    cases = [(3, 21, 20, 23, 70, 3, 3, 1, 1), (2, 64, 18, 18, 130, 3, 3, 1, 1), (2, 9, 21, 22, 40, 2, 2, 1, 0), (3, 37, 20, 23, 70, 1, 1, 1, 0),
+             (2, 5, 15, 17, 33, 3, 3, 2, 1), (1, 1, 9, 9, 4, 3, 3, 1, 1)]
+    for (N, Ch, H, W, Kf, R, S, st, pad) in cases:
+        a = rng.standard_normal((N, Ch, H, W), dtype=np.float32)
+        b = rng.standard_normal((N, Ch, H, W), dtype=np.float32)
+        w = (rng.standard_normal((Kf, 2 * Ch, R, S)) * np.sqrt(1.0 / (Ch * R * S))).astype(np.float32)
+        bias = rng.standard_normal(Kf, dtype=np.float32)
+        P, Q = (H + 2 * pad - R) // st + 1, (W + 2 * pad - S) // st + 1
+        res = rng.standard_normal((N, Kf, P, Q), dtype=np.float32)
+        g, bb, mean, var, eps = _bn_params(rng, Kf)
+        A, B, AB = hip.array(a), hip.array(b), hip.array(np.concatenate([a, b], axis=1))
+        Wd, Bd, Rd = hip.array(w), hip.array(bias), hip.array(res)
+        bn = (hip.array(g), hip.array(bb), hip.array(mean), hip.array(var), eps)
+        hip.set_conv_algo(algo)
+        try:
+            plans = [(-1, 1)] if algo == "direct" else [(-1, 1)] + [(t, sl) for t in range(4) for sl in (1, 3)]
+            for tile, slices in plans:
+                hip.force_conv_plan(tile, slices)
+                for kw in (dict(), dict(bn=bn, residual=Rd, relu=True)):
+                    O1, O2 = hip.empty((N, Kf, P, Q)), hip.empty((N, Kf, P, Q))
+                    hip.conv2D(AB, Wd, Bd, O1, st, st, pad, pad, **kw)
+                    name = hip.last_conv_kernel()
+                    hip.conv2D(A, Wd, Bd, O2, st, st, pad, pad, second=B, **kw)
+                    assert hip.last_conv_kernel() == name
+                    assert np.array_equal(O1.numpy(), O2.numpy()), ((N, Ch, H, W, Kf, R, S), name, sorted(kw))
+        finally:
+            hip.force_conv_plan(-1, 1)
+            hip.set_conv_algo("auto")
+        ref = oracle.conv2d(np.concatenate([a, b], axis=1), w, bias, (st, st), pad, pad, P, Q)
+        O = hip.empty((N, Kf, P, Q))
+        hip.conv2D(A, Wd, Bd, O, st, st, pad, pad, second=B)
+        assert_conv_close(ref, O.numpy(), "two tensors vs oracle %s" % ((N, Ch, H, W, Kf, R, S),))
+    # other filter shapes are refused: the caller concatenates first
+    a = hip.array(rng.standard_normal((1, 4, 12, 12), dtype=np.float32))
+    w5 = hip.array(rng.standard_normal((6, 8, 5, 5), dtype=np.float32))
+    with pytest.raises(EddlHipError, match="concatenate first"):
+        hip.conv2D(a, w5, None, hip.empty((1, 6, 8, 8)), 1, 1, 0, 0, second=a)
+
+
 def test_conv2d_linearity_and_empty_batch(hip, oracle):
     from eddl_amd.descriptors import ConvolDescriptor
     rng = np.random.default_rng(301)
