@@ -250,9 +250,11 @@ class Backend:
     def fill_(self, A, v):
         self._check(self.lib.eddlhip_fill(self.dev, A.ptr, A.size, v))
 
-    def conv2D(self, I, K, bias, O, sr, sc, padrt, padcl, bn=None, residual=None, relu=False, second=None):
+    def conv2D(self, I, K, bias, O, sr, sc, padrt, padcl, bn=None, residual=None, relu=False, second=None, upsample=None):
         """``bn`` = (g, b, mean, var, eps) device tensors (g, b may be None) or None.  ``second``: the other half
-        of the input channels as a tensor of its own (a channel Concat of ``I`` and ``second`` folded into the call)."""
+        of the input channels as a tensor of its own (a channel Concat of ``I`` and ``second`` folded into the call).
+        ``upsample`` = (rows, columns): whole factors of a nearest-neighbour UpSampling2D of ``I`` folded into the call
+        (paddings and the output size then refer to the enlarged image)."""
         N, C, H, W = I.shape
         Kf, C2, R, S = K.shape
         if second is not None:
@@ -269,7 +271,11 @@ class Backend:
             g, b, mean, var, eps = bn
         tail = (K.ptr, _ptr(bias), O.ptr, N, C, H, W, Kf, R, S, sr, sc, padrt, padcl, O.shape[2], O.shape[3], _ptr(g), _ptr(b),
                 _ptr(mean), _ptr(var), eps, _ptr(residual), int(relu))
-        if second is None:
+        if second is not None and upsample is not None:
+            raise ValueError("a two-tensor input and an upsampled input do not combine")
+        if upsample is not None:
+            self._check(self.lib.eddlhip_conv2d_fwd_upsampled(self.dev, I.ptr, int(upsample[0]), int(upsample[1]), *tail))
+        elif second is None:
             self._check(self.lib.eddlhip_conv2d_fwd(self.dev, I.ptr, *tail))
         else:
             self._check(self.lib.eddlhip_conv2d_fwd_concat(self.dev, I.ptr, second.ptr, *tail))

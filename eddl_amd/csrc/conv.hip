@@ -70,6 +70,9 @@ struct ConvParams {
     // One tensor: I2 == I, Csplit == C, Cimg == C.
     const float *I2;
     int Csplit, Cimg;
+    // Nearest-neighbour upsampling folded into the gather: the convolution sees an image of H*uh x W*uw pixels
+    // whose pixel (y, x) is the stored pixel (y / uh, x / uw).  uh == uw == 1: the stored image itself.
+    int uh, uw;
     const float *Wp;  // packed filters [rows][Mp]
     const float *K;   // original OIHW filters (scalar kernel only)
     float *O;
@@ -454,11 +457,23 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         const int op = (int)((unsigned)pq / (unsigned)p.Q), oq = pq - op * p.Q;
         const int ih0 = op * p.sr - p.pt, iw0 = oq * p.sc - p.pl;
         const int pix = img * (p.Cimg * p.H * p.W) + ih0 * p.W + iw0;
+        if (p.uh == 1 && p.uw == 1) {
 #pragma unroll
-        for (int t = 0; t < RS; t++) {
-            const int ky = t / S, kx = t % S;
-            const bool ok = pvalid && (unsigned)(ih0 + ky) < (unsigned)p.H && (unsigned)(iw0 + kx) < (unsigned)p.W;
-            voff[t] = ok ? (pix + ky * p.W + kx) * 4 : OOB;
+            for (int t = 0; t < RS; t++) {
+                const int ky = t / S, kx = t % S;
+                const bool ok = pvalid && (unsigned)(ih0 + ky) < (unsigned)p.H && (unsigned)(iw0 + kx) < (unsigned)p.W;
+                voff[t] = ok ? (pix + ky * p.W + kx) * 4 : OOB;
+            }
+        } else {  // taps address the upsampled image; each reads the stored pixel it is a copy of
+            const int base = img * (p.Cimg * p.H * p.W);
+            const unsigned Hu = (unsigned)(p.H * p.uh), Wu = (unsigned)(p.W * p.uw);
+#pragma unroll
+            for (int t = 0; t < RS; t++) {
+                const int ky = t / S, kx = t % S;
+                const unsigned y = (unsigned)(ih0 + ky), x = (unsigned)(iw0 + kx);
+                const bool ok = pvalid && y < Hu && x < Wu;
+                voff[t] = ok ? (base + (int)(y / (unsigned)p.uh) * p.W + (int)(x / (unsigned)p.uw)) * 4 : OOB;
+            }
         }
     }
     const int HW4 = p.H * p.W * 4;
@@ -915,11 +930,13 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvParams p) {
         const float *flt = p.K + (size_t)k * p.C * p.R * p.S;
         float s = 0.0f;
         for (int x = 0; x < p.R; x++) {
-            const int px = pp * p.sr + x - p.pt;
-            if (px < 0 || px >= p.H) continue;
+            const int pxu = pp * p.sr + x - p.pt;  // row in the (upsampled) image the convolution sees
+            if (pxu < 0 || pxu >= p.H * p.uh) continue;
+            const int px = pxu / p.uh;
             for (int y = 0; y < p.S; y++) {
-                const int py = q * p.sc + y - p.pl;
-                if (py < 0 || py >= p.W) continue;
+                const int pyu = q * p.sc + y - p.pl;
+                if (pyu < 0 || pyu >= p.W * p.uw) continue;
+                const int py = pyu / p.uw;
                 for (int c = 0; c < p.C; c++) {
                     const float v = c < p.Csplit ? img[((size_t)c * p.H + px) * p.W + py] : img2[((size_t)(c - p.Csplit) * p.H + px) * p.W + py];
                     s = __fadd_rn(s, __fmul_rn(flt[((size_t)c * p.R + x) * p.S + y], v));
@@ -1245,8 +1262,9 @@ namespace {
 
 // I2 == nullptr: the input is the one tensor I[N,C,H,W].  Otherwise channels [0, C/2) are I[N,C/2,H,W] and
 // channels [C/2, C) are I2[N,C/2,H,W].
-int conv2d_fwd_impl(int dev, const float *I, const float *I2, const float *K, const float *bias, float *O, int N, int C, int H, int W,
-                    int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g,
+// uh, uw > 1: the convolution runs over I enlarged uh x uw times by nearest-neighbour repetition (H, W stay the stored size).
+int conv2d_fwd_impl(int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
+                    int H, int W, int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g,
                     const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu) {
     EH_REQUIRE(N >= 0 && C > 0 && H > 0 && W > 0, "conv2d: bad input shape %dx%dx%dx%d", N, C, H, W);
     EH_REQUIRE(Kf > 0 && R > 0 && S > 0, "conv2d: bad filter shape %dx%dx%dx%d", Kf, C, R, S);
@@ -1263,6 +1281,19 @@ int conv2d_fwd_impl(int dev, const float *I, const float *I2, const float *K, co
         EH_REQUIRE(g_algo == 2 || (R == S && (R == 1 || R == 2 || R == 3)),
                    "conv2d: a two-tensor input is taken by the 1x1, 2x2 and 3x3 kernels only (filter %dx%d): concatenate first", R, S);
     }
+    if (uh != 1 || uw != 1) {
+        EH_REQUIRE(uh >= 1 && uw >= 1 && (long long)H * uh <= (1 << 20) && (long long)W * uw <= (1 << 20), "conv2d: bad upsampling factors %d x %d", uh, uw);
+        EH_REQUIRE(g_algo == 2 || (R == S && (R == 1 || R == 2 || R == 3)),
+                   "conv2d: an upsampled input is taken by the 1x1, 2x2 and 3x3 kernels only (filter %dx%d): resize first", R, S);
+        // the reference's mapping, source = (int)((float)dst / ((float)new / in)) (src/hardware/cpu/cpu_da.cpp:109-113), must be
+        // the integer division the gather uses
+        for (int axis = 0; axis < 2; axis++) {
+            const int in = axis ? W : H, u = axis ? uw : uh;
+            const float scale = (float)(in * u) / (float)in;
+            for (int d = 0; d < in * u; d++)
+                EH_REQUIRE((int)((float)d / scale) == d / u, "conv2d: upsampling %d -> %d is not a whole-pixel repetition at %d", in, in * u, d);
+        }
+    }
     const long long img_elems = (long long)Cimg * H * W;
     EH_REQUIRE(img_elems <= (1LL << 28), "conv2d: one image of %lld elements exceeds the 1 GiB a buffer descriptor may cover", img_elems);
     EH_REQUIRE((long long)C * R * S <= (1LL << 24), "conv2d: filter too large");
@@ -1275,6 +1306,7 @@ int conv2d_fwd_impl(int dev, const float *I, const float *I2, const float *K, co
 
     ConvParams p;
     p.I = I; p.I2 = two ? I2 : I; p.Csplit = two ? C / 2 : C; p.Cimg = Cimg;
+    p.uh = uh; p.uw = uw;
     p.K = K; p.O = O; p.Wp = nullptr;
     p.bias = bias; p.bn_g = bn_g; p.bn_b = bn_b; p.bn_mean = bn_mean; p.bn_var = bn_var; p.residual = residual;
     p.bn_eps = bn_eps; p.relu = relu;
@@ -1402,7 +1434,7 @@ extern "C" {
 int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bias, float *O, int N, int C, int H, int W, int Kf,
                        int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b,
                        const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu) {
-    return conv2d_fwd_impl(dev, I, nullptr, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean,
+    return conv2d_fwd_impl(dev, I, nullptr, 1, 1, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean,
                            bn_var, bn_eps, residual, relu);
 }
 
@@ -1412,7 +1444,15 @@ int eddlhip_conv2d_fwd_concat(int dev, const float *I_first, const float *I_seco
                               const float *residual, int relu) {
     EH_REQUIRE(N == 0 || (I_first && I_second), "conv2d_fwd_concat: NULL input tensor");
     if (N == 0) return 0;
-    return conv2d_fwd_impl(dev, I_first, I_second, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
+    return conv2d_fwd_impl(dev, I_first, I_second, 1, 1, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
+                           bn_mean, bn_var, bn_eps, residual, relu);
+}
+
+int eddlhip_conv2d_fwd_upsampled(int dev, const float *I, int up_h, int up_w, const float *K, const float *bias, float *O, int N, int C,
+                                 int H, int W, int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q,
+                                 const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps,
+                                 const float *residual, int relu) {
+    return conv2d_fwd_impl(dev, I, nullptr, up_h, up_w, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
                            bn_mean, bn_var, bn_eps, residual, relu);
 }
 

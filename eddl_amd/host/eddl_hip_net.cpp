@@ -567,6 +567,20 @@ void Net::fuse() {
                 continue;
             }
         }
+        if (LResize *rs = dynamic_cast<LResize *>(l)) {
+            // a nearest upsampling by whole factors read only by a 1x1, 2x2 or 3x3 convolution, directly or through a zero
+            // pad that the convolution absorbs: folded into the convolution's gather (eddlhip_conv2d_fwd_upsampled)
+            Layer *c = sole_child(l);
+            if (LPad *pad = dynamic_cast<LPad *>(c))
+                if (pad->constant == 0.0f) c = sole_child(pad);
+            LConv *cv = dynamic_cast<LConv *>(c);
+            const Tensor *in = rs->parent[0]->output;
+            if (cv != nullptr && in->ndim == 4 && rs->new_shape[0] % in->shape[2] == 0 && rs->new_shape[1] % in->shape[3] == 0 &&
+                cv->cd->kernel_size[0] == cv->cd->kernel_size[1] && cv->cd->kernel_size[0] >= 1 && cv->cd->kernel_size[0] <= 3) {
+                fused_away.push_back(l);
+                continue;
+            }
+        }
         if (LConcat *cat = dynamic_cast<LConcat *>(l)) {
             // a channel Concat of two equal-shaped 4-D tensors read only by a 1x1, 2x2 or 3x3 convolution: that
             // convolution takes the two halves of its channels from the two tensors (eddlhip_conv2d_fwd_concat)
@@ -588,6 +602,13 @@ void Net::fuse() {
                     s.pad_top += pad->padding[0];   // (top, right, bottom, left)
                     s.pad_left += pad->padding[3];
                     s.src = pad->parent[0];
+                }
+            }
+            if (LResize *rs = dynamic_cast<LResize *>(s.src)) {
+                if (is_fused_away(rs)) {
+                    s.src = rs->parent[0];
+                    s.up_h = rs->new_shape[0] / s.src->output->shape[2];
+                    s.up_w = rs->new_shape[1] / s.src->output->shape[3];
                 }
             }
             if (LConcat *cat = dynamic_cast<LConcat *>(s.src)) {
@@ -669,7 +690,12 @@ void Net::run_step(const FusedStep &s) {
         const float *mean = bn ? bn->mean->ptr : nullptr, *var = bn ? bn->variance->ptr : nullptr;
         const float eps = bn ? bn->epsilon : 0.0f;
         const float *res = s.res ? s.res->output->ptr : nullptr;
-        if (s.src2 != nullptr)
+        if (s.up_h != 1 || s.up_w != 1)
+            gpu_check(eddlhip_conv2d_fwd_upsampled(device, I->ptr, s.up_h, s.up_w, D->K->ptr, bias, O->ptr, I->shape[0], I->shape[1],
+                                                   I->shape[2], I->shape[3], D->nk, D->kr, D->kc, D->sr, D->sc, s.pad_top, s.pad_left,
+                                                   D->r, D->c, g, b, mean, var, eps, res, s.relu ? 1 : 0),
+                      "Net::forward (fused convolution over an upsampled tensor)");
+        else if (s.src2 != nullptr)
             gpu_check(eddlhip_conv2d_fwd_concat(device, I->ptr, s.src2->output->ptr, D->K->ptr, bias, O->ptr, I->shape[0], 2 * I->shape[1],
                                                 I->shape[2], I->shape[3], D->nk, D->kr, D->kc, D->sr, D->sc, s.pad_top, s.pad_left, D->r,
                                                 D->c, g, b, mean, var, eps, res, s.relu ? 1 : 0),

@@ -223,6 +223,7 @@ struct FusedStep {
     Layer *res = nullptr;       // conv chains: the other operand of a residual LSum
     bool relu = false;
     int pad_top = 0, pad_left = 0;
+    int up_h = 1, up_w = 1;     // conv chains: whole factors of a folded nearest UpSampling2D (src is then its parent)
     bool chain = false;         // false: first->forward()
 };
 

@@ -368,6 +368,8 @@ class Net:
                     continue  # folded into the convolution below (its op is emitted when the conv is reached)
             if fuse and self._concat_folds(l, sole_child):
                 continue  # the convolution below reads the two tensors itself; no concatenated copy is made
+            if fuse and self._resize_folds(l, sole_child):
+                continue  # the convolution below reads the small tensor through the upsampling's index map
             if l.kind == "conv2d":
                 self._emit_conv(l, fuse, absorbed, sole_child)
                 continue
@@ -399,6 +401,24 @@ class Net:
         cd = c.attrs["cd"]
         return cd.kr == cd.kc and cd.kr in (1, 2, 3)
 
+    @staticmethod
+    def _resize_folds(l, sole_child):
+        """A nearest UpSampling2D by whole factors whose only consumer is a 1x1, 2x2 or 3x3 convolution - directly
+        or through a zero Pad that the convolution absorbs - is folded into that convolution's gather
+        (``eddlhip_conv2d_fwd_upsampled``): the enlarged tensor is never written."""
+        if l.kind != "resize" or len(l.out_shape) != 4:
+            return False
+        (H, W), (NH, NW) = l.parents[0].out_shape[2:], l.attrs["new_shape"]
+        if NH % H or NW % W or list(l.out_shape[2:]) != [NH, NW]:
+            return False
+        c = sole_child(l)
+        if c is not None and c.kind == "pad" and c.attrs["constant"] == 0.0:
+            c = sole_child(c)
+        if c is None or c.kind != "conv2d":
+            return False
+        cd = c.attrs["cd"]
+        return cd.kr == cd.kc and cd.kr in (1, 2, 3)
+
     def _emit_conv(self, l, fuse, absorbed, sole_child):
         hip, cd = self.backend, l.attrs["cd"]
         src = l.parents[0]
@@ -406,6 +426,11 @@ class Net:
         if fuse and src.kind == "pad" and id(src) not in self.out:
             t, r, b, le = src.attrs["pads"]  # (top, right, bottom, left) -> added to the conv's top/left
             pt, pl = pt + t, pl + le
+            src = src.parents[0]
+        upsample = None
+        if fuse and src.kind == "resize" and id(src) not in self.out:
+            (NH, NW), (H0, W0) = src.attrs["new_shape"], src.parents[0].out_shape[2:]
+            upsample = (NH // H0, NW // W0)
             src = src.parents[0]
         second = None
         if fuse and src.kind == "concat" and id(src) not in self.out:
@@ -462,7 +487,8 @@ class Net:
         if src is not l.parents[0]:
             name = l.parents[0].name + "+" + name
         self.ops.append(Op("conv2d", name,
-                           lambda: hip.conv2D(I, dp["K"], bias, O, cd.sr, cd.sc, pt, pl, bn=dbn, residual=R, relu=relu, second=second),
+                           lambda: hip.conv2D(I, dp["K"], bias, O, cd.sr, cd.sc, pt, pl, bn=dbn, residual=R, relu=relu, second=second,
+                                              upsample=upsample),
                            flops, nbytes, [l] + chain))
 
     def _emit_dense(self, l, fuse, absorbed, sole_child):

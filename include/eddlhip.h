@@ -160,6 +160,20 @@ int eddlhip_conv2d_fwd_concat(int dev, const float *I_first, const float *I_seco
                               const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var,
                               float bn_eps, const float *residual, int relu);
 
+/* Nearest-neighbour UpSampling2D by whole factors folded into the convolution that consumes it (no counterpart in
+ * the reference, which writes the enlarged tensor: src/layers/core/layer_resize.cpp:22-47 followed by
+ * LConv::forward).  I[N,C,H,W] is the tensor BEFORE upsampling; the convolution runs over the image of
+ * H*up_h x W*up_w pixels whose pixel (y, x) is I's pixel (y / up_h, x / up_w) - the mapping of the reference's
+ * nearest / asymmetric scale for whole factors (src/hardware/cpu/cpu_da.cpp:109-113; checked on the host, the call
+ * is refused where the two differ).  pad_top / pad_left, P and Q refer to the enlarged image.  Everything else,
+ * and the result, are those of eddlhip_conv2d_fwd on the enlarged tensor, bit for bit.  Taken by the 1x1, 2x2 and
+ * 3x3 kernels; other filter shapes are refused with EDDLHIP_EINVAL and the caller resizes first. */
+int eddlhip_conv2d_fwd_upsampled(int dev, const float *I, int up_h, int up_w, const float *K, const float *bias, float *O,
+                                 int N, int C, int H, int W, int Kf, int R, int S, int sr, int sc,
+                                 int pad_top, int pad_left, int P, int Q,
+                                 const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var,
+                                 float bn_eps, const float *residual, int relu);
+
 /* Selects the convolution kernel: 0 = automatic; 1 = matrix-core (MFMA) implicit GEMM;
  * 2 = the scalar direct kernel (one thread per output; taps summed in the reference's ky,kx,c
  * order with its rounding - used to cross-check the MFMA kernels on the device);

@@ -275,6 +275,49 @@ def test_conv2d_two_tensor_input_equals_conv_of_the_concatenation(hip, oracle, a
         hip.conv2D(a, w5, None, hip.empty((1, 6, 8, 8)), 1, 1, 0, 0, second=a)
 
 
+@pytest.mark.parametrize("algo", ["mfma_staged", "mfma_lds", "direct"])
+def test_conv2d_upsampled_input_equals_conv_of_the_resized_tensor(hip, oracle, algo):
+    """Nearest UpSampling2D by whole factors folded into the gather: bit for bit what the same kernel gives on the
+    tensor the resize kernel writes - the decoder shape (x2, zero pad right/bottom, 2x2 valid), 3x3 same, 1x1,
+    unequal factors, strides, every tile shape, divided along K and not."""
+    from eddl_amd import EddlHipError
+    rng = np.random.default_rng(306)
+    # N, C, H, W, Kf, R, S, stride, (pad_top, pad_left), (extra bottom, extra right), (uh, uw)
+    cases = [(2, 24, 9, 11, 20, 2, 2, 1, (0, 0), (1, 1), (2, 2)), (3, 21, 10, 12, 70, 3, 3, 1, (1, 1), (1, 1), (2, 2)),
+             (2, 37, 7, 9, 40, 1, 1, 1, (0, 0), (0, 0), (3, 2)), (2, 64, 8, 8, 130, 3, 3, 2, (1, 1), (1, 1), (2, 3)),
+             (1, 3, 5, 6, 4, 3, 3, 1, (1, 1), (1, 1), (1, 4))]
+    for (N, C, H, W, Kf, R, S, st, (pt, pl), (pb, pr), (uh, uw)) in cases:
+        x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+        w = (rng.standard_normal((Kf, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32)
+        bias = rng.standard_normal(Kf, dtype=np.float32)
+        Hu, Wu = H * uh, W * uw
+        P, Q = (Hu + pt + pb - R) // st + 1, (Wu + pl + pr - S) // st + 1
+        X, Wd, Bd = hip.array(x), hip.array(w), hip.array(bias)
+        XU = hip.empty((N, C, Hu, Wu))
+        hip.scale(X, XU, (Hu, Wu))
+        assert np.array_equal(XU.numpy(), oracle.scale_nearest(x, (Hu, Wu)))
+        hip.set_conv_algo(algo)
+        try:
+            plans = [(-1, 1)] if algo == "direct" else [(-1, 1)] + [(t, sl) for t in range(4) for sl in (1, 3)]
+            for tile, slices in plans:
+                hip.force_conv_plan(tile, slices)
+                O1, O2 = hip.empty((N, Kf, P, Q)), hip.empty((N, Kf, P, Q))
+                hip.conv2D(XU, Wd, Bd, O1, st, st, pt, pl, relu=True)
+                name = hip.last_conv_kernel()
+                hip.conv2D(X, Wd, Bd, O2, st, st, pt, pl, relu=True, upsample=(uh, uw))
+                assert hip.last_conv_kernel() == name
+                assert np.array_equal(O1.numpy(), O2.numpy()), ((N, C, H, W, Kf, R, S, uh, uw), name)
+        finally:
+            hip.force_conv_plan(-1, 1)
+            hip.set_conv_algo("auto")
+    x = hip.array(rng.standard_normal((1, 4, 6, 6), dtype=np.float32))
+    w5 = hip.array(rng.standard_normal((6, 4, 5, 5), dtype=np.float32))
+    with pytest.raises(EddlHipError, match="resize first"):
+        hip.conv2D(x, w5, None, hip.empty((1, 6, 8, 8)), 1, 1, 0, 0, upsample=(2, 2))
+    with pytest.raises(EddlHipError, match="bad upsampling factors"):
+        hip.conv2D(x, hip.array(np.zeros((6, 4, 3, 3), np.float32)), None, hip.empty((1, 6, 4, 4)), 1, 1, 0, 0, upsample=(0, 2))
+
+
 def test_conv2d_linearity_and_empty_batch(hip, oracle):
     from eddl_amd.descriptors import ConvolDescriptor
     rng = np.random.default_rng(301)
