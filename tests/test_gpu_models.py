@@ -206,3 +206,32 @@ def test_captured_plan_replays_bit_for_bit(hip, oracle):
     g = hip.record(m.run)
     g.launch()
     hip.synchronize()
+
+
+def test_bench_line_carries_the_contract_fields(hip):
+    """bench.py on the smallest workload: ONE JSON line with the agreed fields, roofline and CPU baseline with its
+    end-to-end parity gate; the layer-by-layer and recorded-plan modes run too."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from conftest import ROOT
+    base = [sys.executable, os.path.join(ROOT, "bench.py"), "--workload", "conv", "--steps", "5", "--warmup", "2", "--no-device-probe"]
+    res = subprocess.run(base, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-2000:]
+    lines = [l for l in res.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    r = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
+                "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in r, key
+    assert r["n_gpus"] == 1 and r["steps"] == 5 and r["warmup"] == 2 and r["dtype"] == "f32" and r["vs_baseline"] is None
+    assert r["value"] > 0 and "workload" in r["config"]
+    rf = r["roofline"]
+    assert rf["bound"] in ("hbm", "mfma") and rf["peak"] == 157.3 and abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-9
+    cb = r["cpu_baseline"]
+    assert cb["kind"] == "port" and cb["cores"] >= 1 and cb["value"] > 0 and cb["parity"]["ok"]
+    for extra in (["--unfused"], ["--graph"]):
+        res = subprocess.run(base + ["--no-cpu-baseline"] + extra, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+        assert res.returncode == 0, res.stderr[-2000:]
+        assert json.loads(res.stdout.strip().splitlines()[-1])["value"] > 0
