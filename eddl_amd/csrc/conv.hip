@@ -135,6 +135,11 @@ __device__ __forceinline__ float apply_epilogue(const ConvParams &p, const Chann
 // filled from the buffer being read), which would serialise the loads of step t+1 with the MFMAs
 // of step t.  With the instruction opaque to it, the kernel places the one wait that is needed
 // itself: vmcnt(0) before the barrier that publishes the buffer.
+// The statements write M0 without declaring it: the compiler treats M0 as a reserved register, warns about it in
+// a clobber list and does not promise to honour it there.  Its own uses of M0 (indexed register access, message
+// sends, its LDS-direct builtin) set the register immediately before the instruction that reads it, and the
+// kernels of this file contain none of them between these statements (every register array is indexed by
+// compile-time constants after unrolling).
 __device__ __forceinline__ int32x4 make_rsrc_words(const void *base, unsigned bytes) {
     const unsigned long long a = (unsigned long long)base;
     int32x4 r;
@@ -1186,6 +1191,8 @@ int eddlhip_conv2d_cache_filters(int dev, const float *K, int Kf, int C, int R, 
     e.Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
     e.Wp = nullptr;
     e.stale = true;
+    EH_REQUIRE((size_t)e.rows * e.Mp * sizeof(float) < ((size_t)1 << 31),
+               "conv2d_cache_filters: the repacked filter matrix (%d taps x %d channels) exceeds the 2 GiB a buffer descriptor covers", e.rows, e.Mp);
     EH_TRY_HIP(hipMalloc((void **)&e.Wp, (size_t)e.rows * e.Mp * sizeof(float)));
     int rc = repack(dev, e);
     if (rc != 0) {
@@ -1365,6 +1372,9 @@ int conv2d_fwd_impl(int dev, const float *I, const float *I2, int uh, int uw, co
     // ---- packed filters (the registered copy, or a repack into the workspace), then the partial
     // tiles of the K-split launch
     const int rows = p.nsteps * bk;
+    // the kernels address the packed filters through a buffer descriptor with 32-bit byte offsets
+    EH_REQUIRE((size_t)rows * p.Mp * sizeof(float) < ((size_t)1 << 31),
+               "conv2d: the repacked filter matrix (%d taps x %d channels) exceeds the 2 GiB a buffer descriptor covers", rows, p.Mp);
     const float *cached = nullptr;
     {
         std::lock_guard<std::mutex> lock(g_cache_mutex);
