@@ -48,6 +48,7 @@ PROTOTYPES = {
     "eddlhip_probe_mfma_f32": [c_int, c_int, c_int, ctypes.POINTER(c_float), ctypes.POINTER(c_float), ctypes.POINTER(c_float)],
     "eddlhip_probe_hbm": [c_int, c_size_t, ctypes.POINTER(c_float), ctypes.POINTER(c_float), ctypes.POINTER(c_float)],
     "eddlhip_conv2d_fwd": [c_int, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
+    "eddlhip_conv2d_fwd_noalloc": [c_int, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_fwd_concat": [c_int, P, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_fwd_upsampled": [c_int, P, c_int, c_int, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_cache_filters": [c_int, P, c_int, c_int, c_int, c_int],

@@ -37,6 +37,9 @@ int get_workspace(int dev, size_t bytes, void **ptr);
 // change is repacked before its next use and one that is freed is forgotten.
 void conv_filters_written(int dev, const void *dst, size_t bytes);
 void conv_filters_released(int dev, const void *base, size_t bytes);
+// Per-device set-up of the convolution code (address of its fixed scratch array, kernel occupancies);
+// use_device calls it once, when it initialises the device.
+int conv_setup_device(int dev);
 
 }  // namespace eddlhip
 

@@ -50,7 +50,16 @@
 
 using namespace eddlhip;
 
+// Device memory of eddlhip_conv2d_fwd_noalloc: what eddlhip_conv2d_fwd takes from the library's grow-only
+// workspace (repacked filters, tap table, partial tiles of a K-split launch) comes out of this fixed array
+// instead, so that entry point never allocates.  Each device the library runs on holds its own copy, at its
+// own address, until the process ends.  In host code the name is only a handle for hipGetSymbolAddress:
+// conv_setup_device asks for the device address once per device and everything else uses that pointer.
+static __device__ __align__(256) unsigned char scratch[EDDLHIP_CONV_NOALLOC_SCRATCH_BYTES];
+
 namespace {
+
+void *g_scratch_ptr[EDDLHIP_MAX_DEVICES];  // device address of `scratch` on each initialised device
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -1086,6 +1095,18 @@ Plan plan_conv(const Variant *family, int Kf, int C, int RS, long long npix, int
     return best;
 }
 
+// Resident workgroups per CU of each variant of a family, asked of the runtime once.
+int family_occupancy(const Variant *family) {
+    for (int t = 0; t < 4; t++) {
+        if (family[t].occupancy == 0) {
+            int occ = 0;
+            EH_TRY_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, family[t].kernel, 256, 0));
+            family[t].occupancy = occ > 0 ? occ : 1;
+        }
+    }
+    return 0;
+}
+
 // A plan with a given tile shape and slice count (every leftover tile is divided; with fewer
 // tiles than CUs that is every tile).
 Plan forced_plan(const Variant *family, int tile, int slices, int Kf, int C, int RS, long long npix, int num_cu) {
@@ -1139,6 +1160,19 @@ int repack(int dev, CachedFilters &e) {
 }  // namespace
 
 namespace eddlhip {
+
+// Called once per device from the library's initialisation, with that device current: looks up where this
+// device keeps its copy of `scratch`, and asks the runtime how many workgroups of each kernel variant fit
+// on a CU (the launch planner's input), so that eddlhip_conv2d_fwd_noalloc finds both ready.
+int conv_setup_device(int dev) {
+    void *ptr = nullptr;
+    EH_TRY_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    EH_REQUIRE(ptr != nullptr, "device %d: no address for the convolution scratch array", dev);
+    g_scratch_ptr[dev] = ptr;
+    for (const Variant(*fam)[4] : {k3x3, k1x1, k2x2, kgen})
+        for (int d = 0; d < 2; d++) EH_TRY(family_occupancy(fam[d]));
+    return 0;
+}
 
 void conv_filters_written(int dev, const void *dst, size_t bytes) {
     if (dev < 0 || dev >= EDDLHIP_MAX_DEVICES) return;
@@ -1270,7 +1304,9 @@ namespace {
 // I2 == nullptr: the input is the one tensor I[N,C,H,W].  Otherwise channels [0, C/2) are I[N,C/2,H,W] and
 // channels [C/2, C) are I2[N,C/2,H,W].
 // uh, uw > 1: the convolution runs over I enlarged uh x uw times by nearest-neighbour repetition (H, W stay the stored size).
-int conv2d_fwd_impl(int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
+// no_alloc: take the scratch memory from the device's fixed array instead of the workspace, and refuse whatever
+// would allocate (an uninitialised device, a need beyond the array, event pairs for the measurement hook).
+int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
                     int H, int W, int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g,
                     const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu) {
     EH_REQUIRE(N >= 0 && C > 0 && H > 0 && W > 0, "conv2d: bad input shape %dx%dx%dx%d", N, C, H, W);
@@ -1307,6 +1343,11 @@ int conv2d_fwd_impl(int dev, const float *I, const float *I2, int uh, int uw, co
     EH_REQUIRE((long long)P * Q <= 0x7fffffffLL, "conv2d: output plane too large");
     if (N == 0) return 0;
     EH_REQUIRE(I && K && O, "conv2d: NULL tensor");
+    if (no_alloc) {
+        EH_REQUIRE(dev >= 0 && dev < EDDLHIP_MAX_DEVICES && state(dev).inited && g_scratch_ptr[dev] != nullptr,
+                   "conv2d_fwd_noalloc: device %d is not initialised; call eddlhip_init(%d) first (initialisation allocates)", dev, dev);
+        EH_REQUIRE(!g_prof_on, "conv2d_fwd_noalloc: not while eddlhip_conv2d_profile collects (its event pairs are allocated)");
+    }
     EH_TRY(use_device(dev));
     EH_REQUIRE(!(g_prof_on && state(dev).capturing), "conv2d: launches cannot be timed (eddlhip_conv2d_profile) while a graph is being recorded");
     hipStream_t st = state(dev).stream;
@@ -1345,13 +1386,7 @@ int conv2d_fwd_impl(int dev, const float *I, const float *I2, int uh, int uw, co
     else if (R == 1 && S == 1) family = k1x1[direct];
     else if (R == 2 && S == 2) family = k2x2[direct];
     else family = kgen[direct];
-    for (int t = 0; t < 4; t++) {
-        if (family[t].occupancy == 0) {
-            int occ = 0;
-            EH_TRY_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, family[t].kernel, 256, 0));
-            family[t].occupancy = occ > 0 ? occ : 1;
-        }
-    }
+    EH_TRY(family_occupancy(family));
     // a launch covers one batch chunk: input within the 2 GiB a buffer descriptor addresses with 32-bit
     // offsets, and fewer than 2^31 output pixels (32-bit pixel arithmetic in the kernels)
     long long max_imgs = (1LL << 29) / img_elems;
@@ -1390,7 +1425,16 @@ int conv2d_fwd_impl(int dev, const float *I, const float *I2, int uh, int uw, co
     const size_t taps_bytes = v->cpb ? 0 : (((size_t)rows * sizeof(int32x4) + 255) & ~(size_t)255);
     const size_t partial_bytes = (size_t)nslices * leftover * tile_floats * sizeof(float);
     void *ws = nullptr;
-    EH_TRY(get_workspace(dev, wp_bytes + taps_bytes + partial_bytes, &ws));
+    if (no_alloc) {
+        const size_t need = wp_bytes + taps_bytes + partial_bytes;
+        EH_REQUIRE(need <= (size_t)EDDLHIP_CONV_NOALLOC_SCRATCH_BYTES,
+                   "conv2d_fwd_noalloc: this call needs %zu bytes of scratch memory (%zu repacked filters + %zu tap table + %zu partial "
+                   "tiles); the fixed array holds %zu.  Register the filters (eddlhip_conv2d_cache_filters) or call eddlhip_conv2d_fwd",
+                   need, wp_bytes, taps_bytes, partial_bytes, (size_t)EDDLHIP_CONV_NOALLOC_SCRATCH_BYTES);
+        ws = g_scratch_ptr[dev];
+    } else {
+        EH_TRY(get_workspace(dev, wp_bytes + taps_bytes + partial_bytes, &ws));
+    }
     p.Wp = cached ? cached : (const float *)ws;
     p.wp_bytes = (unsigned)((size_t)rows * p.Mp * sizeof(float));
     p.taps = (const int32x4 *)((char *)ws + wp_bytes);
@@ -1444,7 +1488,7 @@ extern "C" {
 int eddlhip_conv2d_fwd(int dev, const float *I, const float *K, const float *bias, float *O, int N, int C, int H, int W, int Kf,
                        int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b,
                        const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu) {
-    return conv2d_fwd_impl(dev, I, nullptr, 1, 1, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean,
+    return conv2d_fwd_impl(false, dev, I, nullptr, 1, 1, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean,
                            bn_var, bn_eps, residual, relu);
 }
 
@@ -1454,7 +1498,7 @@ int eddlhip_conv2d_fwd_concat(int dev, const float *I_first, const float *I_seco
                               const float *residual, int relu) {
     EH_REQUIRE(N == 0 || (I_first && I_second), "conv2d_fwd_concat: NULL input tensor");
     if (N == 0) return 0;
-    return conv2d_fwd_impl(dev, I_first, I_second, 1, 1, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
+    return conv2d_fwd_impl(false, dev, I_first, I_second, 1, 1, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
                            bn_mean, bn_var, bn_eps, residual, relu);
 }
 
@@ -1462,7 +1506,15 @@ int eddlhip_conv2d_fwd_upsampled(int dev, const float *I, int up_h, int up_w, co
                                  int H, int W, int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q,
                                  const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps,
                                  const float *residual, int relu) {
-    return conv2d_fwd_impl(dev, I, nullptr, up_h, up_w, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
+    return conv2d_fwd_impl(false, dev, I, nullptr, up_h, up_w, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
+                           bn_mean, bn_var, bn_eps, residual, relu);
+}
+
+int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const float *bias, float *O, int N, int C, int H, int W, int Kf,
+                               int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g,
+                               const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps, const float *residual,
+                               int relu) {
+    return conv2d_fwd_impl(true, dev, I, nullptr, 1, 1, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
                            bn_mean, bn_var, bn_eps, residual, relu);
 }
 

@@ -37,6 +37,7 @@ int use_device(int dev) {
         s.num_cu = prop.multiProcessorCount;
         EH_TRY_HIP(hipMalloc(&s.flag, 256));
         EH_TRY_HIP(hipMemset(s.flag, 0, 256));
+        EH_TRY(conv_setup_device(dev));
         s.inited = true;
         return 0;
     }

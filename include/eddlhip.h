@@ -174,6 +174,27 @@ int eddlhip_conv2d_fwd_upsampled(int dev, const float *I, int up_h, int up_w, co
                                  const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var,
                                  float bn_eps, const float *residual, int relu);
 
+/* eddlhip_conv2d_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid it).  No counterpart in the reference.  Same arguments, same kernels,
+ * same launch plan and therefore the same result, bit for bit, as eddlhip_conv2d_fwd; the difference is where
+ * the call's scratch memory comes from (the repacked filters unless they are registered with
+ * eddlhip_conv2d_cache_filters, the tap table of filter shapes other than 1x1 / 2x2 / 3x3, the partial tiles of
+ * a K-split launch): a fixed array of EDDLHIP_CONV_NOALLOC_SCRATCH_BYTES in the library's device image, one copy
+ * per device, instead of the grow-only workspace.  The call makes no hipMalloc / hipFree and no allocating
+ * library call.  It returns EDDLHIP_EINVAL, and launches nothing, when
+ *   - the device has not been initialised (call eddlhip_init(dev) once beforehand; that call allocates),
+ *   - the scratch need exceeds the array (the message gives the figures),
+ *   - eddlhip_conv2d_profile is collecting (its event pairs are allocated on demand).
+ * Every call on a device uses that device's one array, which keeps the previous call's contents; each call
+ * writes what it reads from it before reading, so nothing has to be cleared, but two calls that overlap on
+ * one device (from two threads, or on two streams) race on it. */
+#define EDDLHIP_CONV_NOALLOC_SCRATCH_BYTES (64u << 20)
+int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const float *bias, float *O,
+                               int N, int C, int H, int W, int Kf, int R, int S, int sr, int sc,
+                               int pad_top, int pad_left, int P, int Q,
+                               const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var,
+                               float bn_eps, const float *residual, int relu);
+
 /* Selects the convolution kernel: 0 = automatic; 1 = matrix-core (MFMA) implicit GEMM;
  * 2 = the scalar direct kernel (one thread per output; taps summed in the reference's ky,kx,c
  * order with its rounding - used to cross-check the MFMA kernels on the device);
