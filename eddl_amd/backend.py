@@ -139,6 +139,7 @@ class Backend:
     def __init__(self, dev=0):
         self.lib = _lib.load()
         self.dev = int(dev)
+        self._deferred_free = []  # pointers whose free was refused (a graph was being recorded)
         self._check(self.lib.eddlhip_init(self.dev))
 
     # ---- plumbing
@@ -152,7 +153,21 @@ class Backend:
         return p.value
 
     def _free(self, ptr):
-        self.lib.eddlhip_free(self.dev, ptr)
+        """Frees device memory; a free is refused while a graph is being recorded (``record``), so such a pointer is
+        kept and freed when the recording has ended."""
+        if self.lib.eddlhip_free(self.dev, ptr) != 0:
+            self._deferred_free.append(ptr)
+
+    def _free_deferred(self):
+        pending, self._deferred_free = self._deferred_free, []
+        for ptr in pending:
+            if self.lib.eddlhip_free(self.dev, ptr) != 0:
+                self._deferred_free.append(ptr)
+
+    def workspace_bytes(self):
+        n = ctypes.c_size_t()
+        self._check(self.lib.eddlhip_workspace_bytes(self.dev, ctypes.byref(n)))
+        return n.value
 
     def record(self, fn):
         """Records the launches ``fn()`` makes into a Graph instead of running them.  ``fn`` must have
@@ -165,8 +180,11 @@ class Backend:
             self.lib.eddlhip_graph_end(self.dev, ctypes.byref(h))  # leaves recording mode; the first error is the one to report
             if h.value:
                 self.lib.eddlhip_graph_destroy(self.dev, h)
+            self._free_deferred()
             raise
-        self._check(self.lib.eddlhip_graph_end(self.dev, ctypes.byref(h)))
+        rc = self.lib.eddlhip_graph_end(self.dev, ctypes.byref(h))
+        self._free_deferred()
+        self._check(rc)
         return Graph(self, h)
 
     @property

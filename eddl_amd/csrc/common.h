@@ -17,6 +17,8 @@ struct DeviceState {
     int num_cu = 0;
     void *workspace = nullptr;  // private, grow-only (repacked filters, split-K partials)
     size_t workspace_bytes = 0;
+    unsigned long workspace_generation = 0;  // counts replacements of the workspace by a larger one
+    bool capture_used_workspace = false;     // a call recorded into the graph being captured took the workspace
     void *flag = nullptr;  // one int of device memory for kernels that report a condition
     hipStream_t copy_stream[2] = {nullptr, nullptr};  // uploads, downloads: created on first use (non-blocking, default priority)
     // eddlhip_graph_begin .. _end: launches go to capture_stream and are recorded, not run

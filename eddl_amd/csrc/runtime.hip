@@ -64,7 +64,9 @@ int get_workspace(int dev, size_t bytes, void **ptr) {
             return set_error(EDDLHIP_ENOMEM, "workspace of %zu bytes: %s", want, hipGetErrorString(e));
         }
         s.workspace_bytes = want;
+        s.workspace_generation++;
     }
+    if (s.capturing && bytes > 0) s.capture_used_workspace = true;
     *ptr = s.workspace;
     return 0;
 }
@@ -100,7 +102,16 @@ int eddlhip_shutdown(int dev) {
     for (hipStream_t cs : s.copy_stream)
         if (cs) EH_TRY_HIP(hipStreamDestroy(cs));
     if (s.capture_stream) EH_TRY_HIP(hipStreamDestroy(s.capture_stream));
+    const unsigned long generation = s.workspace_generation;
     s = DeviceState();
+    s.workspace_generation = generation + 1;  // graphs recorded before the shutdown name a workspace that is gone
+    return 0;
+}
+
+int eddlhip_workspace_bytes(int dev, size_t *bytes) {
+    EH_REQUIRE(bytes != nullptr, "bytes is NULL");
+    EH_TRY(use_device(dev));
+    *bytes = state(dev).workspace_bytes;
     return 0;
 }
 
@@ -268,6 +279,19 @@ int eddlhip_download_wait_event(int dev, void *event) {
 
 // ---- graphs: a fixed sequence of launches recorded once and replayed with one call, for plans whose
 // kernels are so short that queueing them one by one takes longer than running them
+//
+// A recorded kernel that took the library's workspace has that address frozen into its arguments, and the
+// workspace is replaced (freed) when a later call needs a larger one.  The handle therefore remembers which
+// workspace the recording saw, and a replay after a replacement is refused instead of writing into freed memory.
+namespace {
+struct RecordedGraph {
+    hipGraphExec_t exec;
+    int dev;
+    bool uses_workspace;
+    unsigned long workspace_generation;
+};
+}  // namespace
+
 int eddlhip_graph_begin(int dev) {
     EH_TRY(use_device(dev));
     DeviceState &s = state(dev);
@@ -277,6 +301,7 @@ int eddlhip_graph_begin(int dev) {
     s.stream_before_capture = s.stream;
     s.stream = s.capture_stream;
     s.capturing = true;
+    s.capture_used_workspace = false;
     return 0;
 }
 
@@ -303,7 +328,7 @@ int eddlhip_graph_end(int dev, void **graph) {
         (void)hipGetLastError();
         return set_error(EDDLHIP_EHIP, "graph_end: hipGraphInstantiate: %s", hipGetErrorString(ei));
     }
-    *graph = (void *)exec;
+    *graph = (void *)new RecordedGraph{exec, dev, s.capture_used_workspace, s.workspace_generation};
     return 0;
 }
 
@@ -311,14 +336,22 @@ int eddlhip_graph_launch(int dev, void *graph) {
     EH_REQUIRE(graph != nullptr, "graph_launch: graph is NULL");
     EH_TRY(use_device(dev));
     EH_NOT_CAPTURING(dev, "eddlhip_graph_launch");
-    EH_TRY_HIP(hipGraphLaunch((hipGraphExec_t)graph, state(dev).stream));
+    const RecordedGraph *g = (const RecordedGraph *)graph;
+    EH_REQUIRE(g->dev == dev, "graph_launch: the graph was recorded on device %d, not %d", g->dev, dev);
+    EH_REQUIRE(!g->uses_workspace || g->workspace_generation == state(dev).workspace_generation,
+               "graph_launch: the library's workspace was reallocated since recording (a later call needed a larger one) and the "
+               "graph's kernels still name the old one: record again");
+    EH_TRY_HIP(hipGraphLaunch(g->exec, state(dev).stream));
     return 0;
 }
 
 int eddlhip_graph_destroy(int dev, void *graph) {
     if (!graph) return 0;
     EH_TRY(use_device(dev));
-    EH_TRY_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
+    RecordedGraph *g = (RecordedGraph *)graph;
+    const hipError_t e = hipGraphExecDestroy(g->exec);
+    delete g;
+    EH_TRY_HIP(e);
     return 0;
 }
 

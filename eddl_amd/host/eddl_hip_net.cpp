@@ -593,6 +593,9 @@ void Net::fuse() {
             }
         }
         if (LConv *conv = dynamic_cast<LConv *>(l)) {
+            // the steps call the library directly, past tensorNN::Conv2D and its check (src/tensor/nn/tensor_conv.cpp:48-51)
+            if (conv->cd->dilation_rate[0] != 1 || conv->cd->dilation_rate[1] != 1)
+                msg("Dilated convolutions are only available with CuDNN", "Net::fuse");
             s.chain = true;
             s.src = l->parent[0];
             s.pad_top = conv->cd->padrt;
@@ -685,6 +688,9 @@ void Net::run_step(const FusedStep &s) {
         const Tensor *I = s.src->output;
         Tensor *O = s.last->output;
         const LBatchNorm *bn = s.bn;
+        // the step computes the inference form; the layer walk would raise in gpu_batchnorm_forward
+        if (bn != nullptr && bn->mode == TRMODE)
+            msg("training-mode batch normalisation is outside this forward/inference backend", "Net::forward (fused convolution)");
         const float *bias = D->use_bias ? D->bias->ptr : nullptr;
         const float *g = bn && bn->affine ? bn->bn_g->ptr : nullptr, *b = bn && bn->affine ? bn->bn_b->ptr : nullptr;
         const float *mean = bn ? bn->mean->ptr : nullptr, *var = bn ? bn->variance->ptr : nullptr;

@@ -60,6 +60,9 @@ int eddlhip_memcpy_h2d(int dev, void *dev_dst, const void *host_src, size_t byte
 int eddlhip_memcpy_d2h(int dev, void *host_dst, const void *dev_src, size_t bytes);
 int eddlhip_memcpy_d2d(int dev, void *dev_dst, const void *dev_src, size_t bytes);
 int eddlhip_fill(int dev, float *A, size_t n, float v);
+/* Size of the library's private workspace on the device right now (it only grows; 0 before the first call that
+ * needs one).  No counterpart in the reference. */
+int eddlhip_workspace_bytes(int dev, size_t *bytes);
 
 /* Batch staging.  The reference moves a batch to the device through pageable host tensors and
  * blocking copies (Net::distributeTensor / collectTensor, src/net/net_func.cpp:195-249; a D2H +
@@ -94,6 +97,9 @@ int eddlhip_event_synchronize(int dev, void *event);
  * its final size and registered filters are repacked; calls that wait for the device, copy from or to the
  * host, allocate or free are refused while recording.  A call that fails while recording leaves the
  * recording open: close it with eddlhip_graph_end (which then reports the failure too).
+ * A recorded convolution or dense call that took the library's workspace names it by address; when a later,
+ * larger call has made the library replace that workspace, eddlhip_graph_launch refuses the graph with
+ * EDDLHIP_EINVAL ("record again") instead of letting its kernels write into freed memory.
  * No counterpart in the reference, which synchronises after every kernel. */
 int eddlhip_graph_begin(int dev);
 int eddlhip_graph_end(int dev, void **graph);

@@ -149,6 +149,22 @@ static int errors() {
         Tensor a({2, 3, 8, 8}), b({2, 3, 8, 8});
         predict(m, {&a, &b});
     }, "two inputs for one input layer");
+    ok &= throws([] {  // the fused plan calls the library past tensorNN::Conv2D: it has to refuse dilations itself
+        layer x = Input({3, 12, 12});
+        model m = Model({x}, {ReLu(Conv2D(x, 4, {3, 3}, {1, 1}, "same", true, 1, {2, 2}))});
+        build(m, CS_HIP({1}));
+        fuse(m);
+        Tensor a({2, 3, 12, 12});
+        predict(m, {&a});
+    }, "dilated convolution in a fused plan");
+    ok &= throws([] {  // a batch norm absorbed into a convolution step must not run as inference in training mode
+        model m = block(3, 8, 4);
+        build(m, CS_HIP({1}));
+        fuse(m);
+        set_mode(m, TRMODE);
+        Tensor a({2, 3, 8, 8});
+        forward(m, {&a});
+    }, "training-mode batch norm in a fused plan");
     return ok ? 0 : 1;
 }
 

@@ -208,6 +208,57 @@ def test_captured_plan_replays_bit_for_bit(hip, oracle):
     hip.synchronize()
 
 
+def test_recorded_graph_is_refused_after_the_workspace_was_replaced(hip):
+    """A recorded convolution with unregistered filters names the library's workspace by address.  When a later,
+    larger call has made the library replace that workspace, the replay is refused (not run over freed memory);
+    a new recording works.  A tensor collected while recording is freed once the recording has ended."""
+    from eddl_amd import EddlHipError
+    rng = np.random.default_rng(5)
+    x, w = hip.array(rng.standard_normal((2, 8, 12, 12), dtype=np.float32)), hip.array(rng.standard_normal((16, 8, 3, 3), dtype=np.float32))
+    O = hip.empty((2, 16, 12, 12))
+    box = [hip.empty((1024,))]
+
+    def step():
+        hip.conv2D(x, w, None, O, 1, 1, 1, 1)
+        box.pop() if box else None  # a DeviceTensor collected while recording: its free is refused, then made up for
+
+    hip.conv2D(x, w, None, O, 1, 1, 1, 1)
+    want = O.numpy()
+    g = hip.record(step)
+    assert hip._deferred_free == []
+    hip.fill_(O, 0.0)
+    g.launch()
+    assert np.array_equal(O.numpy(), want)
+    # an eager convolution whose repacked filters need more than the whole workspace of the moment
+    ws = hip.workspace_bytes()
+    C = 64
+    Kf = ((ws + (1 << 20)) // (9 * C * 4) // 128 + 1) * 128
+    big_w, big_x, big_O = hip.full((Kf, C, 3, 3), 0.0), hip.full((1, C, 4, 4), 1.0), hip.empty((1, Kf, 4, 4))
+    hip.conv2D(big_x, big_w, None, big_O, 1, 1, 1, 1)
+    hip.synchronize()
+    assert hip.workspace_bytes() > ws
+    with pytest.raises(EddlHipError, match="record again"):
+        g.launch()
+    g2 = hip.record(lambda: hip.conv2D(x, w, None, O, 1, 1, 1, 1))
+    hip.fill_(O, 0.0)
+    g2.launch()
+    assert np.array_equal(O.numpy(), want)
+    # a graph whose calls do not take the workspace (registered filters, no K split) stays valid
+    hip.cache_conv_filters(w)
+    hip.conv2D(x, w, None, O, 1, 1, 1, 1)
+    g3 = hip.record(lambda: hip.conv2D(x, w, None, O, 1, 1, 1, 1))
+    ws = hip.workspace_bytes()
+    Kf2 = ((ws + (1 << 20)) // (9 * C * 4) // 128 + 1) * 128
+    big_w2, big_O2 = hip.full((Kf2, C, 3, 3), 0.0), hip.empty((1, Kf2, 4, 4))
+    hip.conv2D(big_x, big_w2, None, big_O2, 1, 1, 1, 1)
+    hip.synchronize()
+    assert hip.workspace_bytes() > ws
+    hip.fill_(O, 0.0)
+    g3.launch()
+    assert np.array_equal(O.numpy(), want)
+    hip.uncache_conv_filters(w)
+
+
 def test_bench_line_carries_the_contract_fields(hip):
     """bench.py on the smallest workload: ONE JSON line with the agreed fields, roofline and CPU baseline with its
     end-to-end parity gate; the layer-by-layer and recorded-plan modes run too."""
