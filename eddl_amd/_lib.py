@@ -71,6 +71,13 @@ PROTOTYPES = {
     "eddlhip_add": [c_int, c_float, P, c_float, P, P, c_int, c_size_t],
     "eddlhip_inc": [c_int, P, P, c_size_t],
     "eddlhip_pad": [c_int, P, P] + [c_int] * 8,
+    "eddlhip_rand_uniform": [c_int, P, c_size_t, c_float, ctypes.c_ulonglong],
+    "eddlhip_rand_signed_uniform": [c_int, P, c_size_t, c_float, ctypes.c_ulonglong],
+    "eddlhip_rand_binary": [c_int, P, c_size_t, c_float, ctypes.c_ulonglong],
+    "eddlhip_rand_normal": [c_int, P, c_size_t, c_float, c_float, ctypes.c_ulonglong],
+    "eddlhip_rand_words": [c_int, P, c_size_t, ctypes.c_ulonglong, ctypes.c_ulonglong, ctypes.c_ulonglong],
+    "eddlhip_mult_scalar": [c_int, P, P, c_size_t, c_float],
+    "eddlhip_add_scalar": [c_int, P, P, c_size_t, c_float],
     "eddlhip_mult2d": [c_int, P, P, P, c_int, c_int, c_int, c_int],
     "eddlhip_sum2d_rowwise": [c_int, P, P, P, c_int, c_int],
     "eddlhip_dense_fwd": [c_int, P, P, P, P, c_int, c_int, c_int, c_int],

@@ -268,6 +268,31 @@ class Backend:
     def fill_(self, A, v):
         self._check(self.lib.eddlhip_fill(self.dev, A.ptr, A.size, v))
 
+    # ---- parameter initialisation on the device (gpu_rand_*, gpu_mult / gpu_add with a scalar)
+    def rand_uniform(self, A, v, seed):
+        self._check(self.lib.eddlhip_rand_uniform(self.dev, A.ptr, A.size, v, seed))
+
+    def rand_signed_uniform(self, A, v, seed):
+        self._check(self.lib.eddlhip_rand_signed_uniform(self.dev, A.ptr, A.size, v, seed))
+
+    def rand_binary(self, A, v, seed):
+        self._check(self.lib.eddlhip_rand_binary(self.dev, A.ptr, A.size, v, seed))
+
+    def rand_normal(self, A, mean, stddev, seed):
+        self._check(self.lib.eddlhip_rand_normal(self.dev, A.ptr, A.size, mean, stddev, seed))
+
+    def rand_words(self, n, seed, first_block=0, counter_hi=0):
+        """The generator's raw 32-bit words as a numpy uint32 array (known-answer tests)."""
+        t = self.empty((n,))
+        self._check(self.lib.eddlhip_rand_words(self.dev, t.ptr, n, seed, first_block, counter_hi))
+        return t.numpy().view(np.uint32)
+
+    def mult_scalar(self, A, B, v):
+        self._check(self.lib.eddlhip_mult_scalar(self.dev, A.ptr, B.ptr, A.size, v))
+
+    def add_scalar(self, A, B, v):
+        self._check(self.lib.eddlhip_add_scalar(self.dev, A.ptr, B.ptr, A.size, v))
+
     def conv2D(self, I, K, bias, O, sr, sc, padrt, padcl, bn=None, residual=None, relu=False, second=None, upsample=None):
         """``bn`` = (g, b, mean, var, eps) device tensors (g, b may be None) or None.  ``second``: the other half
         of the input channels as a tensor of its own (a channel Concat of ``I`` and ``second`` folded into the call).

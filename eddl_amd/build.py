@@ -5,7 +5,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["runtime.hip", "elementwise.hip", "pool.hip", "conv.hip", "dense.hip", "probe.hip"]
+SOURCES = ["runtime.hip", "elementwise.hip", "pool.hip", "conv.hip", "dense.hip", "generator.hip", "probe.hip"]
 LIB = os.path.join(HERE, "libeddlhip.so")
 
 HIPCC_FLAGS = [

@@ -309,6 +309,37 @@ int eddlhip_inc(int dev, const float *A, float *B, size_t n);
 int eddlhip_pad(int dev, const float *A, float *B, int N, int C, int H, int W,
                 int top, int right, int bottom, int left);
 
+/* ------------------------------------------------------------------ parameter initialisation on the device
+ * What EDDL's initialisers run on a GPU tensor when eddl::build creates the device copy of a net
+ * (Net::split -> make_graph -> do_initialize, src/net/net_build.cpp:235-237,401; e.g. IGlorotUniform::apply,
+ * src/initializers/initializer_glorot_uniform.cpp:35-60): the four random fills
+ * gpu_rand_uniform / gpu_rand_signed_uniform / gpu_rand_normal / gpu_rand_binary
+ * (include/eddl/hardware/gpu/gpu_hw.h:58-61; distributions as src/hardware/cpu/cpu_generator.cpp:14-49) and the
+ * scalar operations gpu_mult(A, B, v) and gpu_add(A, B, v) (gpu_hw.h:89,106) behind Tensor::mult_ / add_ / sub_.
+ *
+ * Random fills are counter-based (Philox4x32-10): element i of a fill is a function of (seed, i) alone, so a
+ * fill is reproducible whatever the launch shape, and different seeds give independent streams; the caller
+ * picks a new seed per fill (the C++ binding counts fills per device from a fixed base, as the reference's
+ * cuRAND generator is seeded with a constant, src/hardware/gpu/gpu_tensor.cu:179-185).  With u uniform on
+ * [0, 1) in steps of 2^-24:
+ *   eddlhip_rand_uniform         A[i] = u * v
+ *   eddlhip_rand_signed_uniform  A[i] = (2u - 1) * v
+ *   eddlhip_rand_binary          A[i] = u < v ? 1 : 0
+ *   eddlhip_rand_normal          A[i] = z * stddev + mean, z standard normal (Box-Muller)
+ * The reference's own random streams (cuRAND MRG32k3a on the GPU, std::mt19937 seeded from std::random_device
+ * on the CPU) are not reproduced: only the distributions are its contract.
+ * eddlhip_rand_words writes the generator's raw 32-bit words (bit patterns stored in the float slots; block b of
+ * four words is Philox4x32-10 with key = seed and counter = (first_block + b, counter_hi)): for known-answer tests.
+ * eddlhip_mult_scalar: B = A * v;  eddlhip_add_scalar: B = A + v;  A == B is allowed. */
+int eddlhip_rand_uniform(int dev, float *A, size_t n, float v, unsigned long long seed);
+int eddlhip_rand_signed_uniform(int dev, float *A, size_t n, float v, unsigned long long seed);
+int eddlhip_rand_binary(int dev, float *A, size_t n, float v, unsigned long long seed);
+int eddlhip_rand_normal(int dev, float *A, size_t n, float mean, float stddev, unsigned long long seed);
+int eddlhip_rand_words(int dev, float *A, size_t n, unsigned long long seed, unsigned long long first_block,
+                       unsigned long long counter_hi);
+int eddlhip_mult_scalar(int dev, const float *A, float *B, size_t n, float v);
+int eddlhip_add_scalar(int dev, const float *A, float *B, size_t n, float v);
+
 /* ------------------------------------------------------------------ dense
  * eddlhip_mult2d replaces gpu_mult2D(A, tA, B, tB, C, incC) for the forward case
  * tA = tB = 0 used by LDense::forward (src/layers/core/layer_dense.cpp:65-73,
