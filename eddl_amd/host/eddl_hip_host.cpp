@@ -22,78 +22,15 @@ void msg(const string &text, const string &title) {
     throw std::runtime_error("RuntimeError: " + title);
 }
 
-// A failed C ABI call becomes the reference's device-error exception
-// (check_cuda throws std::runtime_error("[CUDA ERROR]: ..."), src/hardware/gpu/gpu_tensor.cu:103-112);
-// a rejected argument becomes a msg().
-void gpu_check(int rc, const char *where) {
-    if (rc == 0) return;
-    string text = eddlhip_last_error();
-    if (rc == EDDLHIP_EINVAL) msg(text, where);
-    throw std::runtime_error(string("[HIP ERROR]: ") + text + " (" + where + ")");
-}
-
-static void check(int rc, const char *where) { gpu_check(rc, where); }
-
-static bool g_synchronous = true;
-
-void gpu_set_synchronous(bool on) { g_synchronous = on; }
-bool gpu_get_synchronous() { return g_synchronous; }
-void gpu_synchronize(int gpu_device) { check(eddlhip_synchronize(gpu_device), "gpu_synchronize"); }
-
-static void sync(int gpu_device) {
-    if (g_synchronous) gpu_synchronize(gpu_device);
-}
-
-// ---------------------------------------------------------------- runtime
-static bool g_init[16] = {false};
-
-void gpu_init(int device) {
-    int n = gpu_devices();
-    if (device < 0 || device >= n) {
-        std::cerr << "[HIP ERROR]: GPU " << device << " not available. Number of available GPUs is " << n
-                  << ". Further information running rocm-smi\n";
-        throw std::runtime_error("[HIP ERROR]: device not available (gpu_init)");
-    }
-    check(eddlhip_init(device), "gpu_init");
-    if (!g_init[device]) {
-        char name[256];
-        check(eddlhip_device_name(device, name, sizeof(name)), "gpu_init");
-        std::cerr << "EDDL is running on GPU device " << device << ", " << name << "\n";
-        g_init[device] = true;
-    }
-}
-
-void gpu_set_device(int device) { check(eddlhip_init(device), "gpu_set_device"); }
-
-int gpu_devices() {
-    int n = 0;
-    check(eddlhip_device_count(&n), "gpu_devices");
-    return n;
-}
-
-float *gpu_create_tensor(int dev, int size) {
-    void *p = nullptr;
-    check(eddlhip_malloc(dev, (size_t)size * sizeof(float), &p), "gpu_create_tensor");
-    return (float *)p;
-}
-
-void gpu_delete_tensor(int dev, float *p) { check(eddlhip_free(dev, p), "gpu_delete_tensor"); }
-
-void gpu_copy_to_gpu(float *nptr, Tensor *B) { check(eddlhip_memcpy_h2d(B->gpu_device, B->ptr, nptr, B->size * sizeof(float)), "gpu_copy_to_gpu"); }
-
-void gpu_copy_from_gpu(Tensor *A, float *nptr) { check(eddlhip_memcpy_d2h(A->gpu_device, nptr, A->ptr, A->size * sizeof(float)), "gpu_copy_from_gpu"); }
-
-void gpu_copy_gpu(Tensor *A, Tensor *B) {
-    check(eddlhip_memcpy_d2d(B->gpu_device, B->ptr, A->ptr, A->size * sizeof(float)), "gpu_copy_gpu");
-    sync(B->gpu_device);
-}
-
-void gpu_fill_(Tensor *A, float v) {
-    check(eddlhip_fill(A->gpu_device, A->ptr, A->size, v), "gpu_fill_");
-    sync(A->gpu_device);
-}
+// gpu_check, the wait after every call and every gpu_* function are defined in the binding translation unit,
+// integration/eddl/src/hardware/hip/hip_backend.cpp, which the Makefile compiles into this library against the
+// classes below (EDDLHIP_MIRROR_BUILD).
 
 // ---------------------------------------------------------------- Tensor
+static void need_gpu(const Tensor *t, const char *where) {
+    if (!t->isGPU()) msg("this backend only runs tensors that live on a GPU device", where);
+}
+
 void Tensor::updateStrides() {
     stride.assign(ndim, 1);
     for (int i = (int)ndim - 2; i >= 0; i--) stride[i] = stride[i + 1] * shape[i + 1];
@@ -188,6 +125,33 @@ void Tensor::fill_(float v) {
     }
 }
 
+// Random fills and scalar arithmetic as the reference's initialisers use them on a device tensor
+// (src/tensor/tensor_generator.cpp:25-110, src/tensor/tensor_math.cpp:1455-1470)
+void Tensor::fill_rand_uniform_(float v) {
+    need_gpu(this, "Tensor::fill_rand_uniform_");
+    gpu_rand_uniform(this, v);
+}
+void Tensor::fill_rand_signed_uniform_(float v) {
+    need_gpu(this, "Tensor::fill_rand_signed_uniform_");
+    gpu_rand_signed_uniform(this, v);
+}
+void Tensor::fill_rand_normal_(float m, float s) {
+    need_gpu(this, "Tensor::fill_rand_normal_");
+    gpu_rand_normal(this, m, s);
+}
+void Tensor::fill_rand_binary_(float v) {
+    need_gpu(this, "Tensor::fill_rand_binary_");
+    gpu_rand_binary(this, v);
+}
+void Tensor::mult_(float v) {
+    need_gpu(this, "Tensor::mult_");
+    gpu_mult(this, this, v);
+}
+void Tensor::add_(float v) {
+    need_gpu(this, "Tensor::add_");
+    gpu_add(this, this, v);
+}
+
 void Tensor::resize(int b) {
     if (b == shape[0]) return;
     release();
@@ -221,10 +185,6 @@ void Tensor::copy(Tensor *A, Tensor *B) {
     else if (A->isCPU() && B->isGPU()) gpu_copy_to_gpu(A->ptr, B);
     else if (A->isGPU() && B->isCPU()) gpu_copy_from_gpu(A, B->ptr);
     else gpu_copy_gpu(A, B);
-}
-
-static void need_gpu(const Tensor *t, const char *where) {
-    if (!t->isGPU()) msg("this backend only runs tensors that live on a GPU device", where);
 }
 
 void Tensor::add(float scA, Tensor *A, float scB, Tensor *B, Tensor *C, int incC) {
@@ -296,7 +256,11 @@ void Tensor::sum2D_rowwise(Tensor *A, Tensor *B, Tensor *C) {
     gpu_sum2D_rowwise(A, B, C);
 }
 
-// ---------------------------------------------------------------- geometry (float arithmetic as in the reference)
+// ---------------------------------------------------------------- window geometry, shared by both descriptors
+// One routine holds the rules (float arithmetic as in the reference, src/descriptors/descriptor_conv2D.cpp:295-360,
+// descriptor_pool2D.cpp:162-211): named paddings give out = ceil(in / stride) ("same", "zeros") or
+// ceil((in - (k - 1) dilation) / stride) ("valid", "none") and the pads that go with it (total split low = pad / 2,
+// high = the rest); "custom" takes the pads as given and out = int((in - (k - 1) dilation + lo + hi - 1) / stride + 1).
 static int out_named(const string &padding, int input_size, int kernel_size, int stride, int dilation_rate, const char *where) {
     if (padding == "same" || padding == "zeros") return (int)std::ceil((float)input_size / (float)stride);
     if (padding == "valid" || padding == "none")
@@ -325,30 +289,57 @@ static vector<int> pads_named(int output_size, int input_size, int kernel_size, 
     return {-1};
 }
 
+struct WindowGeometry {
+    int r, c;          // output rows, columns
+    vector<int> pads;  // {rows-top, rows-bottom, cols-left, cols-right}
+};
+
+// custom_cols_read_row_pads: PoolDescriptor::build hands the whole 4-vector to compute_output for both axes, which
+// reads entries [0] and [1] (src/descriptors/descriptor_pool2D.cpp:78-79); ConvolDescriptor::build hands {pads[2], pads[3]}.
+static WindowGeometry window_geometry(const char *who, const Tensor *A, const string &padding, const vector<int> &pads, int kr, int kc,
+                                      int sr, int sc, int dil_r, int dil_c, bool custom_cols_read_row_pads) {
+    const string where = string(who) + "::build";
+    if (A->ndim != 4) msg("Tensors are not 4D", where);
+    const int ir = A->shape[2], ic = A->shape[3];
+    WindowGeometry g;
+    if (padding == "custom") {
+        g.pads = pads;
+        g.r = out_custom({pads[0], pads[1]}, ir, kr, sr, dil_r);
+        g.c = custom_cols_read_row_pads ? out_custom({pads[0], pads[1]}, ic, kc, sc, dil_c) : out_custom({pads[2], pads[3]}, ic, kc, sc, dil_c);
+    } else {
+        const string pr = padding == "same,none" ? "same" : padding == "none,same" ? "none" : padding;
+        const string pc = padding == "same,none" ? "none" : padding == "none,same" ? "same" : padding;
+        const string wo = string(who) + "::compute_output", wp = string(who) + "::compute_padding";
+        g.r = out_named(pr, ir, kr, sr, dil_r, wo.c_str());
+        g.c = out_named(pc, ic, kc, sc, dil_c, wo.c_str());
+        const vector<int> padr = pads_named(g.r, ir, kr, sr, padding, true, dil_r, wp.c_str());
+        const vector<int> padc = pads_named(g.c, ic, kc, sc, padding, false, dil_c, wp.c_str());
+        g.pads = {padr[0], padr[1], padc[0], padc[1]};
+    }
+    if (g.r <= 0 || g.c <= 0) {
+        if (g.r <= 0) std::cerr << "'Rows' are reach 0 or less (" << g.r << ")" << std::endl;
+        if (g.c <= 0) std::cerr << "'Columns' are reach 0 or less (" << g.c << ")" << std::endl;
+        msg("Invalid output shape", where);
+    }
+    return g;
+}
+
 // ---------------------------------------------------------------- ConvolDescriptor
 ConvolDescriptor::ConvolDescriptor(int filters, const vector<int> &kernel_size, const vector<int> &strides, string padding,
-                                   const vector<int> &pads, int groups, const vector<int> &dilation_rate, bool use_bias, int mem) {
+                                   const vector<int> &pads, int groups, const vector<int> &dilation_rate, bool use_bias, int mem)
+    : ksize(kernel_size), stride(strides), pads(pads), filters(filters), kernel_size(kernel_size), strides(strides), padding(padding),
+      groups(groups), dilation_rate(dilation_rate), use_bias(use_bias), mem_level(mem) {
     const char *where = "ConvolDescriptor::ConvolDescriptor";
     if (groups > 1) msg("Grouped convolutions are only available with CuDNN", where);
     if (kernel_size.size() != 2) msg("Kernels must have 3 dimensions", where);
     if (strides.size() != 2) msg("Strides must have 2 dimensions", where);
     if (dilation_rate.size() != 2) msg("Dilations must have 2 elements", where);
     if (groups < 1) msg("The number of groups should be greater or equal to 1", where);
-    this->filters = filters;
-    this->kernel_size = kernel_size;
-    this->strides = strides;
-    this->padding = padding;
-    this->pads = vector<int>(pads);
-    this->groups = groups;
-    this->dilation_rate = dilation_rate;
-    this->use_bias = use_bias;
-    this->mem_level = mem;
-    ksize = vector<int>(kernel_size);
     ksize.insert(ksize.begin(), 1, filters);
-    stride = vector<int>(strides);
-    if (!(padding == "custom" || padding == "same" || padding == "none" || padding == "valid" || padding == "zeros" ||
-          padding == "same,none" || padding == "none,same"))
-        msg("Incorrect padding type (" + padding + ")", where);
+    static const char *const known[] = {"custom", "same", "none", "valid", "zeros", "same,none", "none,same"};
+    bool ok = false;
+    for (const char *k : known) ok = ok || padding == k;
+    if (!ok) msg("Incorrect padding type (" + padding + ")", where);
     if (filters % groups) msg("The number of filters must be divisible by the number groups.", where);
 }
 
@@ -368,42 +359,16 @@ vector<int> ConvolDescriptor::compute_padding(int output_size, int input_size, i
 }
 
 void ConvolDescriptor::build(Tensor *A) {
-    if (A->ndim != 4) msg("Tensors are not 4D", "ConvolDescriptor::build");
-    I = A;
-    nk = ksize[0];
-    kr = ksize[1];
-    kc = ksize[2];
+    const WindowGeometry g = window_geometry("ConvolDescriptor", A, padding, pads, ksize[1], ksize[2], stride[0], stride[1],
+                                             dilation_rate[0], dilation_rate[1], false);
     if (A->shape[1] % groups) msg("The number of input channels must be divisible by the number groups.", "ConvolDescriptor::build");
-    kz = A->shape[1] / groups;
-    sr = stride[0];
-    sc = stride[1];
-    in = A->shape[0];
-    iz = A->shape[1];
-    ir = A->shape[2];
-    ic = A->shape[3];
-    z = nk;
-    if (padding == "custom") {
-        r = compute_output(vector<int>{pads[0], pads[1]}, ir, kr, sr, dilation_rate[0]);
-        c = compute_output(vector<int>{pads[2], pads[3]}, ic, kc, sc, dilation_rate[1]);
-    } else {
-        const string pr = padding == "same,none" ? "same" : padding == "none,same" ? "none" : padding;
-        const string pc = padding == "same,none" ? "none" : padding == "none,same" ? "same" : padding;
-        r = compute_output(pr, ir, kr, sr, dilation_rate[0]);
-        c = compute_output(pc, ic, kc, sc, dilation_rate[1]);
-        vector<int> padr = compute_padding(r, ir, kr, sr, padding, true, dilation_rate[0]);
-        vector<int> padc = compute_padding(c, ic, kc, sc, padding, false, dilation_rate[1]);
-        pads = {padr[0], padr[1], padc[0], padc[1]};
-    }
-    padrt = pads[0];
-    padrb = pads[1];
-    padcl = pads[2];
-    padcr = pads[3];
-    if (r <= 0 || c <= 0) {
-        if (r <= 0) std::cerr << "'Rows' are reach 0 or less (" << r << ")" << std::endl;
-        if (c <= 0) std::cerr << "'Columns' are reach 0 or less (" << c << ")" << std::endl;
-        msg("Invalid output shape", "ConvolDescriptor::build");
-    }
-    O = new Tensor(vector<int>{A->shape[0], z, r, c}, A->device);
+    I = A;
+    nk = z = ksize[0], kr = ksize[1], kc = ksize[2], kz = A->shape[1] / groups;
+    sr = stride[0], sc = stride[1];
+    in = A->shape[0], iz = A->shape[1], ir = A->shape[2], ic = A->shape[3];
+    r = g.r, c = g.c, pads = g.pads;
+    padrt = pads[0], padrb = pads[1], padcl = pads[2], padcr = pads[3];
+    O = new Tensor(vector<int>{in, z, r, c}, A->device);
     K = new Tensor(vector<int>{nk, kz, kr, kc}, A->device);
     bias = new Tensor(vector<int>{nk}, A->device);
     // no lowering buffer: the convolution is an implicit GEMM
@@ -416,24 +381,17 @@ void ConvolDescriptor::resize(int b) {
 }
 
 // ---------------------------------------------------------------- PoolDescriptor
-PoolDescriptor::PoolDescriptor(const vector<int> &ks, const vector<int> &st, const vector<int> &p, int mem) {
-    ksize = ks;
-    stride = st;
-    pad = p;
-    mem_level = mem;
-    padding = "custom";
+PoolDescriptor::PoolDescriptor(const vector<int> &ks, const vector<int> &st, const vector<int> &p, int mem)
+    : ksize(ks), stride(st), pad(p), padding("custom"), mem_level(mem) {
     if (ksize.size() != 2) msg("Pooling Kernels must have 2 dimensions", "PoolDescriptor::PoolDescriptor");
     if (stride.size() != 2) msg("Strides must have 2 dimensions", "PoolDescriptor::PoolDescriptor");
 }
 
-PoolDescriptor::PoolDescriptor(const vector<int> &ks, const vector<int> &st, const string &p, int mem) {
+PoolDescriptor::PoolDescriptor(const vector<int> &ks, const vector<int> &st, const string &p, int mem)
+    : ksize(ks), stride(st), padding(p), mem_level(mem) {
     if (ks.size() != 2) msg("Pooling Kernels must have 2 dimensions", "PoolDescriptor::PoolDescriptor");
     if (st.size() != 2) msg("Strides must have 2 dimensions", "PoolDescriptor::PoolDescriptor");
-    ksize = ks;
-    stride = st;
-    mem_level = mem;
-    if (p == "same" || p == "none" || p == "valid" || p == "zeros") padding = p;
-    else msg("Incorrect padding type", "PoolDescriptor::PoolDescriptor");
+    if (!(p == "same" || p == "none" || p == "valid" || p == "zeros")) msg("Incorrect padding type", "PoolDescriptor::PoolDescriptor");
 }
 
 PoolDescriptor::~PoolDescriptor() {
@@ -452,164 +410,23 @@ vector<int> PoolDescriptor::compute_padding(int output_size, int input_size, int
 }
 
 void PoolDescriptor::build(Tensor *A) {
-    if (A->ndim != 4) msg("Tensors are not 4D", "PoolDescriptor::build");
+    const WindowGeometry g = window_geometry("PoolDescriptor", A, padding, pad, ksize[0], ksize[1], stride[0], stride[1], 1, 1, true);
     I = A;
-    kr = ksize[0];
-    kc = ksize[1];
-    sr = stride[0];
-    sc = stride[1];
-    in = A->shape[0];
-    iz = A->shape[1];
-    ir = A->shape[2];
-    ic = A->shape[3];
-    z = iz;
-    if (padding == "custom") {
-        // as the reference: the whole 4-vector is handed over and entries [0], [1] are read for both axes
-        r = compute_output(pad, ir, kr, sr);
-        c = compute_output(pad, ic, kc, sc);
-    } else {
-        r = compute_output(padding, ir, kr, sr);
-        c = compute_output(padding, ic, kc, sc);
-        vector<int> padr = compute_padding(r, ir, kr, sr, padding, true);
-        vector<int> padc = compute_padding(c, ic, kc, sc, padding, false);
-        pad = {padr[0], padr[1], padc[0], padc[1]};
-    }
-    padrt = pad[0];
-    padrb = pad[1];
-    padcl = pad[2];
-    padcr = pad[3];
-    if (r <= 0 || c <= 0) {
-        if (r <= 0) std::cerr << "'Rows' are reach 0 or less (" << r << ")" << std::endl;
-        if (c <= 0) std::cerr << "'Columns' are reach 0 or less (" << c << ")" << std::endl;
-        msg("Invalid output shape", "PoolDescriptor::build");
-    }
-    O = new Tensor(vector<int>{A->shape[0], z, r, c}, A->device);
-    size = 0;
-    for (int k = 0; k < iz; k++)
-        for (int i = -padrt; i <= ir + padrb - kr; i += sr)
-            for (int j = -padcl; j <= ic + padcr - kc; j += sc, size++) {
-            }
+    kr = ksize[0], kc = ksize[1], sr = stride[0], sc = stride[1];
+    in = A->shape[0], iz = z = A->shape[1], ir = A->shape[2], ic = A->shape[3];
+    r = g.r, c = g.c, pad = g.pads;
+    padrt = pad[0], padrb = pad[1], padcl = pad[2], padcr = pad[3];
+    O = new Tensor(vector<int>{in, z, r, c}, A->device);
+    // outputs the window walk writes per image (the reference counts them by replaying its loop nest)
+    const int rows = ir + padrb - kr >= -padrt ? (ir + padrb - kr + padrt) / sr + 1 : 0;
+    const int cols = ic + padcr - kc >= -padcl ? (ic + padcr - kc + padcl) / sc + 1 : 0;
+    size = iz * rows * cols;
 }
 
 void PoolDescriptor::resize(int b) {
     if (b == O->shape[0]) return;
     O->resize(b);
     in = b;
-}
-
-// ---------------------------------------------------------------- operators
-void gpu_conv2D(ConvolDescriptor *D) {
-    const int dev = D->I->gpu_device;
-    check(eddlhip_conv2d_fwd(dev, D->I->ptr, D->K->ptr, D->use_bias ? D->bias->ptr : nullptr, D->O->ptr, D->I->shape[0], D->iz, D->ir,
-                             D->ic, D->nk, D->kr, D->kc, D->sr, D->sc, D->padrt, D->padcl, D->r, D->c, nullptr, nullptr, nullptr, nullptr,
-                             0.0f, nullptr, 0),
-          "gpu_conv2D");
-    sync(dev);
-}
-
-void gpu_mpool2D(PoolDescriptor *D) {
-    const int dev = D->I->gpu_device;
-    int lp = 0, lq = 0;
-    check(eddlhip_pool2d_out_dims(D->ir, D->ic, D->kr, D->kc, D->sr, D->sc, D->padrt, D->padrb, D->padcl, D->padcr, &lp, &lq), "gpu_mpool2D");
-    if ((unsigned long)D->I->shape[0] * D->iz * lp * lq > D->O->size) msg("the window walk writes more outputs than the output tensor holds", "gpu_mpool2D");
-    check(eddlhip_maxpool2d(dev, D->I->ptr, D->O->ptr, D->indX->ptr, D->indY->ptr, D->I->shape[0], D->iz, D->ir, D->ic, D->kr, D->kc, D->sr,
-                            D->sc, D->padrt, D->padrb, D->padcl, D->padcr),
-          "gpu_mpool2D");
-    sync(dev);
-}
-
-void gpu_avgpool2D(PoolDescriptor *D) {
-    const int dev = D->I->gpu_device;
-    int lp = 0, lq = 0;
-    check(eddlhip_pool2d_out_dims(D->ir, D->ic, D->kr, D->kc, D->sr, D->sc, D->padrt, D->padrb, D->padcl, D->padcr, &lp, &lq), "gpu_avgpool2D");
-    if ((unsigned long)D->I->shape[0] * D->iz * lp * lq > D->O->size) msg("the window walk writes more outputs than the output tensor holds", "gpu_avgpool2D");
-    check(eddlhip_avgpool2d(dev, D->I->ptr, D->O->ptr, D->I->shape[0], D->iz, D->ir, D->ic, D->kr, D->kc, D->sr, D->sc, D->padrt, D->padrb,
-                            D->padcl, D->padcr),
-          "gpu_avgpool2D");
-    sync(dev);
-}
-
-void gpu_batchnorm_forward(int gpu_device, int b, int z, int rc, float *input, float *output, float *opa, float *global_mean,
-                           float *global_variance, float *affine_g, float *affine_b, float *mean, float *variance, bool trmode,
-                           float epsilon, float momentum) {
-    (void)mean;
-    (void)momentum;
-    if (trmode) msg("training-mode batch normalisation is outside this forward/inference backend", "gpu_batchnorm_forward");
-    check(eddlhip_batchnorm_inference(gpu_device, b, z, rc, input, output, opa, global_mean, global_variance, affine_g, affine_b, variance,
-                                      epsilon),
-          "gpu_batchnorm_forward");
-    sync(gpu_device);
-}
-
-void gpu_relu(Tensor *A, Tensor *B) {
-    check(eddlhip_relu(A->gpu_device, A->ptr, B->ptr, A->size), "gpu_relu");
-    sync(A->gpu_device);
-}
-
-void gpu_sigmoid(Tensor *A, Tensor *B) {
-    check(eddlhip_sigmoid(A->gpu_device, A->ptr, B->ptr, A->size), "gpu_sigmoid");
-    sync(A->gpu_device);
-}
-
-void gpu_full_softmax(Tensor *A, Tensor *B, int axis, bool stable) {
-    int outer = 1, inner = 1;
-    for (int i = 0; i < axis; i++) outer *= A->shape[i];
-    for (unsigned i = axis + 1; i < A->ndim; i++) inner *= A->shape[i];
-    check(eddlhip_softmax(A->gpu_device, A->ptr, B->ptr, outer, A->shape[axis], inner, stable ? 1 : 0), "gpu_full_softmax");
-    sync(A->gpu_device);
-}
-
-void gpu_scale(Tensor *A, Tensor *B, vector<int> new_shape, int wrapping_mode, float constant, int transformation_mode) {
-    (void)constant;
-    // UpSampling2D asks for nearest wrapping (2) and asymmetric coordinates (3): include/eddl/utils.h:119-122
-    if (wrapping_mode != 2 || transformation_mode != 3)
-        msg("only nearest wrapping with asymmetric coordinates is implemented on this backend", "gpu_scale");
-    check(eddlhip_scale_nearest(A->gpu_device, A->ptr, B->ptr, A->shape[0], A->shape[1], A->shape[2], A->shape[3], B->shape[2], B->shape[3],
-                                new_shape[0], new_shape[1]),
-          "gpu_scale");
-    sync(A->gpu_device);
-}
-
-void gpu_concat(Tensor *A, vector<Tensor *> t, unsigned int axis, bool derivative) {
-    if (derivative) msg("the backward of concat is outside this forward/inference backend", "gpu_concat");
-    vector<const float *> srcs;
-    vector<int> ext;
-    for (Tensor *x : t) {
-        srcs.push_back(x->ptr);
-        ext.push_back(x->shape[axis]);
-    }
-    int outer = 1;
-    for (unsigned i = 0; i < axis; i++) outer *= A->shape[i];
-    check(eddlhip_concat(A->gpu_device, A->ptr, srcs.data(), ext.data(), (int)t.size(), outer, A->stride[axis]), "gpu_concat");
-    sync(A->gpu_device);
-}
-
-void gpu_add(float scA, Tensor *A, float scB, Tensor *B, Tensor *C, int incC) {
-    check(eddlhip_add(A->gpu_device, scA, A->ptr, scB, B->ptr, C->ptr, incC, A->size), "gpu_add");
-    sync(A->gpu_device);
-}
-
-void gpu_inc(Tensor *A, Tensor *B) {
-    check(eddlhip_inc(A->gpu_device, A->ptr, B->ptr, A->size), "gpu_inc");
-    sync(A->gpu_device);
-}
-
-void gpu_pad(Tensor *A, Tensor *B, vector<int> pads) {
-    check(eddlhip_pad(A->gpu_device, A->ptr, B->ptr, A->shape[0], A->shape[1], A->shape[2], A->shape[3], pads[0], pads[1], pads[2], pads[3]),
-          "gpu_pad");
-    sync(A->gpu_device);
-}
-
-void gpu_mult2D(Tensor *A, int tA, Tensor *B, int tB, Tensor *C, int incC) {
-    if (tA || tB) msg("transposed operands belong to the backward pass, which is outside this backend", "gpu_mult2D");
-    if (A->shape[1] != B->shape[0] || C->shape[0] != A->shape[0] || C->shape[1] != B->shape[1]) msg("Incompatible dims", "gpu_mult2D");
-    check(eddlhip_mult2d(A->gpu_device, A->ptr, B->ptr, C->ptr, A->shape[0], A->shape[1], B->shape[1], incC), "gpu_mult2D");
-    sync(A->gpu_device);
-}
-
-void gpu_sum2D_rowwise(Tensor *A, Tensor *B, Tensor *C) {
-    check(eddlhip_sum2d_rowwise(A->gpu_device, A->ptr, B->ptr, C->ptr, A->shape[0], A->shape[1]), "gpu_sum2D_rowwise");
-    sync(A->gpu_device);
 }
 
 // ---------------------------------------------------------------- dispatchers

@@ -56,6 +56,13 @@ class Tensor {
     void toGPU(int dev = DEV_GPU);
     void toCPU();
     void fill_(float v);
+    // device-side initialisation (GPU tensors): src/tensor/tensor_generator.cpp:25-110, tensor_math.cpp:1455-1470
+    void fill_rand_uniform_(float v);
+    void fill_rand_signed_uniform_(float v);
+    void fill_rand_normal_(float m, float s);
+    void fill_rand_binary_(float v);
+    void mult_(float v);
+    void add_(float v);
     void resize(int b);                         // new batch size; storage is re-created
     void reshape_(const vector<int> &new_shape);  // same storage
     static Tensor *zeros(const vector<int> &shape, int dev = DEV_CPU);
@@ -128,12 +135,25 @@ class PoolDescriptor {
                                        bool row = false);
 };
 
-// ---- the backend seam: same signatures as the reference's gpu_* declarations
+// ---- the backend seam: same signatures as the reference's gpu_* declarations.  They are defined, for this
+// library and for EDDL itself, by one translation unit: integration/eddl/src/hardware/hip/hip_backend.cpp.
 void gpu_init(int device);
 void gpu_set_synchronous(bool on);      // no counterpart in the reference: see the note at the top
 bool gpu_get_synchronous();
 void gpu_synchronize(int gpu_device);   // waits for everything queued on the device
 void gpu_check(int rc, const char *where);  // a C ABI return code -> the reference's exceptions
+void gpu_set_random_seed(unsigned long long base);  // base seed of the device-side random fills (default 1234)
+void gpu_delete_tensor_int(int dev, int *p);
+void cpu2gpu(float *dst, const float *src, unsigned long int size, int gpu_device);
+void gpu2cpu(float *dst, const float *src, unsigned long int size, int gpu_device);
+float *get_gpu_fmem(unsigned long int size, int gpu_device);
+void free_gpu_ptr(float *ptr, int gpu_device);
+void gpu_rand_uniform(Tensor *A, float v);
+void gpu_rand_signed_uniform(Tensor *A, float v);
+void gpu_rand_binary(Tensor *A, float v);
+void gpu_rand_normal(Tensor *A, float m, float s);
+void gpu_mult(Tensor *A, Tensor *B, float v);
+void gpu_add(Tensor *A, Tensor *B, float v);
 void gpu_set_device(int device);
 int gpu_devices();
 float *gpu_create_tensor(int dev, int size);

@@ -51,29 +51,26 @@ void Layer::toGPU(int device) {
     for (Tensor *t : fixed) t->toGPU(device);
 }
 
-// Parameter initialisation of build(init_weights = true): Glorot-uniform filters and weights, zero
-// biases (the reference's defaults, src/layers/conv/layer_conv2D.cpp:109-112 and
-// src/initializers/initializer_glorot.cpp), drawn from a generator of this file's own.
+// Parameter initialisation of build(init_weights = true): Glorot-uniform filters and weights, zero biases (the
+// reference's defaults: LConv::initialize, src/layers/conv/layer_conv2D.cpp:109-112, with IGlorotUniform::apply,
+// src/initializers/initializer_glorot_uniform.cpp:35-60).  It runs on the DEVICE tensors, through the same calls the
+// reference's initialiser makes on the device copy of a net (Net::split -> make_graph -> do_initialize,
+// src/net/net_build.cpp:235-237,401): fill_rand_signed_uniform_(1.0) then mult_(limit).
 namespace {
-struct Rng {
-    uint64_t s;
-    explicit Rng(uint64_t seed) : s(seed * 0x9E3779B97F4A7C15ull + 0x632BE59BD9B4E019ull) {}
-    float uniform() {  // [0, 1)
-        s ^= s << 13;
-        s ^= s >> 7;
-        s ^= s << 17;
-        return (float)((s >> 40) * (1.0 / 16777216.0));
+void glorot_uniform(Tensor *params) {
+    int fin, fout;
+    if (params->ndim == 4) {  // (output_depth, input_depth, kr, kc)
+        const int rf = params->shape[2] * params->shape[3];
+        fin = rf * params->shape[1];
+        fout = rf * params->shape[0];
+    } else if (params->ndim == 2) {
+        fin = params->shape[0];
+        fout = params->shape[1];
+    } else {
+        fin = fout = params->shape[0];
     }
-};
-
-void glorot_uniform(Tensor *t, int fan_in, int fan_out, unsigned seed) {
-    const bool on_gpu = t->isGPU();
-    const int device = t->device;
-    if (on_gpu) t->toCPU();
-    Rng rng(seed);
-    const float limit = std::sqrt(6.0f / (float)(fan_in + fan_out));
-    for (unsigned long i = 0; i < t->size; i++) t->ptr[i] = (2.0f * rng.uniform() - 1.0f) * limit;
-    if (on_gpu) t->toGPU(device);
+    params->fill_rand_signed_uniform_(1.0f);
+    params->mult_(std::sqrt(6.0f / (float)(fin + fout)));
 }
 }  // namespace
 
@@ -117,8 +114,8 @@ void LConv::resize(int batch) {
     cd->resize(batch);
 }
 
-void LConv::initialize(unsigned seed) {
-    glorot_uniform(cd->K, cd->kz * cd->kr * cd->kc, cd->nk * cd->kr * cd->kc, seed);
+void LConv::initialize() {
+    glorot_uniform(cd->K);
     cd->bias->fill_(0.0f);
 }
 
@@ -155,7 +152,7 @@ void LBatchNorm::forward() {
                                mode == TRMODE, epsilon, momentum);
 }
 
-void LBatchNorm::initialize(unsigned) {
+void LBatchNorm::initialize() {
     if (affine) {
         bn_g->fill_(1.0f);
         bn_b->fill_(0.0f);
@@ -430,8 +427,8 @@ void LDense::forward() {
     output->reshape_(outshape);
 }
 
-void LDense::initialize(unsigned seed) {
-    glorot_uniform(W, W->shape[0], W->shape[1], seed);
+void LDense::initialize() {
+    glorot_uniform(W);
     if (use_bias) bias->fill_(0.0f);
 }
 
@@ -504,12 +501,11 @@ void Net::build(CompServ *service, bool init_weights) {
     if (count > 1) msg("this backend runs a net on one GPU; the computing service names " + std::to_string(count), "Net::build");
     if (device >= gpu_devices()) msg("GPU " + std::to_string(device) + " is not present", "Net::build");
     gpu_init(device);
-    if (init_weights) {
-        unsigned seed = 1;
-        for (Layer *l : layers) l->initialize(seed++);
-    }
     dev = DEV_GPU + device;
     for (Layer *l : layers) l->toGPU(dev);
+    // the parameters are drawn on the device, as the reference draws those of the device copy of a net
+    if (init_weights)
+        for (Layer *l : layers) l->initialize();
 }
 
 void Net::resize(int batch) {

@@ -51,7 +51,7 @@ class Layer {
     virtual void forward() = 0;
     virtual void resize(int batch);      // default: the output follows the batch
     virtual void toGPU(int device);      // default: output and parameters move
-    virtual void initialize(unsigned) {}  // parameters at build(init_weights = true)
+    virtual void initialize() {}  // parameters at build(init_weights = true), drawn on the device
     virtual string kind() const = 0;
     vector<int> getShape() const { return output->getShape(); }
     void addchild(Layer *l);
@@ -87,7 +87,7 @@ class LConv : public Layer {
     ~LConv() override;
     void forward() override;
     void resize(int batch) override;
-    void initialize(unsigned seed) override;
+    void initialize() override;
     string kind() const override { return "conv2d"; }
 };
 
@@ -98,7 +98,7 @@ class LBatchNorm : public Layer {
     Tensor *mean, *variance, *bn_mean, *bn_var, *bn_g = nullptr, *bn_b = nullptr, *opa;
     LBatchNorm(Layer *parent, float momentum, float epsilon, bool affine, string name);
     void forward() override;
-    void initialize(unsigned seed) override;
+    void initialize() override;
     string kind() const override { return "batchnorm"; }
 };
 
@@ -199,7 +199,7 @@ class LDense : public Layer {
     Tensor *W, *bias = nullptr;
     LDense(Layer *parent, int ndim, bool use_bias, string name);
     void forward() override;
-    void initialize(unsigned seed) override;
+    void initialize() override;
     string kind() const override { return "dense"; }
 };
 

@@ -10,34 +10,45 @@ from . import net as L
 
 # ---------------------------------------------------------------------------- synthetic parameters
 def init_he_normal(model, seed, bn_stats=True):
-    """Fill every parameter of ``model`` from one seeded generator, layer by layer in graph order,
-    tensor by tensor in the layer's parameter order, row-major:
+    """Fill every parameter of ``model`` from one seeded stream (:class:`eddl_amd.synth.Synth`: mt19937 + Box-Muller,
+    the generator the C++ host shares), layer by layer in graph order, tensor by tensor in the layer's parameter order,
+    row-major:
       conv filters  N(0, sqrt(2 / (C*R*S))), conv bias 0
       dense weights N(0, sqrt(2 / in)), dense bias 0
       batch-norm    gamma U(0.8, 1.2), beta N(0, 0.1), running mean N(0, 0.1), running variance U(0.5, 1.5)
+    ``eddl_hip::synth_he_normal`` (C++) makes the same calls in the same order.
     """
-    rng = np.random.default_rng(seed)
+    from .synth import Synth
+    rng = Synth(seed)
     f32 = np.float32
     for l in model.layers:
         if l.kind == "conv2d":
             k = l.params["K"]
             fan_in = k.shape[1] * k.shape[2] * k.shape[3]
-            l.params["K"] = (rng.standard_normal(k.shape, dtype=f32) * f32(np.sqrt(2.0 / fan_in))).astype(f32)
+            l.params["K"] = rng.normal(k.shape, 0.0, f32(np.sqrt(2.0 / fan_in)))
             l.params["bias"] = np.zeros_like(l.params["bias"])
         elif l.kind == "dense":
             w = l.params["W"]
-            l.params["W"] = (rng.standard_normal(w.shape, dtype=f32) * f32(np.sqrt(2.0 / w.shape[0]))).astype(f32)
+            l.params["W"] = rng.normal(w.shape, 0.0, f32(np.sqrt(2.0 / w.shape[0])))
             l.params["bias"] = np.zeros_like(l.params["bias"])
         elif l.kind == "batchnorm" and bn_stats:
             C = l.params["mean"].shape[0]
             if "bn_g" in l.params:
-                l.params["bn_g"] = rng.uniform(0.8, 1.2, C).astype(f32)
-                l.params["bn_b"] = (rng.standard_normal(C, dtype=f32) * f32(0.1)).astype(f32)
-            l.params["mean"] = (rng.standard_normal(C, dtype=f32) * f32(0.1)).astype(f32)
-            l.params["variance"] = rng.uniform(0.5, 1.5, C).astype(f32)
+                l.params["bn_g"] = rng.uniform(C, 0.8, 1.2)
+                l.params["bn_b"] = rng.normal(C, 0.0, 0.1)
+            l.params["mean"] = rng.normal(C, 0.0, 0.1)
+            l.params["variance"] = rng.uniform(C, 0.5, 1.5)
     if model.backend is not None:
         model._push_parameters()
     return model
+
+
+def synthetic_input(shape, seed, dist):
+    """The input batch of a configuration: ``dist`` "uniform" = U(0, 1), "normal" = N(0, 1), from a stream of its own
+    (``seed``), so that the parameters do not depend on the batch size."""
+    from .synth import Synth
+    rng = Synth(seed)
+    return rng.uniform(shape, 0.0, 1.0) if dist == "uniform" else rng.normal(shape, 0.0, 1.0)
 
 
 # ---------------------------------------------------------------------------- graphs

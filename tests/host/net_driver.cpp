@@ -15,6 +15,7 @@
 
 #include "eddl_hip_net.h"
 #include "eddl_hip_onnx.h"
+#include "eddl_hip_synth.h"
 
 using namespace eddl_hip;
 using namespace eddl_hip::eddl;
@@ -279,25 +280,37 @@ int main(int argc, char **argv) {
             fprintf(stderr, "unknown model %s\n", which.c_str());
             return 2;
         }
-        build(m, CS_HIP({1}));
+        // parameters "synth:<seed>": drawn on the host by the generator the Python host shares, then moved to the device;
+        // "-": drawn on the device by build(); anything else: a bin file loaded after build
+        const bool synth_params = params.compare(0, 6, "synth:") == 0;
+        if (synth_params) eddl_hip::synth_he_normal(m, (uint32_t)strtoul(params.c_str() + 6, nullptr, 10));
+        build(m, CS_HIP({1}), !synth_params);
         if (fused) {
             fuse(m);
             int away = 0;
             for (Layer *l : m->layers) away += m->is_fused_away(l) ? 1 : 0;
             printf("plan: %zu steps, %d layers computed inside another layer's step\n", m->plan.size(), away);
         }
-        if (params != "-") load(m, params);  // after fuse(): the kept filter copies must follow the new values
+        if (params != "-" && !synth_params) load(m, params);  // after fuse(): the kept filter copies must follow the new values
         printf("layers:");
         for (Layer *l : m->layers) printf(" %s", l->kind().c_str());
         printf("\n");
         vector<int> ishape = m->lin[0]->output->getShape();
         ishape[0] = batch;
         Tensor x(ishape, DEV_CPU);
-        std::ifstream ifs(in_path, std::ios::binary);
-        ifs.read(reinterpret_cast<char *>(x.ptr), x.size * sizeof(float));
-        if (!ifs.good()) {
-            fprintf(stderr, "short input file\n");
-            return 2;
+        if (in_path.compare(0, 6, "synth:") == 0) {  // synth:<seed>:<uniform|normal>: no input file either
+            const size_t colon2 = in_path.find(':', 6);
+            eddl_synth *gen = eddl_synth_new((uint32_t)strtoul(in_path.substr(6, colon2 - 6).c_str(), nullptr, 10));
+            if (in_path.substr(colon2 + 1) == "uniform") eddl_synth_uniform(gen, x.ptr, x.size, 0.0f, 1.0f);
+            else eddl_synth_normal(gen, x.ptr, x.size, 0.0f, 1.0f);
+            eddl_synth_free(gen);
+        } else {
+            std::ifstream ifs(in_path, std::ios::binary);
+            ifs.read(reinterpret_cast<char *>(x.ptr), x.size * sizeof(float));
+            if (!ifs.good()) {
+                fprintf(stderr, "short input file\n");
+                return 2;
+            }
         }
         // two forwards at two batch sizes first: every tensor is re-created on the way (resize)
         if (batch > 1) {

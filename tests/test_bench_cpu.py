@@ -56,7 +56,7 @@ def test_cpu_baseline_leg_checks_a_device_output_against_the_oracle(monkeypatch)
     monkeypatch.setattr(os, "sched_getaffinity", lambda pid: {0}, raising=False)
     model = models.conv_bn_relu_pool_block(**kwargs)
     models.init_he_normal(model, 2)
-    x = np.random.default_rng(1002).standard_normal(model.lin[0].out_shape, dtype=np.float32)
+    x = models.synthetic_input(model.lin[0].out_shape, 1002, "normal")   # the benchmark's own input: seed + 1000
     full = net_oracle.forward(Oracle(hpc=False), model, [x])[0]
     good = bench.cpu_baseline("block", want_seconds=0.1, device_output=full)["parity"]
     assert good["ok"] and good["images"] == 1 and good["max_abs_err"] == 0.0

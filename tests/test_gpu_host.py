@@ -163,6 +163,28 @@ def test_cpp_graphs_match_the_python_runner_bit_for_bit(hip, which, fused, tmp_p
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("which", ["block", "resnet50", "unet"])
+def test_cpp_host_builds_a_configuration_from_seeds_alone(hip, which, tmp_path):
+    """No parameter file and no input file: the C++ host draws both from the generator it shares with the Python host
+    (mt19937 + Box-Muller, seeds as the benchmark uses them) and must produce what the Python graph produces."""
+    from eddl_amd import models
+    batch = 2
+    if which == "block":
+        m, size, extra, dist = models.conv_bn_relu_pool_block(batch=batch, channels=6, size=16, filters=8), 16, [6, 8], "normal"
+    elif which == "resnet50":
+        m, size, extra, dist = models.resnet50(batch=batch, size=64, num_classes=10, base=8), 64, [10, 8], "normal"
+    else:
+        m, size, extra, dist = models.unet(batch=batch, size=32, widths=(4, 8), bottleneck=16), 32, [4, 8, 16], "uniform"
+    models.init_he_normal(m, 4)
+    x = models.synthetic_input(m.lin[0].out_shape, 1004, dist)
+    out = run_net_driver(["fused:" + which, "synth:4", "synth:1004:" + dist, tmp_path / "y.raw", batch, size] + extra)
+    assert "FAILED" not in out, out
+    m.build(hip, fuse=False)
+    want = m.predict([x])[0]
+    got = np.fromfile(tmp_path / "y.raw", np.float32).reshape(want.shape)
+    assert np.array_equal(got, want)
+
+
 def test_cpp_graph_errors_and_parameter_round_trip(hip, tmp_path):
     out = run_net_driver(["errors"])
     assert "FAILED" not in out and out.count("ok ") >= 17, out
