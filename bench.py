@@ -149,74 +149,60 @@ def cpu_baseline(workload, want_seconds=20.0, device_output=None):
     return result
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="vgg16", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--layers", action="store_true", help="print the per-op table to stderr")
-    ap.add_argument("--out", default=None, metavar="DIR", help="also write the per-op table and the result into this directory")
-    ap.add_argument("--unfused", action="store_true",
-                    help="one launch per layer (no Conv+BN+Add+ReLU / Pad / Dense+ReLU fusion): measures the stand-alone bandwidth kernels")
-    ap.add_argument("--graph", action="store_true",
-                    help="record the plan once as a graph and replay it with one call per step (for plans of short kernels)")
-    ap.add_argument("--conv-algo", default="auto", choices=["auto", "mfma_staged", "mfma_lds"], help="input gather of the convolution kernels")
-    ap.add_argument("--no-device-probe", action="store_true",
-                    help="skip the pure-MFMA probe of the device's sustained fp32 matrix rate (keeps kernel traces to the workload)")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="after the timed region run one ReLU over 2^26 floats (reads 256 MiB, writes 256 MiB): the plain copy "
-                         "kernel of known size that scales FETCH_SIZE / WRITE_SIZE counter readings")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this backend runs on ONE GPU (the forward path has no collectives); --gpus %d is not supported" % args.gpus)
+def oracle_parity(workload, device_output, max_images):
+    """End-to-end check of a device output against the CPU oracle (strict build) on the first images of the
+    workload's own batch; no timing.  The threads a small sample leaves idle share each image's convolutions
+    (same arithmetic)."""
+    from eddl_amd import models
+    from oracle import net_oracle
+    from oracle.oracle import Oracle
+    kwargs, seed, dist, _ = WORKLOADS[workload]
+    n = min(kwargs["batch"], max_images)
+    ora = Oracle(hpc=False)
+    ora.set_inner_parallel(True)
+    try:
+        model = builder_of(workload)(**dict(kwargs, batch=n))
+        models.init_he_normal(model, seed)
+        x = models.synthetic_input(model.lin[0].out_shape, seed + 1000, dist)
+        ref = net_oracle.forward(ora, model, [x], conv_algo="im2col")[0]
+    finally:
+        ora.set_inner_parallel(False)
+    got = np.asarray(device_output)[:n].reshape(ref.shape)
+    scale, err = float(np.abs(ref).max()), float(np.abs(got - ref).max())
+    return {"images": n, "max_abs_err": err, "max_abs_ref": scale, "err_over_max_ref": err / scale if scale > 0 else err,
+            "bound": PARITY_BOUND, "ok": bool(err <= PARITY_BOUND * scale)}
 
-    import eddl_amd
-    hip = eddl_amd.Backend(0)
-    hip.set_conv_algo(args.conv_algo)
-    model, x, desc = build_workload(args.workload)
-    model.build(hip, fuse=not args.unfused)
+
+RIDGE_FLOP_PER_BYTE = PEAK_FP32_MFMA_TFLOPS * 1e3 / PEAK_HBM_GBS  # 19.7: below it a layer is bound by HBM, not by the matrix cores
+
+
+def measure(hip, workload, steps, warmup, fused=True, graph=False):
+    """Builds the workload, runs `warmup` + `steps` forwards with the input resident in HBM, then times every op.
+    Returns (summary dict, per-op rows, device output of the last forward, model description)."""
+    model, x, desc = build_workload(workload)
+    model.build(hip, fuse=fused)
     batch = x.shape[0]
     model.input_tensor().copy_from(x)  # input resident in HBM before the timed region
     hip.synchronize()
-
     step = model.run
-    if args.graph:
+    if graph:
         model.capture()
         step = model.run_graph
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     hip.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     hip.synchronize()
     wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
     out_host = model.out[id(model.lout[0])].numpy()
     if not np.all(np.isfinite(out_host)):
-        sys.exit("bench.py: non-finite output")
-
-    if args.copy_probe:
-        probe_in, probe_out = hip.full((1 << 26,), 1.0), hip.empty((1 << 26,))
-        hip.relu(probe_in, probe_out)
-        hip.synchronize()
-        del probe_in, probe_out
+        sys.exit("bench.py: non-finite output (%s)" % workload)
 
     # ---- per-op device times (events on the kernels' stream), same resident input
-    reps = max(3, min(args.steps, 10))
+    reps = max(3, min(steps, 10))
     op_ms, op_kernels, kern_ms, kern_launches = time_ops(hip, model, reps)
-    # what an event pair reads around a kernel that does next to nothing (one float filled): the part of every
-    # per-op figure below that is not the op
-    tiny = hip.empty((1,))
-    pairs = [(hip.event(), hip.event()) for _ in range(50)]
-    for s, e in pairs:
-        s.record()
-        hip.fill_(tiny, 0.0)
-        e.record()
-    hip.synchronize()
-    event_floor_ms = float(np.median([s.elapsed_ms(e) for s, e in pairs]))
     rows = []
     for op, ms, kern, kms, kl in zip(model.ops, op_ms, op_kernels, kern_ms, kern_launches):
         row = {"op": op.kind, "name": op.name, "ms": ms, "flops": op.flops, "bytes": op.bytes}
@@ -240,16 +226,94 @@ def main():
     dom_flops, dom_ms = sum(r["flops"] for r in dom), sum(r["kernel_ms"] for r in dom)
     dom_launches = sum(r["kernel_launches"] for r in dom)
     achieved = dom_flops / dom_ms / 1e9 if dom_ms > 0 else 0.0
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic_%s.json" % args.workload)
-    if os.path.exists(tpath) and not args.unfused:  # the committed counter runs are of the fused plan
-        with open(tpath) as fh:
-            traffic = json.load(fh).get("hbm_bytes_per_launch")
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": traffic,
+                "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
                 "kernel": dom_name, "launches_per_step": dom_launches, "layers": len(dom),
                 "flops_per_launch": dom_flops / max(dom_launches, 1), "avg_launch_ms": dom_ms / max(dom_launches, 1),
                 "algorithmic_bytes_per_launch": sum(r["bytes"] for r in dom) / max(dom_launches, 1)}
+    # HBM bytes per launch of that kernel come from committed counter runs (two rocprofv3 --pmc passes cannot run
+    # inside this process); they are reported only when the file names the kernel this run found dominant
+    tpath = os.path.join(ROOT, "profiles", "traffic_%s.json" % workload)
+    if os.path.exists(tpath) and fused:  # the committed counter runs are of the fused plan
+        with open(tpath) as fh:
+            t = json.load(fh)
+        if t.get("kernel", "").replace(" ", "") == dom_name.replace(" ", ""):
+            roofline["traffic"] = t.get("hbm_bytes_per_launch")
+            roofline["traffic_measured_at_commit"] = t.get("commit")
+        else:
+            roofline["traffic_note"] = "profiles/traffic_%s.json is for %s, not this run's dominant kernel" % (workload, t.get("kernel"))
+    # convolutions whose arithmetic intensity is below the ridge (first layers with 1-3 input channels, 1-filter
+    # last layers): priced against the HBM roof
+    hbm_bound = [{"name": r["name"], "kernel": r.get("kernel"), "ms": r.get("kernel_ms", r["ms"]),
+                  "flop_per_byte": r["flops"] / r["bytes"], "gbs": r["bytes"] / r.get("kernel_ms", r["ms"]) / 1e6,
+                  "frac_hbm_peak": r["bytes"] / r.get("kernel_ms", r["ms"]) / 1e6 / PEAK_HBM_GBS}
+                 for r in conv_rows if r["bytes"] > 0 and r["flops"] / r["bytes"] < RIDGE_FLOP_PER_BYTE and r.get("kernel_ms", r["ms"]) > 0]
+    conv_ms = sum(r["ms"] for r in conv_rows)
+    conv_flops = sum(r["flops"] for r in conv_rows)
+    summary = {"value": batch * steps / wall, "unit": "images/sec", "ms_per_step": wall * 1e3 / steps, "steps": steps, "warmup": warmup,
+               "batch": batch, "fused_ops": len(model.ops), "roofline": roofline, "hbm_bound_convs": hbm_bound,
+               "conv_total": {"tflops": conv_flops / conv_ms / 1e9 if conv_ms else 0.0, "ms": conv_ms, "gflop": conv_flops / 1e9,
+                              "frac_fp32_mfma_peak": (conv_flops / conv_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS) if conv_ms else 0.0},
+               "device_ms_sum_of_ops": sum(op_ms)}
+    del model
+    return summary, rows, out_host, desc
+
+
+# the other configurations, run after the headline workload: (steps, warmup, images of the oracle's parity sample)
+OTHER_WORKLOADS = {"conv": (200, 20, 8), "block": (50, 5, 16), "resnet50": (20, 5, 16), "unet": (10, 3, 2)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="vgg16", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--layers", action="store_true", help="print the per-op table to stderr")
+    ap.add_argument("--out", default=None, metavar="DIR", help="also write the per-op table and the result into this directory")
+    ap.add_argument("--unfused", action="store_true",
+                    help="one launch per layer (no Conv+BN+Add+ReLU / Pad / Dense+ReLU fusion): measures the stand-alone bandwidth kernels")
+    ap.add_argument("--graph", action="store_true",
+                    help="record the plan once as a graph and replay it with one call per step (for plans of short kernels)")
+    ap.add_argument("--conv-algo", default="auto", choices=["auto", "mfma_staged", "mfma_lds"], help="input gather of the convolution kernels")
+    ap.add_argument("--no-device-probe", action="store_true",
+                    help="skip the pure-MFMA probe of the device's sustained fp32 matrix rate (keeps kernel traces to the workload)")
+    ap.add_argument("--no-workloads", action="store_true",
+                    help="report the headline workload only (without it a default VGG-16 run also measures the other four "
+                         "configurations, briefly, into the 'workloads' object of the JSON line)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="after the timed region run one ReLU over 2^26 floats (reads 256 MiB, writes 256 MiB): the plain copy "
+                         "kernel of known size that scales FETCH_SIZE / WRITE_SIZE counter readings")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this backend runs on ONE GPU (the forward path has no collectives); --gpus %d is not supported" % args.gpus)
+
+    import eddl_amd
+    hip = eddl_amd.Backend(0)
+    hip.set_conv_algo(args.conv_algo)
+    summary, rows, out_host, desc = measure(hip, args.workload, args.steps, args.warmup, fused=not args.unfused, graph=args.graph)
+    batch = summary["batch"]
+    ms_per_step = summary["ms_per_step"]
+    roofline = summary["roofline"]
+    achieved = roofline["achieved"]
+
+    if args.copy_probe:
+        probe_in, probe_out = hip.full((1 << 26,), 1.0), hip.empty((1 << 26,))
+        hip.relu(probe_in, probe_out)
+        hip.synchronize()
+        del probe_in, probe_out
+
+    # what an event pair reads around a kernel that does next to nothing (one float filled): the part of every
+    # per-op figure that is not the op
+    tiny = hip.empty((1,))
+    pairs = [(hip.event(), hip.event()) for _ in range(50)]
+    for s, e in pairs:
+        s.record()
+        hip.fill_(tiny, 0.0)
+        e.record()
+    hip.synchronize()
+    event_floor_ms = float(np.median([s.elapsed_ms(e) for s, e in pairs]))
 
     # what the matrix pipe sustains on this device with nothing else running (constant operands, then
     # operands that change every instruction): the published peak assumes the top clock throughout
@@ -264,18 +328,16 @@ def main():
         rd, wr, cp = hip.probe_hbm(1 << 30)
         roofline["device_probe"].update(hbm_unit="GB/s", hbm_read_stream=rd, hbm_write_stream=wr, hbm_copy_stream=cp)
 
-    conv_ms = sum(r["ms"] for r in conv_rows)
-    conv_flops = sum(r["flops"] for r in conv_rows)
     result = {
         "metric": "%s forward images/sec (fp32, 1 GPU%s)" % (args.workload, ", layer by layer" if args.unfused else ""),
-        "value": batch * args.steps / wall, "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": summary["value"], "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-        "data": "synthetic (seeded He-normal weights, U(0,1)/N(0,1) inputs, resident in HBM)",
-        "config": {"workload": desc, "batch": batch, "fused": not args.unfused, "fused_ops": len(model.ops), "graph_replay": bool(args.graph), "device": hip.name},
+        "data": "synthetic (mt19937 + Box-Muller: He-normal weights from the configuration's seed, U(0,1)/N(0,1) inputs from seed + 1000; resident in HBM)",
+        "config": {"workload": desc, "batch": batch, "fused": not args.unfused, "fused_ops": summary["fused_ops"], "graph_replay": bool(args.graph), "device": hip.name},
         "roofline": roofline,
-        "conv_total": {"tflops": conv_flops / conv_ms / 1e9 if conv_ms else 0.0, "ms": conv_ms, "gflop": conv_flops / 1e9,
-                       "frac_fp32_mfma_peak": (conv_flops / conv_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS) if conv_ms else 0.0},
-        "device_ms_sum_of_ops": sum(op_ms),
+        "hbm_bound_convs": summary["hbm_bound_convs"],
+        "conv_total": summary["conv_total"],
+        "device_ms_sum_of_ops": summary["device_ms_sum_of_ops"],
         "event_pair_floor_ms": event_floor_ms,
     }
     if not args.no_cpu_baseline:
@@ -285,6 +347,26 @@ def main():
             print(json.dumps(result))
             sys.exit("bench.py: the device's output differs from the CPU oracle's by %.3g of the largest output (bound %.0e)"
                      % (parity["err_over_max_ref"], PARITY_BOUND))
+
+    # ---- the other configurations, each for a fraction of a second of device time: throughput, dominant kernel against
+    # its roof, and the end-to-end parity of the timed run against the CPU oracle
+    if args.workload == "vgg16" and not (args.no_workloads or args.unfused or args.graph):
+        result["workloads"] = {}
+        for w, (steps, warmup, parity_images) in OTHER_WORKLOADS.items():
+            sm, _, out_w, desc_w = measure(hip, w, steps, warmup)
+            entry = {"workload": desc_w, "value": sm["value"], "unit": "images/sec", "ms_per_step": sm["ms_per_step"], "steps": steps,
+                     "warmup": warmup, "batch": sm["batch"], "dominant_kernel": sm["roofline"]["kernel"],
+                     "frac": sm["roofline"]["frac"], "achieved_tflops": sm["roofline"]["achieved"],
+                     "avg_launch_ms": sm["roofline"]["avg_launch_ms"], "launches_per_step": sm["roofline"]["launches_per_step"],
+                     "conv_total": sm["conv_total"], "hbm_bound_convs": sm["hbm_bound_convs"]}
+            if not args.no_cpu_baseline:
+                entry["parity"] = oracle_parity(w, out_w, parity_images)
+            result["workloads"][w] = entry
+        bad = [w for w, e in result["workloads"].items() if "parity" in e and not e["parity"]["ok"]]
+        if bad:
+            print(json.dumps(result))
+            sys.exit("bench.py: the device's output differs from the CPU oracle's beyond %.0e of the largest output in: %s"
+                     % (PARITY_BOUND, ", ".join(bad)))
 
     table = ["# ms = device time between two events around the op; an event pair around a one-element fill reads %.4f ms"
              % event_floor_ms,

@@ -59,6 +59,9 @@ int eddl_oracle_num_threads(void) {
 #endif
 }
 
+static int g_inner_parallel = 0;
+void eddl_oracle_set_inner_parallel(int on) { g_inner_parallel = on; }
+
 void eddl_oracle_set_num_threads(int n) {
 #ifdef _OPENMP
     if (n > 0) omp_set_num_threads(n);
@@ -172,8 +175,9 @@ void eddl_oracle_conv2d_direct_at(const float *I, const float *K, const float *b
  * column i is tap (c = i/(R*S), ky = (i%(R*S))/S, kx = i%S); stored column-major
  * (element (j,i) at j + i*P*Q); out-of-bounds taps read 0. */
 static void oracle_im2col(const float *img, float *col, int C, int H, int W, int R, int S, int sr, int sc, int pt,
-                          int pl, int P, int Q) {
+                          int pl, int P, int Q, int inner) {
     const int PQ = P * Q, CRS = C * R * S, RS = R * S;
+#pragma omp parallel for schedule(static) num_threads(inner) if (inner > 1)
     for (int i = 0; i < CRS; i++) {
         int pz = i / RS, ky = (i % RS) / S, kx = i % S;
         float *dst = col + (size_t)i * PQ;
@@ -197,9 +201,12 @@ static void oracle_im2col(const float *img, float *col, int C, int H, int W, int
  * (Wt(i,k) = K[k][i] over OIHW memory; Out(p,k) = O[b][k][p] in NCHW).
  * The reference's product is Eigen 3.4.0's GEBP kernel (not vendored, absent here): its
  * blocked summation order is Eigen-internal.  This routine sums the CRS products of one
- * output strictly in increasing tap index i, one fp32 accumulator per output. */
-static void oracle_sgemm_colmajor(const float *col, const float *Kw, float *out, int PQ, int CRS, int Kf) {
+ * output strictly in increasing tap index i, one fp32 accumulator per output.
+ * `inner` > 1 spreads the blocks of output pixels over that many more threads: every output is still summed by one
+ * thread in the same order, so the result does not depend on it. */
+static void oracle_sgemm_colmajor(const float *col, const float *Kw, float *out, int PQ, int CRS, int Kf, int inner) {
     enum { KB = 4, PB = 256 };
+#pragma omp parallel for schedule(dynamic, 1) num_threads(inner) if (inner > 1)
     for (int p0 = 0; p0 < PQ; p0 += PB) {
         int pn = PQ - p0 < PB ? PQ - p0 : PB;
         int k = 0;
@@ -243,8 +250,16 @@ int eddl_oracle_conv2d_im2col(const float *I, const float *K, const float *bias,
                               int Kf, int R, int S, int sr, int sc, int pt, int pl, int P, int Q) {
     const size_t PQ = (size_t)P * Q, CRS = (size_t)C * R * S;
     int nthreads = eddl_oracle_num_threads();
+    /* The reference runs one thread per image.  With eddl_oracle_set_inner_parallel(1) (checking runs on batches
+     * smaller than the machine, never the timed baseline) the threads left over also share each image's lowering
+     * and product, which changes no result. */
+    int inner = 1;
+    if (g_inner_parallel && N > 0 && nthreads > N) inner = nthreads / N;
     if (nthreads > N) nthreads = N;
     if (nthreads < 1) nthreads = 1;
+#ifdef _OPENMP
+    if (inner > 1) omp_set_max_active_levels(2);
+#endif
     float *scratch = (float *)malloc(sizeof(float) * PQ * CRS * (size_t)nthreads);
     if (!scratch) return -1;
 #pragma omp parallel for schedule(dynamic, 1) num_threads(nthreads)
@@ -255,8 +270,8 @@ int eddl_oracle_conv2d_im2col(const float *I, const float *K, const float *bias,
         int tid = 0;
 #endif
         float *col = scratch + (size_t)tid * PQ * CRS;
-        oracle_im2col(I + (size_t)b * C * H * W, col, C, H, W, R, S, sr, sc, pt, pl, P, Q);
-        oracle_sgemm_colmajor(col, K, O + (size_t)b * Kf * PQ, (int)PQ, (int)CRS, Kf);
+        oracle_im2col(I + (size_t)b * C * H * W, col, C, H, W, R, S, sr, sc, pt, pl, P, Q, inner);
+        oracle_sgemm_colmajor(col, K, O + (size_t)b * Kf * PQ, (int)PQ, (int)CRS, Kf, inner);
     }
     free(scratch);
     if (bias) {

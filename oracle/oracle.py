@@ -86,6 +86,11 @@ class Oracle:
     def set_num_threads(self, n):
         self.lib.eddl_oracle_set_num_threads(int(n))
 
+    def set_inner_parallel(self, on):
+        """Let the threads that a small batch leaves idle share each image's lowering and product in the im2col
+        convolution (for checking runs; results are unchanged, the reference's one-thread-per-image timing is not)."""
+        self.lib.eddl_oracle_set_inner_parallel(int(bool(on)))
+
     # ---- geometry (descriptor_conv2D.cpp / descriptor_pool2D.cpp)
     def out_size(self, padding, in_size, k, stride, dilation=1):
         """``padding`` is "same"/"zeros", "valid"/"none", or a (lo, hi) pair for custom pads."""
