@@ -88,6 +88,9 @@ struct ConvParams {
     const float *bias, *bn_g, *bn_b, *bn_mean, *bn_var, *residual;
     float bn_eps;
     int relu;
+    // The output is written with the streaming (non-temporal) hint: set by the host for a layer that is bound by its
+    // output traffic and whose output is larger than the last-level cache, so that keeping it there helps no reader.
+    int stream_out;
     int N, C, H, W, Kf, R, S, sr, sc, pt, pl, P, Q;
     int CRS, Mp, nsteps, PQ;
     long long npix;
@@ -268,7 +271,7 @@ __device__ __forceinline__ void store_tile_inside(const ConvParams &p, floatx16 
         rptr[tn] = p.residual + idx;  // not dereferenced without a residual
     }
     const bool has_bias = p.bias != nullptr, has_bn = p.bn_mean != nullptr, affine = p.bn_g != nullptr;
-    const bool has_res = p.residual != nullptr, relu = p.relu != 0;
+    const bool has_res = p.residual != nullptr, relu = p.relu != 0, stream_out = p.stream_out != 0;
 #pragma unroll
     for (int tm = 0; tm < TM; tm++) {
 #pragma unroll
@@ -322,10 +325,17 @@ __device__ __forceinline__ void store_tile_inside(const ConvParams &p, floatx16 
 #pragma unroll
                     for (int tn = 0; tn < TN; tn++) x[j][tn] = x[j][tn] > 0.0f ? x[j][tn] : 0.0f;
             }
+            if (stream_out) {
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+                for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int tn = 0; tn < TN; tn++) optr[tn][roff + (size_t)j * plane] = x[j][tn];
+                    for (int tn = 0; tn < TN; tn++) __builtin_nontemporal_store(x[j][tn], optr[tn] + roff + (size_t)j * plane);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) optr[tn][roff + (size_t)j * plane] = x[j][tn];
+            }
         }
     }
 }
@@ -926,6 +936,57 @@ __global__ __launch_bounds__(64) void conv_reduce_kernel(const ConvParams p) {
     store_tile<1, 1, 32>(p, acc, epi, m0, 0, (int)n0, lane);
 }
 
+// ---------------------------------------------------------------- 1x1 convolution onto a few filters
+// A 1x1, stride-1, unpadded convolution with at most four filters (a segmentation head: 64 -> 1) reads C values and
+// writes KF per pixel: no matrix-core tile has work for 32 filter rows, and the layer is a read stream.  One thread
+// takes VEC consecutive pixels of one image for all KF filters and walks the channels with eight loads in flight;
+// per output the products are added in increasing channel order with a separate multiply and add, which is the
+// reference's direct form (src/hardware/cpu/nn/cpu_conv.cpp:296-311) for a one-tap filter, rounding for rounding.
+template <int KF, int VEC>
+__global__ __launch_bounds__(256) void conv_pointwise_few_kernel(const ConvParams p) {
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
+    const size_t PQ = (size_t)p.PQ, per_img = PQ / VEC, total = (size_t)p.N * per_img;
+    ChannelEpilogue epi[KF];
+#pragma unroll
+    for (int k = 0; k < KF; k++) epi[k] = load_channel(p, k);
+    for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < total; g += (size_t)gridDim.x * 256) {
+        const size_t img = g / per_img, pq = (g - img * per_img) * VEC;
+        const float *src = p.I + img * (size_t)p.C * PQ + pq;
+        float acc[KF][VEC];
+#pragma unroll
+        for (int k = 0; k < KF; k++)
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[k][v] = 0.0f;
+        for (int c0 = 0; c0 < p.C; c0 += 8) {
+            vec_t x[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int c = c0 + u < p.C ? c0 + u : p.C - 1;  // a short last group re-reads the last channel; unused below
+                x[u] = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(src + (size_t)c * PQ));
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                if (c0 + u < p.C) {
+#pragma unroll
+                    for (int k = 0; k < KF; k++) {
+                        const float w = p.K[(size_t)k * p.C + c0 + u];
+#pragma unroll
+                        for (int v = 0; v < VEC; v++) acc[k][v] = __fadd_rn(acc[k][v], __fmul_rn(w, x[u][v]));
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < KF; k++) {
+            const size_t o = (img * KF + k) * PQ + pq;
+            vec_t y;
+#pragma unroll
+            for (int v = 0; v < VEC; v++) y[v] = apply_epilogue(p, epi[k], acc[k][v], o + v);
+            *reinterpret_cast<vec_t *>(p.O + o) = y;
+        }
+    }
+}
+
 // ---------------------------------------------------------------- scalar direct kernel
 // One thread per output, taps in the order ky, kx, c with a separate multiply and add per tap
 // (src/hardware/cpu/nn/cpu_conv.cpp:282-314).  Slow; exists to check the MFMA kernels on the
@@ -1358,6 +1419,13 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     p.K = K; p.O = O; p.Wp = nullptr;
     p.bias = bias; p.bn_g = bn_g; p.bn_b = bn_b; p.bn_mean = bn_mean; p.bn_var = bn_var; p.residual = residual;
     p.bn_eps = bn_eps; p.relu = relu;
+    {
+        // bound by its output traffic (arithmetic intensity under the ridge of 157.3 TFLOP/s over 8 TB/s) and an output that
+        // the 256 MB last-level cache cannot hold for the next layer anyway
+        const double out_bytes = 4.0 * N * Kf * P * Q, in_bytes = 4.0 * N * C * H * W;
+        const double flops = 2.0 * N * Kf * (double)C * R * S * P * Q;
+        p.stream_out = (out_bytes >= 256e6 && out_bytes > 2 * in_bytes && flops / (out_bytes + in_bytes) < 19.7) ? 1 : 0;
+    }
     p.N = N; p.C = C; p.H = H; p.W = W; p.Kf = Kf; p.R = R; p.S = S; p.sr = sr; p.sc = sc; p.pt = pad_top; p.pl = pad_left;
     p.P = P; p.Q = Q;
     p.CRS = C * R * S;
@@ -1374,6 +1442,30 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
         snprintf(g_last_kernel, sizeof(g_last_kernel), "conv_direct_kernel");
         EH_TRY(prof_begin(st));
         hipLaunchKernelGGL(conv_direct_kernel, dim3(eh_blocks(total, 256, 1u << 20)), dim3(256), 0, st, p);
+        EH_CHECK_LAUNCH();
+        EH_TRY(prof_end(st));
+        return 0;
+    }
+
+    // ---- a 1x1 convolution onto at most four filters: a read stream, no tile
+    if (g_algo == 0 && g_force_tile < 0 && R == 1 && S == 1 && sr == 1 && sc == 1 && pad_top == 0 && pad_left == 0 && Kf <= 4 && !two &&
+        uh == 1 && uw == 1 && P == H && Q == W) {
+        const bool vec4 = p.PQ % 4 == 0 && (((size_t)I | (size_t)O | (size_t)(residual ? residual : O)) & 15) == 0;
+        void (*kern)(const ConvParams) = nullptr;
+        switch (Kf * 2 + (vec4 ? 1 : 0)) {
+            case 2: kern = conv_pointwise_few_kernel<1, 1>; break;
+            case 3: kern = conv_pointwise_few_kernel<1, 4>; break;
+            case 4: kern = conv_pointwise_few_kernel<2, 1>; break;
+            case 5: kern = conv_pointwise_few_kernel<2, 4>; break;
+            case 6: kern = conv_pointwise_few_kernel<3, 1>; break;
+            case 7: kern = conv_pointwise_few_kernel<3, 4>; break;
+            case 8: kern = conv_pointwise_few_kernel<4, 1>; break;
+            default: kern = conv_pointwise_few_kernel<4, 4>; break;
+        }
+        const size_t groups = (size_t)N * (p.PQ / (vec4 ? 4 : 1));
+        snprintf(g_last_kernel, sizeof(g_last_kernel), "conv_pointwise_few_kernel<%d,%d>", Kf, vec4 ? 4 : 1);
+        EH_TRY(prof_begin(st));
+        hipLaunchKernelGGL(kern, dim3(eh_blocks(groups, 256, 256 * 16)), dim3(256), 0, st, p);
         EH_CHECK_LAUNCH();
         EH_TRY(prof_end(st));
         return 0;

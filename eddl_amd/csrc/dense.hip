@@ -39,25 +39,33 @@ __global__ __launch_bounds__(256) void dense_transpose_kernel(const float *__res
     }
 }
 
-// grid: (column tiles of 128, k slices, row tiles of 32); block: one wavefront.
+// grid: (column tiles of 128, k slices, groups of MT row tiles of 32); block: one wavefront, which multiplies every
+// float4 of weights it loads into MT accumulator sets: one pass over B serves MT x 32 rows (a batch of up to 128 rows
+// reads the weights once; the activations, transposed, are small and come from L2).
 // VEC: n is a multiple of 4 and B is 16-byte aligned, so a lane's four columns are one float4.
 // STREAM (with VEC): the weights are read with the streaming (non-temporal) hint - for matrices larger than
 // the device's caches, which no later kernel finds there anyway (25088 x 4096: 96 -> 88 us).
-template <bool VEC, bool STREAM>
+template <bool VEC, bool STREAM, int MT>
 __global__ __launch_bounds__(64) void dense_partial_kernel(const float *__restrict__ At, const float *__restrict__ B,
                                                            float *__restrict__ part, int m, int k, int n, int kslice) {
     const int lane = threadIdx.x, half = lane >> 5, l = lane & 31;
-    const int n0 = blockIdx.x * 128, ks = blockIdx.y, mt = blockIdx.z;
+    const int n0 = blockIdx.x * 128, ks = blockIdx.y, mt0 = blockIdx.z * MT;
     const int kbeg = ks * kslice;
     int kend = kbeg + kslice;
     if (kend > k) kend = k;
     const int col0 = n0 + 4 * l;
-    const float *ap = At + (size_t)mt * k * 32 + l;
-    floatx16 acc[4];
+    const int mtiles = (m + 31) / 32;
+    // row tile mt0 + t of this group, or the last existing one again (its results are not stored)
+    const float *ap[MT];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int t = 0; t < MT; t++) ap[t] = At + (size_t)(mt0 + t < mtiles ? mt0 + t : mtiles - 1) * k * 32 + l;
+    floatx16 acc[MT][4];
 #pragma unroll
-        for (int v = 0; v < 16; v++) acc[j][v] = 0.0f;
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[t][j][v] = 0.0f;
     auto load_b = [&](int ki) -> floatx4 {
         floatx4 b = {0.0f, 0.0f, 0.0f, 0.0f};
         if (ki < kend) {
@@ -73,15 +81,25 @@ __global__ __launch_bounds__(64) void dense_partial_kernel(const float *__restri
         }
         return b;
     };
-    constexpr int U = 8;
+    auto multiply = [&](const float (&a)[MT], const floatx4 &b) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            acc[t][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b.x, acc[t][0], 0, 0, 0);
+            acc[t][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b.y, acc[t][1], 0, 0, 0);
+            acc[t][2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b.z, acc[t][2], 0, 0, 0);
+            acc[t][3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b.w, acc[t][3], 0, 0, 0);
+        }
+    };
+    constexpr int U = MT == 1 ? 8 : 4;  // k pairs (float4 of weights per lane) in flight
     int kk = kbeg;
-    for (; kk + 2 * U <= kend; kk += 2 * U) {  // U k pairs (U float4 of weights per lane) in flight
-        float a[U];
+    for (; kk + 2 * U <= kend; kk += 2 * U) {
+        float a[U][MT];
         floatx4 b[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int ki = kk + 2 * u + half;
-            a[u] = ap[(size_t)ki * 32];
+#pragma unroll
+            for (int t = 0; t < MT; t++) a[u][t] = ap[t][(size_t)ki * 32];
             const float *row = B + (size_t)ki * n;
             if (VEC) {
                 const floatx4 *src = reinterpret_cast<const floatx4 *>(row + col0);
@@ -91,37 +109,32 @@ __global__ __launch_bounds__(64) void dense_partial_kernel(const float *__restri
             }
         }
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].x, acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].y, acc[1], 0, 0, 0);
-            acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].z, acc[2], 0, 0, 0);
-            acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u].w, acc[3], 0, 0, 0);
-        }
+        for (int u = 0; u < U; u++) multiply(a[u], b[u]);
     }
     for (; kk < kend; kk += 2) {
         const int ki = kk + half;
-        const float a = ki < kend ? ap[(size_t)ki * 32] : 0.0f;
-        const floatx4 b = load_b(ki);
-        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b.x, acc[0], 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b.y, acc[1], 0, 0, 0);
-        acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b.z, acc[2], 0, 0, 0);
-        acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b.w, acc[3], 0, 0, 0);
+        float a[MT];
+#pragma unroll
+        for (int t = 0; t < MT; t++) a[t] = ki < kend ? ap[t][(size_t)ki * 32] : 0.0f;
+        multiply(a, load_b(ki));
     }
     // part[ks][row][col]: accumulator j, lane column l -> column col0 + j; rows 8*(v/4) + 4*half + v%4
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
-        const int r = mt * 32 + 8 * (v / 4) + 4 * half + (v % 4);
-        if (r < m) {
-            float *dst = part + ((size_t)ks * m + r) * n + col0;
-            if (VEC) {
-                if (col0 < n) *reinterpret_cast<floatx4 *>(dst) = floatx4{acc[0][v], acc[1][v], acc[2][v], acc[3][v]};
-            } else {
+    for (int t = 0; t < MT; t++)
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (col0 + j < n) dst[j] = acc[j][v];
+        for (int v = 0; v < 16; v++) {
+            const int r = (mt0 + t) * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+            if (r < m) {
+                float *dst = part + ((size_t)ks * m + r) * n + col0;
+                if (VEC) {
+                    if (col0 < n) *reinterpret_cast<floatx4 *>(dst) = floatx4{acc[t][0][v], acc[t][1][v], acc[t][2][v], acc[t][3][v]};
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (col0 + j < n) dst[j] = acc[t][j][v];
+                }
             }
         }
-    }
 }
 
 // Adds the K slices in slice order; then, in the reference's order, C += (incC), + bias[column]
@@ -164,7 +177,9 @@ int dense_impl(int dev, const float *A, const float *B, float *C, int m, int k, 
     // Wavefronts to cover the device eight times over, in slices of at least 128 taps (shorter
     // slices cost more in partial blocks written and read back than they gain) - unless that
     // leaves fewer than four wavefronts per CU, when slices go down to 64 taps.
-    const long long blocks = (long long)nt * mt;
+    const int MT = mt >= 3 ? 4 : mt;  // row tiles one wavefront serves with each float4 of weights it loads
+    const int mgroups = (mt + MT - 1) / MT;
+    const long long blocks = (long long)nt * mgroups;
     const long long num_cu = state(dev).num_cu;
     long long nsl = (8 * num_cu + blocks - 1) / blocks;
     const long long max128 = (k + 127) / 128, max64 = (k + 63) / 64;
@@ -172,7 +187,7 @@ int dense_impl(int dev, const float *A, const float *B, float *C, int m, int k, 
     int nslices = (int)std::max(1LL, nsl);
     int kslice = ((k + nslices - 1) / nslices + 1) & ~1;  // even, so MFMA tap pairs do not straddle slices
     nslices = (k + kslice - 1) / kslice;
-    EH_REQUIRE(nslices <= 65535 && mt <= 65535, "%s: shape out of range", what);
+    EH_REQUIRE(nslices <= 65535 && mgroups <= 65535, "%s: shape out of range", what);
     const size_t at_bytes = ((size_t)mt * k * 32 * sizeof(float) + 255) & ~(size_t)255;
     void *ws = nullptr;
     EH_TRY(get_workspace(dev, at_bytes + (size_t)nslices * m * n * sizeof(float), &ws));
@@ -181,8 +196,13 @@ int dense_impl(int dev, const float *A, const float *B, float *C, int m, int k, 
     EH_CHECK_LAUNCH();
     const bool vec = (n % 4 == 0) && (((uintptr_t)B & 15u) == 0);
     const bool stream = vec && (size_t)k * n * sizeof(float) > ((size_t)256 << 20);  // beyond the 256 MB last-level cache
-    auto kern = !vec ? dense_partial_kernel<false, false> : (stream ? dense_partial_kernel<true, true> : dense_partial_kernel<true, false>);
-    hipLaunchKernelGGL(kern, dim3(nt, nslices, mt), dim3(64), 0, st, At, B, part, m, k, n, kslice);
+    typedef void (*partial_fn)(const float *, const float *, float *, int, int, int, int);
+    static const partial_fn kernels[3][3] = {
+        {dense_partial_kernel<false, false, 1>, dense_partial_kernel<true, false, 1>, dense_partial_kernel<true, true, 1>},
+        {dense_partial_kernel<false, false, 2>, dense_partial_kernel<true, false, 2>, dense_partial_kernel<true, true, 2>},
+        {dense_partial_kernel<false, false, 4>, dense_partial_kernel<true, false, 4>, dense_partial_kernel<true, true, 4>}};
+    const partial_fn kern = kernels[MT == 1 ? 0 : MT == 2 ? 1 : 2][!vec ? 0 : (stream ? 2 : 1)];
+    hipLaunchKernelGGL(kern, dim3(nt, nslices, mgroups), dim3(64), 0, st, At, B, part, m, k, n, kslice);
     EH_CHECK_LAUNCH();
     size_t mn = (size_t)m * n;
     hipLaunchKernelGGL(dense_reduce_kernel, dim3(eh_blocks(mn, 256, 65536)), dim3(256), 0, st, (const float *)part, C, mn, nslices, incC,

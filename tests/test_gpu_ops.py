@@ -139,6 +139,34 @@ def test_conv2d_mfma_against_oracle(hip, oracle, shape, algo):
     assert_conv_close(ref, out, str(shape) + " " + hip.last_conv_kernel())
 
 
+@pytest.mark.parametrize("kf", [1, 2, 3, 4])
+def test_conv2d_onto_few_filters_is_the_direct_form_bit_for_bit(hip, oracle, kf):
+    """A 1x1 stride-1 convolution onto at most four filters takes the streaming kernel, which adds the products in
+    increasing channel order with a separate multiply and add: the reference's direct form for a one-tap filter
+    (src/hardware/cpu/nn/cpu_conv.cpp:296-311).  Whole fused tail, odd channel counts, planes of a multiple of four
+    pixels (16-byte accesses) and not."""
+    rng = np.random.default_rng(600 + kf)
+    for N, C, H, W in ((3, 64, 16, 12), (2, 5, 7, 9), (1, 13, 1, 1), (4, 8, 32, 32)):
+        x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+        w = rng.standard_normal((kf, C, 1, 1), dtype=np.float32)
+        b = rng.standard_normal(kf).astype(np.float32)
+        bn = (rng.uniform(0.8, 1.2, kf).astype(np.float32), rng.standard_normal(kf).astype(np.float32),
+              rng.standard_normal(kf).astype(np.float32), rng.uniform(0.5, 1.5, kf).astype(np.float32), 1e-5)
+        res = rng.standard_normal((N, kf, H, W), dtype=np.float32)
+        for kw in ({}, dict(bn=bn, residual=res, relu=True)):
+            ref, out = run_conv(hip, oracle, x, w, b, (1, 1), "valid", **kw)
+            assert hip.last_conv_kernel().startswith("conv_pointwise_few_kernel<%d," % kf), hip.last_conv_kernel()
+            assert np.array_equal(ref, out), (kf, (N, C, H, W), kw.keys())
+    # the same layer through the matrix-core kernels (forced plan) agrees to the convolution tolerance
+    hip.force_conv_plan(3, 1)
+    try:
+        ref, out = run_conv(hip, oracle, x, w, b, (1, 1), "valid")
+    finally:
+        hip.force_conv_plan(-1, 1)
+    assert hip.last_conv_kernel().startswith("conv_tap_kernel")
+    assert_conv_close(ref, out, "few filters through the tile kernel")
+
+
 @pytest.mark.parametrize("shape", CONV_SHAPES[:6], ids=lambda s: "x".join(str(v) for v in s[:9]))
 def test_conv2d_direct_kernel_is_bit_exact(hip, oracle, shape):
     N, C, H, W, Kf, R, S, sr, sc, padding, pads, use_bias = shape
@@ -506,7 +534,8 @@ def test_upsample_concat_pad_bit_exact(hip, oracle):
 
 def test_dense_sigmoid_softmax_within_tolerance(hip, oracle):
     rng = np.random.default_rng(405)
-    for m, k, n in [(32, 512, 1000), (5, 37, 300), (64, 2048, 10), (33, 100, 65), (70, 1001, 131), (32, 3136, 4096), (1, 2, 1)]:
+    for m, k, n in [(32, 512, 1000), (5, 37, 300), (64, 2048, 10), (33, 100, 65), (70, 1001, 131), (32, 3136, 4096), (1, 2, 1),
+                    (128, 777, 256), (129, 300, 132), (200, 64, 40), (96, 2048, 1000)]:  # 4, 5, 7, 3 row tiles: one pass over the weights serves four
         a = rng.standard_normal((m, k), dtype=np.float32)
         w = (rng.standard_normal((k, n)) * np.sqrt(2.0 / k)).astype(np.float32)
         bias = rng.standard_normal(n, dtype=np.float32)
