@@ -375,10 +375,12 @@ def test_conv2d_argument_errors(hip):
 # ------------------------------------------------------------------ bandwidth-bound operators
 def test_batchnorm_inference_bit_exact(hip, oracle):
     rng = np.random.default_rng(400)
-    # planes below 4096 elements take the flat kernel (float4 groups that cross plane borders when the plane size is
-    # not a multiple of 4, a ragged end), larger ones and planes of fewer than 4 elements the plane-per-workgroup kernel
+    # planes of 16 .. 4095 elements and a multiple of four take the channel-per-workgroup kernel (image groups, partly
+    # filled thread rows), other planes below 4096 elements the flat kernel (float4 groups that cross plane borders, a
+    # ragged end), larger ones and planes of fewer than 4 elements the plane-per-workgroup kernel
     for shape in [(4, 64, 28, 28), (3, 5, 7, 9), (2, 130, 1, 1), (2, 3, 6, 6), (1, 20000, 1, 2), (2, 7, 5, 1), (2, 70, 7, 7),
-                  (1, 3, 7, 7), (1, 2, 64, 63), (1, 2, 64, 64), (3, 2, 70, 70), (5, 300, 2, 2)]:
+                  (1, 3, 7, 7), (1, 2, 64, 63), (1, 2, 64, 64), (3, 2, 70, 70), (5, 300, 2, 2),
+                  (70, 3, 14, 14), (9, 33, 56, 56), (2, 2100, 4, 4), (37, 40, 20, 3), (1, 1, 4, 4)]:
         C = shape[1]
         x = rng.standard_normal(shape, dtype=np.float32)
         g, b, mean, var, eps = _bn_params(rng, C)
