@@ -8,6 +8,9 @@
 #include <iostream>
 #include <stdexcept>
 
+#include <stdio.h>
+#include <sys/time.h>
+
 #include "../../include/eddlhip.h"
 
 namespace eddl_hip {
@@ -25,6 +28,56 @@ void msg(const string &text, const string &title) {
 // gpu_check, the wait after every call and every gpu_* function are defined in the binding translation unit,
 // integration/eddl/src/hardware/hip/hip_backend.cpp, which the Makefile compiles into this library against the
 // classes below (EDDLHIP_MIRROR_BUILD).
+
+// ---------------------------------------------------------------- profile
+static vector<ProfileCounter *> &profile_registry() {
+    static vector<ProfileCounter *> all;
+    return all;
+}
+ProfileCounter::ProfileCounter(const char *n) : name(n) { profile_registry().push_back(this); }
+
+static long long now_us() {
+    struct timeval tv;
+    gettimeofday(&tv, nullptr);
+    return (long long)tv.tv_sec * 1000000 + tv.tv_usec;
+}
+ProfileScope::ProfileScope(ProfileCounter &c) : counter(c), t0_us(now_us()) {}
+ProfileScope::~ProfileScope() {
+    counter.time_us += (unsigned long long)(now_us() - t0_us);
+    counter.calls += 1;
+}
+
+#define EDDL_HIP_PROFILE(fn)                 \
+    static ProfileCounter prof_##fn(#fn);    \
+    ProfileScope prof_scope_##fn(prof_##fn)
+
+ProfileCounter &profile_forward() {
+    static ProfileCounter forward("forward");
+    return forward;
+}
+
+static void profile_line(const ProfileCounter *c) {
+    if (c->calls > 0)
+        printf("| %-50s: %8lld calls, %12lld us , %12.4f us/call |\n", c->name, (long long)c->calls, (long long)c->time_us,
+               (float)c->time_us / (float)c->calls);
+}
+
+void __show_profile() {
+    const char *bar = "==============================================================================================================\n";
+    const char *rule = "-------------------------------------------------------------------------------------------------------------|\n";
+    printf("%s| Profiling (model)                                                                                          |\n%s", bar, rule);
+    profile_line(&profile_forward());
+    printf("%s| Profiling (functions)                                                                                      |\n%s", bar, rule);
+    for (const ProfileCounter *c : profile_registry())
+        if (c != &profile_forward()) profile_line(c);
+    printf("%s", bar);
+    fflush(stdout);
+}
+
+void __reset_profile() {
+    profile_forward();
+    for (ProfileCounter *c : profile_registry()) c->time_us = c->calls = 0;
+}
 
 // ---------------------------------------------------------------- Tensor
 static void need_gpu(const Tensor *t, const char *where) {
@@ -128,26 +181,32 @@ void Tensor::fill_(float v) {
 // Random fills and scalar arithmetic as the reference's initialisers use them on a device tensor
 // (src/tensor/tensor_generator.cpp:25-110, src/tensor/tensor_math.cpp:1455-1470)
 void Tensor::fill_rand_uniform_(float v) {
+    EDDL_HIP_PROFILE(fill_rand_uniform);
     need_gpu(this, "Tensor::fill_rand_uniform_");
     gpu_rand_uniform(this, v);
 }
 void Tensor::fill_rand_signed_uniform_(float v) {
+    EDDL_HIP_PROFILE(fill_rand_signed_uniform);
     need_gpu(this, "Tensor::fill_rand_signed_uniform_");
     gpu_rand_signed_uniform(this, v);
 }
 void Tensor::fill_rand_normal_(float m, float s) {
+    EDDL_HIP_PROFILE(fill_rand_normal);
     need_gpu(this, "Tensor::fill_rand_normal_");
     gpu_rand_normal(this, m, s);
 }
 void Tensor::fill_rand_binary_(float v) {
+    EDDL_HIP_PROFILE(fill_rand_binary);
     need_gpu(this, "Tensor::fill_rand_binary_");
     gpu_rand_binary(this, v);
 }
 void Tensor::mult_(float v) {
+    EDDL_HIP_PROFILE(mult);
     need_gpu(this, "Tensor::mult_");
     gpu_mult(this, this, v);
 }
 void Tensor::add_(float v) {
+    EDDL_HIP_PROFILE(add);
     need_gpu(this, "Tensor::add_");
     gpu_add(this, this, v);
 }
@@ -188,6 +247,7 @@ void Tensor::copy(Tensor *A, Tensor *B) {
 }
 
 void Tensor::add(float scA, Tensor *A, float scB, Tensor *B, Tensor *C, int incC) {
+    EDDL_HIP_PROFILE(add);
     if (A->device != B->device || A->device != C->device) msg("Tensors in different devices", "Tensor::add");
     if (A->size != B->size || A->size != C->size) msg("Incompatible dims", "Tensor::add");
     need_gpu(A, "Tensor::add");
@@ -195,6 +255,7 @@ void Tensor::add(float scA, Tensor *A, float scB, Tensor *B, Tensor *C, int incC
 }
 
 void Tensor::inc(Tensor *A, Tensor *B) {
+    EDDL_HIP_PROFILE(inc);
     if (A->size != B->size) msg("Tensors with different shape", "Tensor::inc");
     need_gpu(A, "Tensor::inc");
     gpu_inc(A, B);
@@ -221,6 +282,7 @@ Tensor *Tensor::concat(const vector<Tensor *> A, unsigned int axis, Tensor *outp
 }
 
 void Tensor::scale(Tensor *A, Tensor *B, vector<int> new_shape, int wrapping_mode, float cval, int mode) {
+    EDDL_HIP_PROFILE(scale);
     if (new_shape[0] <= 0 || new_shape[1] <= 0) msg("The new shape must be a greater than zero", "Tensor::scale");
     if (A->ndim != 4 || B->ndim != 4) msg("This method requires two 4D tensors", "Tensor::scale");
     if (A->device != B->device) msg("Tensors in different devices", "Tensor::scale");
@@ -243,6 +305,7 @@ void Tensor::pad(Tensor *A, Tensor *B, vector<int> pads) {
 }
 
 void Tensor::mult2D(Tensor *A, int tA, Tensor *B, int tB, Tensor *C, int incC) {
+    EDDL_HIP_PROFILE(mult2D);
     if (A->device != B->device || A->device != C->device) msg("Tensors in different devices", "Tensor::mult2D");
     if (A->ndim != 2 || B->ndim != 2 || C->ndim != 2) msg("Only 2D tensors", "Tensor::mult2D");
     need_gpu(A, "Tensor::mult2D");
@@ -250,6 +313,7 @@ void Tensor::mult2D(Tensor *A, int tA, Tensor *B, int tB, Tensor *C, int incC) {
 }
 
 void Tensor::sum2D_rowwise(Tensor *A, Tensor *B, Tensor *C) {
+    EDDL_HIP_PROFILE(sum2D_rowwise);
     if (A->ndim != 2 || B->ndim != 1 || C->ndim != 2) msg("sum2D_rowwise dims", "Tensor::sum2D_rowwise");
     if (A->shape[1] != B->shape[0] || A->shape != C->shape) msg("Incompatible dims", "Tensor::sum2D_rowwise");
     need_gpu(A, "Tensor::sum2D_rowwise");
@@ -433,6 +497,7 @@ void PoolDescriptor::resize(int b) {
 namespace tensorNN {
 
 void Conv2D(ConvolDescriptor *D) {
+    EDDL_HIP_PROFILE(Conv2D);
     if ((D->I->ndim != 4)) msg("Tensors are not 4D", "Tensor::Conv2D");
     if (D->dilation_rate[0] != 1 || D->dilation_rate[1] != 1) msg("Dilated convolutions are only available with CuDNN", "Tensor::Conv2D");
     need_gpu(D->I, "Tensor::Conv2D");
@@ -440,12 +505,14 @@ void Conv2D(ConvolDescriptor *D) {
 }
 
 void MPool2D(PoolDescriptor *D) {
+    EDDL_HIP_PROFILE(MPool2D);
     if ((D->I->ndim != 4)) msg("Tensors are not 4D", "Tensor::MPool2D");
     need_gpu(D->I, "Tensor::MPool2D");
     gpu_mpool2D(D);
 }
 
 void AvgPool2D(PoolDescriptor *D) {
+    EDDL_HIP_PROFILE(AvgPool2D);
     if ((D->I->ndim != 4)) msg("Tensors are not 4D", "Tensor::AvgPool2D");
     need_gpu(D->I, "Tensor::AvgPool2D");
     gpu_avgpool2D(D);
@@ -460,6 +527,7 @@ void BatchNormForward(Tensor *input, Tensor *output, Tensor *opa, Tensor *mean, 
 }
 
 void ReLu(Tensor *A, Tensor *B) {
+    EDDL_HIP_PROFILE(ReLu);
     if (A->device != B->device) msg("Tensors in different devices", "Tensor::ReLu");
     if (A->size != B->size) msg("Incompatible dims", "Tensor::ReLu");
     need_gpu(A, "Tensor::ReLu");
@@ -467,6 +535,7 @@ void ReLu(Tensor *A, Tensor *B) {
 }
 
 void Sigmoid(Tensor *A, Tensor *B) {
+    EDDL_HIP_PROFILE(Sigmoid);
     if (A->device != B->device) msg("Tensors in different devices", "Tensor::Sigmoid");
     if (A->size != B->size) msg("Incompatible dims", "Tensor::Sigmoid");
     need_gpu(A, "Tensor::Sigmoid");
@@ -474,6 +543,7 @@ void Sigmoid(Tensor *A, Tensor *B) {
 }
 
 void FullSoftmax(Tensor *A, Tensor *B, int axis, bool stable) {
+    EDDL_HIP_PROFILE(Softmax);
     if (A->device != B->device) msg("Tensors in different devices", "Tensor::FullSoftmax");
     if (A->shape != B->shape) msg("Incompatible dims", "Tensor::FullSoftmax");
     need_gpu(A, "Tensor::FullSoftmax");

@@ -179,6 +179,30 @@ void gpu_pad(Tensor *A, Tensor *B, vector<int> pads);
 void gpu_mult2D(Tensor *A, int tA, Tensor *B, int tB, Tensor *C, int incC);
 void gpu_sum2D_rowwise(Tensor *A, Tensor *B, Tensor *C);
 
+// ---- host wall-clock profile of the dispatchers, as the reference keeps it (include/eddl/profiling.h:27-66,
+// src/profiling.cpp:200-330): per function, the number of calls and the microseconds between entry and return
+// (gettimeofday).  With the wait after every gpu_* call the figure contains the kernel; with gpu_set_synchronous(false) it
+// is the time to queue it.  Counter names are the reference's: forward, Conv2D, MPool2D, AvgPool2D, ReLu, Sigmoid,
+// Softmax, add, inc, mult, mult2D, sum2D_rowwise, scale, fill_rand_uniform, fill_rand_signed_uniform, fill_rand_normal,
+// fill_rand_binary.
+struct ProfileCounter {
+    const char *name;
+    unsigned long long time_us = 0, calls = 0;
+    explicit ProfileCounter(const char *n);
+};
+class ProfileScope {
+  public:
+    explicit ProfileScope(ProfileCounter &c);
+    ~ProfileScope();
+
+  private:
+    ProfileCounter &counter;
+    long long t0_us;
+};
+void __show_profile();   // the reference's two tables on stdout (src/profiling.cpp:200-330): "forward", then the functions called
+void __reset_profile();  // src/profiling.cpp:332-480
+ProfileCounter &profile_forward();  // the counter Net::forward charges (Net::do_forward, src/net/net_func.cpp:49-55)
+
 // ---- the dispatchers the layers call (GPU branch only: this backend has no CPU path)
 namespace tensorNN {
 void Conv2D(ConvolDescriptor *D);

@@ -519,6 +519,7 @@ void Net::setmode(int m) {
 }
 
 void Net::forward() {
+    ProfileScope profile(profile_forward());
     if (plan.empty()) {
         for (Layer *l : layers) l->forward();
         return;
@@ -851,6 +852,8 @@ compserv CS_GPU(const vector<int> &g, const string &mem) { return CS_HIP(g, mem)
 
 void build(model net, compserv cs, bool init_weights) { net->build(cs, init_weights); }
 void fuse(model net) { net->fuse(); }
+void show_profile() { __show_profile(); }
+void reset_profile() { __reset_profile(); }
 void set_mode(model net, int mode) { net->setmode(mode); }
 void summary(model m) { m->summary(true); }
 void load(model m, const string &fname, const string &format) { m->load(fname, format); }

@@ -284,6 +284,8 @@ compserv CS_HIP(const vector<int> &g, const string &mem = "full_mem");
 compserv CS_GPU(const vector<int> &g, const string &mem = "full_mem");  // the reference's spelling, same service
 void build(model net, compserv cs, bool init_weights = true);
 void fuse(model net);  // Net::fuse: the fused inference plan (this backend's addition)
+void show_profile();   // src/apis/eddl.cpp:291-297: the host wall-clock profile of forward and of the functions it called
+void reset_profile();
 void set_mode(model net, int mode);
 void summary(model m);
 void load(model m, const string &fname, const string &format = "bin");

@@ -330,6 +330,7 @@ int main(int argc, char **argv) {
             delete t;
         }
         ofs.close();
+        show_profile();
         if (timed) {  // forwards with the input already on the device
             for (int i = 0; i < 5; i++) m->forward();
             const auto t0 = std::chrono::steady_clock::now();

@@ -148,6 +148,11 @@ def test_cpp_graphs_match_the_python_runner_bit_for_bit(hip, which, fused, tmp_p
     x.tofile(tmp_path / "x.raw")
     out = run_net_driver([("fused:" if fused else "") + which, tmp_path / "params.bin", tmp_path / "x.raw", tmp_path / "y.raw", batch, size] + extra)
     assert "FAILED" not in out and "ok  get_parameters / set_parameters round trip" in out and "ok  set_parameters with a missing layer" in out, out
+    # the reference's host profile (eddl::show_profile): forward is counted in both modes, the dispatchers of the layer walk
+    # only when the layers are walked
+    prof = {l.split(":")[0].strip("| "): int(l.split(":")[1].split("calls")[0]) for l in out.splitlines() if l.startswith("| ") and " calls," in l}
+    assert prof.get("forward", 0) >= 1, out
+    assert ("Conv2D" in prof) == (not fused), prof
     if fused:
         assert "ok  getOutput of a fused-away layer" in out, out
         steps = int([l for l in out.splitlines() if l.startswith("plan:")][0].split()[1])
