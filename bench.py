@@ -176,7 +176,7 @@ def oracle_parity(workload, device_output, max_images):
 RIDGE_FLOP_PER_BYTE = PEAK_FP32_MFMA_TFLOPS * 1e3 / PEAK_HBM_GBS  # 19.7: below it a layer is bound by HBM, not by the matrix cores
 
 
-def measure(hip, workload, steps, warmup, fused=True, graph=False):
+def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True):
     """Builds the workload, runs `warmup` + `steps` forwards with the input resident in HBM, then times every op.
     Returns (summary dict, per-op rows, device output of the last forward, model description)."""
     model, x, desc = build_workload(workload)
@@ -184,6 +184,17 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False):
     batch = x.shape[0]
     model.input_tensor().copy_from(x)  # input resident in HBM before the timed region
     hip.synchronize()
+    if tune:
+        # the library's plan search (the reference's cudnnFindConvolutionForwardAlgorithm on a layer's first forward): with the
+        # clocks warm, one forward in which every new convolution geometry is run under every launch plan; all of it
+        # before the timed region
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 0.1:
+            model.run()
+            hip.synchronize()
+        hip.conv_autotune(True)
+        model.run()
+        hip.synchronize()
     step = model.run
     if graph:
         model.capture()
@@ -282,6 +293,9 @@ def main():
     ap.add_argument("--no-workloads", action="store_true",
                     help="report the headline workload only (without it a default VGG-16 run also measures the other four "
                          "configurations, briefly, into the 'workloads' object of the JSON line)")
+    ap.add_argument("--no-tune", action="store_true",
+                    help="keep the launch planner's own choice for every convolution (without it the library searches the launch "
+                         "plans of every convolution geometry once, before the timed region: eddlhip_conv2d_autotune)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="after the timed region run one ReLU over 2^26 floats (reads 256 MiB, writes 256 MiB): the plain copy "
                          "kernel of known size that scales FETCH_SIZE / WRITE_SIZE counter readings")
@@ -292,7 +306,7 @@ def main():
     import eddl_amd
     hip = eddl_amd.Backend(0)
     hip.set_conv_algo(args.conv_algo)
-    summary, rows, out_host, desc = measure(hip, args.workload, args.steps, args.warmup, fused=not args.unfused, graph=args.graph)
+    summary, rows, out_host, desc = measure(hip, args.workload, args.steps, args.warmup, fused=not args.unfused, graph=args.graph, tune=not args.no_tune)
     batch = summary["batch"]
     ms_per_step = summary["ms_per_step"]
     roofline = summary["roofline"]
@@ -333,7 +347,8 @@ def main():
         "value": summary["value"], "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (mt19937 + Box-Muller: He-normal weights from the configuration's seed, U(0,1)/N(0,1) inputs from seed + 1000; resident in HBM)",
-        "config": {"workload": desc, "batch": batch, "fused": not args.unfused, "fused_ops": summary["fused_ops"], "graph_replay": bool(args.graph), "device": hip.name},
+        "config": {"workload": desc, "batch": batch, "fused": not args.unfused, "fused_ops": summary["fused_ops"], "graph_replay": bool(args.graph), "plan_search": not args.no_tune,
+                   "device": hip.name},
         "roofline": roofline,
         "hbm_bound_convs": summary["hbm_bound_convs"],
         "conv_total": summary["conv_total"],
@@ -353,7 +368,7 @@ def main():
     if args.workload == "vgg16" and not (args.no_workloads or args.unfused or args.graph):
         result["workloads"] = {}
         for w, (steps, warmup, parity_images) in OTHER_WORKLOADS.items():
-            sm, _, out_w, desc_w = measure(hip, w, steps, warmup)
+            sm, _, out_w, desc_w = measure(hip, w, steps, warmup, tune=not args.no_tune)
             entry = {"workload": desc_w, "value": sm["value"], "unit": "images/sec", "ms_per_step": sm["ms_per_step"], "steps": steps,
                      "warmup": warmup, "batch": sm["batch"], "dominant_kernel": sm["roofline"]["kernel"],
                      "frac": sm["roofline"]["frac"], "achieved_tflops": sm["roofline"]["achieved"],

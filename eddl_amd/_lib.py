@@ -59,6 +59,9 @@ PROTOTYPES = {
     "eddlhip_conv2d_force_plan": [c_int, c_int],
     "eddlhip_conv2d_profile": [c_int],
     "eddlhip_conv2d_profile_read": [intp, ctypes.POINTER(c_float)],
+    "eddlhip_conv2d_trace": [P, ctypes.c_longlong],
+    "eddlhip_conv2d_autotune": [c_int],
+    "eddlhip_conv2d_tuned_plans": [c_int],
     "eddlhip_batchnorm_inference": [c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, c_float],
     "eddlhip_relu": [c_int, P, P, c_size_t],
     "eddlhip_sigmoid": [c_int, P, P, c_size_t],

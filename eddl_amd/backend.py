@@ -264,6 +264,24 @@ class Backend:
         self._check(self.lib.eddlhip_conv2d_profile_read(ctypes.byref(n), ctypes.byref(ms)))
         return n.value, ms.value
 
+    def conv_autotune(self, on=True):
+        """Search the launch plans on the first call of every new convolution geometry (True), stop using what was found
+        (False), or also forget it (-1)."""
+        self._check(self.lib.eddlhip_conv2d_autotune(int(on)))
+
+    def conv_tuned_plans(self):
+        return self.lib.eddlhip_conv2d_tuned_plans(self.dev)
+
+    def conv_trace(self, workgroups):
+        """Per-workgroup timeline records of the next convolution launches (at most `workgroups` workgroups each);
+        returns the device tensor that receives them (two floats hold one 64-bit word), or switches tracing off with 0."""
+        if not workgroups:
+            self._check(self.lib.eddlhip_conv2d_trace(None, 0))
+            return None
+        buf = self.full((int(workgroups) * 16,), 0.0)
+        self._check(self.lib.eddlhip_conv2d_trace(buf.ptr, int(workgroups)))
+        return buf
+
     # ---- operators (names follow the reference's gpu_* functions)
     def fill_(self, A, v):
         self._check(self.lib.eddlhip_fill(self.dev, A.ptr, A.size, v))

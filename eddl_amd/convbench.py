@@ -3,6 +3,7 @@
     python3 -m eddl_amd.convbench layers  <shapes file | resnet50 | vgg16> [--reps R]
     python3 -m eddl_amd.convbench planfit <shapes file | resnet50 | vgg16> [--reps R]
     python3 -m eddl_amd.convbench one     N C H W Kf R S stride pad [flags] [--tile T --slices S] [--reps R]
+    python3 -m eddl_amd.convbench timeline N C H W Kf R S stride pad [flags] [--tile T --slices S]
 
 A shape line reads  N C H W Kf R S stride pad count [flags];  flags: b = inference BatchNorm in the epilogue, r = ReLU,
 s = residual add.  `count` is how often the layer occurs in the network (weights the totals).
@@ -12,6 +13,12 @@ layers   one row per layer: time per launch, TFLOP/s = 2 N Kf C R S P Q / time, 
 planfit  the planner's choice against every (tile family, K slices) plan forced through eddlhip_conv2d_force_plan: how far
          the planned launch is from the fastest forced one, per layer and summed over the list.
 one      a single layer, optionally with a forced plan.
+timeline one launch of a single layer (1x1, 2x2 or 3x3 filters) with eddlhip_conv2d_trace switched on: every workgroup
+         leaves four stamps of the device's 100 MHz clock (entry, first operands in LDS, end of the K loop, stores
+         drained) and the CU it ran on.  Printed: how long the three phases last per workgroup (shader cycles at the
+         engine clock the records themselves give), how many workgroups a CU holds and how many of them are inside their
+         K loop at a time (share of the launch), and the timeline of one CU.  A workgroup outside its K loop uses no
+         matrix instruction: the second histogram is the supply side of the matrix pipe.
 
 Launches repeat back to back on one stream between two events, so the figures include no host gaps; a layer timed this
 way runs somewhat slower than inside a network (the same launch forty times in a row keeps the chip at its power limit
@@ -175,9 +182,66 @@ def cmd_planfit(hip, source, reps):
     print("SUM planned %.1f us  fastest forced %.1f us  ratio %.3f" % (tot_auto, tot_best, tot_auto / tot_best))
 
 
+def cmd_timeline(hip, dims, flags, tile, slices):
+    layer = Layer(hip, dims, flags, np.random.default_rng(0))
+    hip.force_conv_plan(tile, slices)
+    us = layer.time_us(20, warm_seconds=0.2)
+    buf = hip.conv_trace(1 << 16)
+    try:
+        for _ in range(3):
+            layer.call()
+        hip.synchronize()
+    finally:
+        hip.conv_trace(0)
+        hip.force_conv_plan(-1, 1)
+    rec = buf.numpy().view(np.uint64).reshape(-1, 8)
+    rec = rec[rec[:, 0] != 0].astype(np.int64)
+    n = len(rec)
+    print("%s %s  %s  %.1f us per launch untraced, %d workgroups" % (" ".join(str(v) for v in dims), flags, hip.last_conv_kernel(), us, n))
+    if n == 0:
+        print("no records: the launch was not one of the traced kernels")
+        return
+    t = rec[:, 0:4] - rec[:, 0].min()
+    mhz = float(np.median((rec[:, 6] - rec[:, 5]) / np.maximum(t[:, 3] - t[:, 0], 1))) * 100.0
+    t = (t * (mhz / 100.0)).astype(np.int64)  # shader cycles
+    span = int(t[:, 3].max())
+    print("engine clock %.0f MHz (shader-clock difference over 100 MHz-clock difference, median over the workgroups); the launch "
+          "spans %d cycles = %.1f us with the stores drained" % (mhz, span, span / mhz))
+    phases = (("entry -> first operands in LDS", t[:, 1] - t[:, 0]), ("K loop", t[:, 2] - t[:, 1]), ("K loop end -> stores drained", t[:, 3] - t[:, 2]),
+              ("workgroup lifetime", t[:, 3] - t[:, 0]))
+    for name, v in phases:
+        print("  %-30s mean %7.0f  median %7.0f  p10 %7.0f  p90 %7.0f cycles  (mean %.2f us)" % (name, v.mean(), np.median(v), np.percentile(v, 10), np.percentile(v, 90), v.mean() / mhz))
+    cu = ((rec[:, 4] >> 8) & 0xff) | (((rec[:, 4] >> 32) & 0xf) << 8)  # CU, shader array and engine bits of HW_ID, XCC_ID above them
+    cus = np.unique(cu)
+    in_loop, resident = np.zeros(10), np.zeros(10)
+    per_cu = []
+    for c in cus:
+        tt = t[cu == c]
+        per_cu.append(len(tt))
+        ev = sorted([(r[0], 0, 1) for r in tt] + [(r[1], 1, 0) for r in tt] + [(r[2], -1, 0) for r in tt] + [(r[3], 0, -1) for r in tt])
+        a = b = last = 0
+        for when, da, db in ev:
+            in_loop[min(a, 9)] += when - last
+            resident[min(b, 9)] += when - last
+            a, b, last = a + da, b + db, when
+        in_loop[0] += span - last
+        resident[0] += span - last
+    print("%d CUs; workgroups per CU %.2f (min %d, max %d)" % (len(cus), np.mean(per_cu), min(per_cu), max(per_cu)))
+    print("share of the launch (%) by the number of a CU's workgroups that are     0     1     2     3     4     5     6     7     8    9+")
+    print("  resident                                                         " + " ".join("%5.1f" % v for v in resident / resident.sum() * 100))
+    print("  inside their K loop                                              " + " ".join("%5.1f" % v for v in in_loop / in_loop.sum() * 100))
+    c0 = cus[len(cus) // 2]
+    sel = np.where(cu == c0)[0]
+    sel = sel[np.argsort(t[sel, 0])]
+    print("one CU, thousands of cycles:   entry  K loop from      to  drained")
+    for i in sel:
+        print("                             %7.1f %12.1f %7.1f %8.1f" % tuple(t[i] / 1e3))
+    layer.close()
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("cmd", choices=["layers", "planfit", "one"])
+    ap.add_argument("cmd", choices=["layers", "planfit", "one", "timeline"])
     ap.add_argument("args", nargs="+")
     ap.add_argument("--reps", type=int, default=10)
     ap.add_argument("--tile", type=int, default=-1)
@@ -189,6 +253,8 @@ def main():
         cmd_layers(hip, a.args[0], a.reps)
     elif a.cmd == "planfit":
         cmd_planfit(hip, a.args[0], a.reps)
+    elif a.cmd == "timeline":
+        cmd_timeline(hip, [int(v) for v in a.args[:9]], a.args[9] if len(a.args) > 9 else "", a.tile, a.slices)
     else:
         dims = [int(v) for v in a.args[:9]]
         flags = a.args[9] if len(a.args) > 9 else ""

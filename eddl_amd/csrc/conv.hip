@@ -41,6 +41,8 @@
 // neighbouring pixel tiles for all channel tiles: the input slice they share stays in that
 // XCD's L2.
 #include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
 
 #include <mutex>
 #include <utility>
@@ -104,7 +106,25 @@ struct ConvParams {
     float *partial;
     // conv_gen_kernel only: one entry per tap of the padded K range (tap_table_kernel)
     const int32x4 *taps;
+    // eddlhip_conv2d_trace: eight 64-bit words per workgroup (see trace_mark), or nullptr
+    unsigned long long *trace;
 };
+
+// Timeline of a workgroup for eddlhip_conv2d_trace: words 0..3 = the device's constant 100 MHz clock at the marks (entry,
+// operands of the first K-step in LDS, end of the K loop, end of the kernel with its stores drained), word 4 = where the
+// workgroup runs (HW_ID register in the low half, XCC_ID in the high half), words 5 and 6 = the shader clock at the
+// first and the last mark (their difference over that of words 0 and 3 is the engine clock).
+__device__ __forceinline__ void trace_mark(const ConvParams &p, int slot) {
+    if (p.trace != nullptr && threadIdx.x == 0) {
+        unsigned long long *w = p.trace + (size_t)blockIdx.x * 8;
+        if (slot == 0) {
+            w[4] = (unsigned long long)__builtin_amdgcn_s_getreg(0xF804) | ((unsigned long long)__builtin_amdgcn_s_getreg(0xF814) << 32);
+            w[5] = __builtin_readcyclecounter();
+        }
+        if (slot == 3) w[6] = __builtin_readcyclecounter();
+        w[slot] = __builtin_amdgcn_s_memrealtime();
+    }
+}
 
 // The fused tail of a Conv -> BatchNorm(inference) -> Add -> ReLU chain; every step rounded
 // to fp32, no contraction.  sd is sqrtf(var + eps) for channel k (unused without batch-norm).
@@ -254,7 +274,7 @@ __device__ __forceinline__ void stage_channel_constants(const ConvParams &p, flo
 // the channel constants of four consecutive rows come from LDS in one read; which of batch norm,
 // affine, residual and ReLU apply is decided once per group of four rows (the flags are the same for
 // every lane) instead of once per value.  The arithmetic per value is that of store_tile, step by step.
-template <int TM, int TN, int BM>
+template <int TM, int TN, int BM, bool HAS_RES>
 __device__ __forceinline__ void store_tile_inside(const ConvParams &p, floatx16 (&acc)[TM][TN], const float *epi, int m0, int m_local,
                                                   int n_base, int lane) {
     const int half = lane >> 5;
@@ -271,7 +291,8 @@ __device__ __forceinline__ void store_tile_inside(const ConvParams &p, floatx16 
         rptr[tn] = p.residual + idx;  // not dereferenced without a residual
     }
     const bool has_bias = p.bias != nullptr, has_bn = p.bn_mean != nullptr, affine = p.bn_g != nullptr;
-    const bool has_res = p.residual != nullptr, relu = p.relu != 0, stream_out = p.stream_out != 0;
+    constexpr bool has_res = HAS_RES;
+    const bool relu = p.relu != 0, stream_out = p.stream_out != 0;
 #pragma unroll
     for (int tm = 0; tm < TM; tm++) {
 #pragma unroll
@@ -279,7 +300,7 @@ __device__ __forceinline__ void store_tile_inside(const ConvParams &p, floatx16 
             const int row0 = m_local + tm * 32 + 8 * q4 + 4 * half;
             const size_t roff = (size_t)(tm * 32 + 8 * q4) * plane;
             float res[4][TN];
-            if (has_res) {
+            if constexpr (has_res) {
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -313,7 +334,7 @@ __device__ __forceinline__ void store_tile_inside(const ConvParams &p, floatx16 
                         for (int tn = 0; tn < TN; tn++) x[j][tn] = __fadd_rn(__fmul_rn(x[j][tn], g[j]), b[j]);
                 }
             }
-            if (has_res) {
+            if constexpr (has_res) {
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -346,13 +367,27 @@ __device__ __forceinline__ void store_tile_inside(const ConvParams &p, floatx16 
 // `epi` holds the tile's channel constants (stage_channel_constants); m_local is the first of the
 // wavefront's rows within the tile.  The residual values of a 32-row block are all requested
 // before the first of them is used, so their latencies overlap.
+// (The residual's presence is a template parameter of the two bodies so that the loads of the residual values and their
+// uses sit in one branch: a kernel that goes on to further work after a tile then carries no load that looks pending.)
+template <int TM, int TN, int BM, bool HAS_RES>
+__device__ __forceinline__ void store_tile_edge(const ConvParams &p, floatx16 (&acc)[TM][TN], const float *epi, int m0, int m_local, int n_base,
+                                                int lane);
+
 template <int TM, int TN, int BM>
 __device__ __forceinline__ void store_tile(const ConvParams &p, floatx16 (&acc)[TM][TN], const float *epi, int m0, int m_local, int n_base,
                                            int lane) {
     if (m0 + m_local + TM * 32 <= p.Kf && (long long)n_base + TN * 32 <= p.npix) {
-        store_tile_inside<TM, TN, BM>(p, acc, epi, m0, m_local, n_base, lane);
+        if (p.residual != nullptr) store_tile_inside<TM, TN, BM, true>(p, acc, epi, m0, m_local, n_base, lane);
+        else store_tile_inside<TM, TN, BM, false>(p, acc, epi, m0, m_local, n_base, lane);
         return;
     }
+    if (p.residual != nullptr) store_tile_edge<TM, TN, BM, true>(p, acc, epi, m0, m_local, n_base, lane);
+    else store_tile_edge<TM, TN, BM, false>(p, acc, epi, m0, m_local, n_base, lane);
+}
+
+template <int TM, int TN, int BM, bool HAS_RES>
+__device__ __forceinline__ void store_tile_edge(const ConvParams &p, floatx16 (&acc)[TM][TN], const float *epi, int m0, int m_local, int n_base,
+                                                int lane) {
     size_t obase[TN];
     bool nok[TN];
 #pragma unroll
@@ -364,13 +399,13 @@ __device__ __forceinline__ void store_tile(const ConvParams &p, floatx16 (&acc)[
         const unsigned pq = nc - img * (unsigned)p.PQ;
         obase[tn] = (size_t)img * p.Kf * p.PQ + pq;
     }
-    const bool has_res = p.residual != nullptr;
+    constexpr bool has_res = HAS_RES;
 #pragma unroll
     for (int tm = 0; tm < TM; tm++) {
 #pragma unroll
         for (int vh = 0; vh < 16; vh += 8) {  // eight rows at a time: their residual loads are in flight together
             float res[8][TN];
-            if (has_res) {
+            if constexpr (has_res) {
 #pragma unroll
                 for (int vv = 0; vv < 8; vv++) {
                     const int v = vh + vv;
@@ -397,7 +432,7 @@ __device__ __forceinline__ void store_tile(const ConvParams &p, floatx16 (&acc)[
                         x = __fdiv_rn(__fsub_rn(x, mean), sd);
                         if (p.bn_g) x = __fadd_rn(__fmul_rn(x, g), b);
                     }
-                    if (has_res) x = __fadd_rn(x, res[vv][tn]);
+                    if constexpr (has_res) x = __fadd_rn(x, res[vv][tn]);
                     if (p.relu) x = x > 0.0f ? x : 0.0f;
                     if (mok && nok[tn]) p.O[obase[tn] + (size_t)(m0 + ml) * p.PQ] = x;
                 }
@@ -458,6 +493,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     const int wm = wave / WN, wn = wave % WN;
     int m_tile, n_tile, local_tile, slice;
     bool split;
+    trace_mark(p, 0);
     tile_of_block(p, m_tile, n_tile, local_tile, slice, split);
     const int step_lo = split ? slice * p.slice_steps : 0;
     const int step_hi = split ? min(step_lo + p.slice_steps, p.nsteps) : p.nsteps;
@@ -563,6 +599,20 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     };
     // gather of one step; `checked` adds the test for channels past C (last step of an odd channel count)
     auto load_b = [&](int step, lds_float *bs, bool checked) {
+        if constexpr (DIRECT) {
+            // one input tensor and every channel of the step exists (nearly every step of every layer): the channel's
+            // offset advances by one plane per load and nothing is selected
+            if (!checked && p.Csplit == p.C) {
+                int soff = (step * CPB + cg * CPW) * HW4;
+#pragma unroll
+                for (int jc = 0; jc < CPW; jc++) {
+#pragma unroll
+                    for (int t = 0; t < RS; t++) lds_dma_b32(dma_in, bs + ((cg * CPW + jc) * RS + t) * LDB + seg * 64, voff[t], soff);
+                    soff += HW4;
+                }
+                return;
+            }
+        }
 #pragma unroll
         for (int jc = 0; jc < CPW; jc++) {
             const int cl = cg * CPW + jc;
@@ -615,18 +665,18 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         // operands of tap pair ks+1 are read from LDS while the MFMAs of pair ks run
         float a[2][TM], b[2][TN];
 #pragma unroll
-        for (int tm = 0; tm < TM; tm++) a[0][tm] = a_cur[a_off + tm * 32];
+        for (int tm = 0; tm < TM; tm++) a[0][tm] = (a_cur[a_off + tm * 32]);
 #pragma unroll
-        for (int tn = 0; tn < TN; tn++) b[0][tn] = b_cur[b_off + tn * 32];
+        for (int tn = 0; tn < TN; tn++) b[0][tn] = (b_cur[b_off + tn * 32]);
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // the two reads of pair 0
 #pragma unroll
         for (int ks = 0; ks < BK / 2; ks++) {
             const int cur = ks & 1, nxt = cur ^ 1;
             if (ks + 1 < BK / 2) {
 #pragma unroll
-                for (int tm = 0; tm < TM; tm++) a[nxt][tm] = a_cur[(ks + 1) * 2 * LDA + a_off + tm * 32];
+                for (int tm = 0; tm < TM; tm++) a[nxt][tm] = (a_cur[(ks + 1) * 2 * LDA + a_off + tm * 32]);
 #pragma unroll
-                for (int tn = 0; tn < TN; tn++) b[nxt][tn] = b_cur[(ks + 1) * 2 * LDB + b_off + tn * 32];
+                for (int tn = 0; tn < TN; tn++) b[nxt][tn] = (b_cur[(ks + 1) * 2 * LDB + b_off + tn * 32]);
             }
 #pragma unroll
             for (int tm = 0; tm < TM; tm++)
@@ -650,6 +700,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     store_b(bs_of(0));
     if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's LDS-direct loads have landed
     __syncthreads();
+    trace_mark(p, 1);
 
     for (int step = step_lo; step < step_hi; step++) {
         const int buf = (step - step_lo) & 1;
@@ -660,6 +711,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         __syncthreads();
     }
 
+    trace_mark(p, 2);
     if (split) {
         store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
     } else {
@@ -667,6 +719,11 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         put_channel_constants<BM>(epi, chan, tid);
         __syncthreads();
         store_tile<TM, TN, BM>(p, acc, epi, m0, wm * TM * 32, (int)n0 + wn * TN * 32, lane);
+    }
+    if (p.trace != nullptr) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        trace_mark(p, 3);
     }
 }
 
@@ -1054,6 +1111,17 @@ int prof_end(hipStream_t st) {
 thread_local char g_last_kernel[128] = "";
 int g_split = 1;  // divide the tiles left over after a whole number per CU along K (set_algo 5 turns it off)
 int g_force_tile = -1, g_force_slices = -1;  // eddlhip_conv2d_force_plan
+unsigned long long *g_trace = nullptr;       // eddlhip_conv2d_trace
+long long g_trace_wgs = 0;
+
+// eddlhip_conv2d_autotune: launch plans found by measurement, by device and geometry.  The epilogue is not part of the
+// key: a convolution sums in the same order whether its batch norm runs fused or as a launch of its own.
+struct TunedPlan {
+    int key[17];       // N C H W Kf R S sr sc pad_top pad_left P Q two-tensor uh uw direct
+    int tile, slices;  // tile -1: the planner's own choice was the fastest
+};
+bool g_autotune = false, g_tuning = false;
+std::vector<TunedPlan> g_tuned[EDDLHIP_MAX_DEVICES];
 
 struct Variant {
     const char *name;
@@ -1325,6 +1393,25 @@ int eddlhip_conv2d_force_plan(int tile, int slices) {
     return 0;
 }
 
+int eddlhip_conv2d_trace(unsigned long long *words, long long workgroups) {
+    EH_REQUIRE(workgroups >= 0 && (words != nullptr || workgroups == 0), "conv2d_trace: bad buffer");
+    g_trace = workgroups > 0 ? words : nullptr;
+    g_trace_wgs = workgroups;
+    return 0;
+}
+
+int eddlhip_conv2d_autotune(int on) {
+    g_autotune = on != 0;
+    if (on < 0)
+        for (auto &t : g_tuned) t.clear();
+    return 0;
+}
+
+int eddlhip_conv2d_tuned_plans(int dev) {
+    EH_REQUIRE(dev >= 0 && dev < EDDLHIP_MAX_DEVICES, "conv2d_tuned_plans: bad device %d", dev);
+    return (int)g_tuned[dev].size();
+}
+
 int eddlhip_conv2d_set_algo(int algo) {
     EH_REQUIRE(algo >= 0 && algo <= 6, "conv2d_set_algo: unknown algorithm %d", algo);
     if (algo == 5 || algo == 6) {
@@ -1436,6 +1523,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     p.Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
     p.in_bytes = p.wp_bytes = 0;
     p.main_tiles = 0; p.nslices = 1; p.slice_steps = 0; p.partial = nullptr;
+    p.trace = nullptr;
 
     if (g_algo == 2) {
         size_t total = (size_t)p.npix * Kf;
@@ -1487,6 +1575,72 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     const int chunk_imgs = (int)((N < max_imgs) ? N : max_imgs);
     Plan plan = plan_conv(family, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu, g_split != 0);
     if (g_force_tile >= 0) plan = forced_plan(family, g_force_tile, g_force_slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
+    if (g_autotune && !g_tuning && g_force_tile < 0 && g_algo == 0 && g_split != 0) {
+        const int key[17] = {N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, two ? 1 : 0, uh, uw, direct};
+        const TunedPlan *found = nullptr;
+        for (const TunedPlan &t : g_tuned[dev])
+            if (memcmp(t.key, key, sizeof(key)) == 0) found = &t;
+        if (found == nullptr && !no_alloc && !state(dev).capturing && !g_prof_on) {
+            // First call with this geometry: run every plan on the call's own tensors (each writes the same output, up to
+            // the rounding of its summation order) and keep the fastest.  The planner's choice stays unless another plan
+            // beats it by more than the noise of the measurement.
+            TunedPlan best;
+            memcpy(best.key, key, sizeof(key));
+            best.tile = -1;
+            best.slices = 1;
+            hipEvent_t e0, e1;
+            EH_TRY_HIP(hipEventCreate(&e0));
+            EH_TRY_HIP(hipEventCreate(&e1));
+            auto measure = [&](int tile, int slices, float *ms) -> int {
+                g_force_tile = tile;
+                g_force_slices = slices;
+                int rc = 0;
+                for (int rep = 0; rep < 4 && rc == 0; rep++) {  // the first launch is not timed
+                    if (rep == 1) rc = hipEventRecord(e0, st) == hipSuccess ? 0 : EDDLHIP_EHIP;
+                    if (rc == 0)
+                        rc = conv2d_fwd_impl(false, dev, I, I2, uh, uw, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
+                                             bn_mean, bn_var, bn_eps, residual, relu);
+                }
+                g_force_tile = -1;
+                g_force_slices = -1;
+                if (rc != 0) return rc;
+                if (hipEventRecord(e1, st) != hipSuccess || hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(ms, e0, e1) != hipSuccess)
+                    return EDDLHIP_EHIP;
+                return 0;
+            };
+            g_tuning = true;
+            float planned_ms = 0.0f, best_ms = 0.0f;
+            int rc = measure(-1, -1, &planned_ms);
+            best_ms = planned_ms;
+            static const int kSlices[8] = {1, 2, 3, 4, 6, 8, 12, 16};
+            for (int tile = 0; tile < 4 && rc == 0; tile++) {
+                int last_slices = 0;
+                for (int si = 0; si < 8 && rc == 0; si++) {
+                    const Plan fp = forced_plan(family, tile, kSlices[si], Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
+                    if (fp.nslices == last_slices) continue;  // the same plan as the one before
+                    last_slices = fp.nslices;
+                    float ms = 0.0f;
+                    if (measure(tile, kSlices[si], &ms) != 0) continue;  // a plan that does not apply here
+                    if (ms < best_ms && ms < 0.98f * planned_ms) {
+                        best_ms = ms;
+                        best.tile = tile;
+                        best.slices = kSlices[si];
+                    }
+                }
+            }
+            g_tuning = false;
+            (void)hipEventDestroy(e0);
+            (void)hipEventDestroy(e1);
+            if (rc != 0) return rc;
+            if (getenv("EDDLHIP_TUNE_VERBOSE"))
+                fprintf(stderr, "tune %d %d %d %d -> %d %dx%d s%d: planned %.1f us, best %.1f us (tile %d x %d slices)\n", N, C, H, W, Kf, R, S, sr,
+                        planned_ms * 1e3f / 3, best_ms * 1e3f / 3, best.tile, best.slices);
+            g_tuned[dev].push_back(best);
+            found = &g_tuned[dev].back();
+        }
+        if (found != nullptr && found->tile >= 0)
+            plan = forced_plan(family, found->tile, found->slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
+    }
     const Variant *v = &family[plan.tile];
     const int bk = v->cpb ? v->cpb * R * S : 16;
     p.nsteps = plan.nsteps;
@@ -1559,6 +1713,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
         q.main_tiles = (int)main_tiles;
         q.nslices = split_tiles > 0 ? nslices : 1;
         q.slice_steps = split_tiles > 0 ? slice_steps : p.nsteps;
+        q.trace = (g_trace != nullptr && main_tiles + split_tiles * q.nslices <= g_trace_wgs) ? g_trace : nullptr;
         EH_TRY(prof_begin(st));
         hipLaunchKernelGGL(v->kernel, dim3((unsigned)(main_tiles + split_tiles * q.nslices)), dim3(256), 0, st, q);
         EH_CHECK_LAUNCH();

@@ -108,40 +108,6 @@ __global__ __launch_bounds__(TPB) void bn_inference_kernel(int plane0, int z, in
     }
 }
 
-// Planes of 16 .. 4095 elements whose length is a multiple of four (ResNet's 56x56 .. 14x14): a workgroup takes ONE
-// channel and a group of images, so the channel's constants (one square root included) are worked out once per
-// workgroup instead of once per float4, and the loop has no division.  Threads are laid out LX x LY with LX the power of
-// two that covers a plane's float4s (at most 256): LY images are in flight at a time.  Same operations per element.
-__global__ __launch_bounds__(TPB) void bn_inference_channel_kernel(int b, int z, int rc4, int lx_log2, int imgs_per_block,
-                                                                   const float *__restrict__ in, float *__restrict__ out,
-                                                                   float *__restrict__ opa, const float *__restrict__ gmean,
-                                                                   const float *__restrict__ gvar, const float *__restrict__ g,
-                                                                   const float *__restrict__ bb, float *__restrict__ variance, float eps) {
-    const int c = blockIdx.x;
-    const float sd = sqrtf(__fadd_rn(gvar[c], eps));
-    const float mean = gmean[c];
-    const bool affine = g != nullptr;
-    const float gg = affine ? g[c] : 1.0f, bc = affine ? bb[c] : 0.0f;
-    if (blockIdx.y == 0 && threadIdx.x == 0) variance[c] = sd;
-    const int lx = 1 << lx_log2, ly = TPB >> lx_log2;
-    const int tx = threadIdx.x & (lx - 1), ty = threadIdx.x >> lx_log2;
-    const int img0 = blockIdx.y * imgs_per_block, img1 = min(img0 + imgs_per_block, b);
-    auto norm = [&](float x) -> float { return __fdiv_rn(__fsub_rn(x, mean), sd); };
-    auto aff = [&](float o) -> float { return __fadd_rn(__fmul_rn(o, gg), bc); };
-    for (int img = img0 + ty; img < img1; img += ly) {
-        const size_t base4 = ((size_t)img * z + c) * rc4;
-        for (int j = tx; j < rc4; j += lx) {
-            const float4 x = reinterpret_cast<const float4 *>(in)[base4 + j];
-            float4 o = make_float4(norm(x.x), norm(x.y), norm(x.z), norm(x.w));
-            if (affine) {
-                if (opa) reinterpret_cast<float4 *>(opa)[base4 + j] = o;
-                o = make_float4(aff(o.x), aff(o.y), aff(o.z), aff(o.w));
-            }
-            reinterpret_cast<float4 *>(out)[base4 + j] = o;
-        }
-    }
-}
-
 // Small planes (a 7x7 plane would leave most of a workgroup idle above): one float4 of the whole tensor per
 // thread, whatever plane it falls into.  A float4 may cross from one plane into the next (planes of at
 // least 4 elements: at most one crossing), so the constants of both channels are at hand.  Same operations
@@ -432,23 +398,6 @@ int eddlhip_batchnorm_inference(int dev, int b, int z, int rc, const float *inpu
     EH_TRY(use_device(dev));
     const bool all_aligned = aligned16(input) && aligned16(output) && (!opa || aligned16(opa));
     long long planes = (long long)b * z;
-    if (rc >= 16 && rc % 4 == 0 && rc < kBnFlatBelow && all_aligned && z <= 65535 * 32) {
-        const int rc4 = rc / 4;
-        int lx_log2 = 2;
-        while ((1 << lx_log2) < rc4 && lx_log2 < 8) lx_log2++;
-        // enough workgroups for eight per CU, each with at least a few images so that the constants pay off
-        const long long want = 8LL * state(dev).num_cu;
-        long long groups = (want + z - 1) / z;
-        if (groups > b) groups = b;
-        if (groups < 1) groups = 1;
-        const int per = (int)((b + groups - 1) / groups);
-        groups = (b + per - 1) / per;
-        EH_REQUIRE(groups <= 65535, "batchnorm: too many image groups");
-        hipLaunchKernelGGL(bn_inference_channel_kernel, dim3((unsigned)z, (unsigned)groups), dim3(TPB), 0, state(dev).stream, b, z, rc4,
-                           lx_log2, per, input, output, opa, global_mean, global_variance, affine_g, affine_b, variance, epsilon);
-        EH_CHECK_LAUNCH();
-        return 0;
-    }
     if (rc >= 4 && rc < kBnFlatBelow && all_aligned) {
         const size_t total = (size_t)planes * rc;
         const unsigned grid = eh_blocks(total / 4 + 1, TPB, 1u << 20);

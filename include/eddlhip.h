@@ -213,6 +213,21 @@ int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const fl
 int eddlhip_conv2d_set_algo(int algo);
 const char *eddlhip_conv2d_last_kernel(void);
 
+/* Plan search on first use.  eddlhip_conv2d_autotune(1): from now on the first eddlhip_conv2d_fwd* call with a geometry the
+ * device has not seen (N, C, H, W, Kf, R, S, strides, paddings, output size, input form) runs that convolution under
+ * every launch plan (tile shape x K slices, three timed launches each, on the call's own tensors) and remembers the
+ * fastest; later calls with that geometry take it.  The reference does the same on a layer's first forward, with
+ * cudnnFindConvolutionForwardAlgorithm (src/hardware/gpu/nn/gpu_conv.cu:42-66, 211-213).  The epilogue is not part of
+ * the geometry, so a layer computes the same sums whether its batch norm, residual and ReLU are fused or not; a plan
+ * that divides tiles along K adds its slices in another order than an undivided one, so results with and without the
+ * search agree to the convolution's tolerance, not bit for bit.  Calls that must not allocate or wait (graph
+ * recording, eddlhip_conv2d_fwd_noalloc, eddlhip_conv2d_profile collecting) do not search; they use what was found.
+ * eddlhip_conv2d_autotune(0) stops searching and using the table, eddlhip_conv2d_autotune(-1) also empties it.
+ * eddlhip_conv2d_tuned_plans(dev) = number of geometries in the table.  With EDDLHIP_TUNE_VERBOSE set in the environment every
+ * search prints one line to stderr (geometry, the planner's time, the best time and plan). */
+int eddlhip_conv2d_autotune(int on);
+int eddlhip_conv2d_tuned_plans(int dev);
+
 /* Overrides the launch planner of the MFMA kernels (tuning and tests): tile = 0 (128x128 outputs per
  * workgroup), 1 (64x128), 2 (64x64), 3 (32x128) or -1 to give the choice back to the planner;
  * slices = number of K slices the tiles left over after a whole number per CU are divided into
@@ -242,6 +257,14 @@ int eddlhip_conv2d_uncache_filters(int dev, const float *K);
  * sum of their durations; eddlhip_conv2d_profile(0) stops collecting.  Either call of
  * eddlhip_conv2d_profile forgets what was collected before. */
 int eddlhip_conv2d_profile(int collect);
+/* Measurement hook (no counterpart in the reference): while `words` (device memory, 8 x workgroups 64-bit words) is
+ * set, every launch of a compile-time-filter-shape MFMA kernel (1x1, 2x2, 3x3) of at most `workgroups` workgroups
+ * writes one record per workgroup, indexed by workgroup id: words 0..3 = the device's constant 100 MHz clock at entry,
+ * when the operands of the first K-step are in LDS, at the end of the K loop and at the end of the kernel with its
+ * stores drained (tracing adds that wait); word 4 = the HW_ID register (low half: wavefront slot, SIMD, CU, shader
+ * engine) and the XCC_ID register (high half); words 5 and 6 = the shader clock at the first and the last mark.
+ * A later launch overwrites the records.  eddlhip_conv2d_trace(NULL, 0) switches it off. */
+int eddlhip_conv2d_trace(unsigned long long *words, long long workgroups);
 int eddlhip_conv2d_profile_read(int *launches, float *total_ms);
 
 /* ------------------------------------------------------------------ batch normalisation (inference)

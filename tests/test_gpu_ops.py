@@ -678,3 +678,70 @@ def test_device_probes_report_plausible_rates(hip):
         hip.probe_hbm(1000)
     mean, best, worst = hip.probe_mfma_f32(vary_operands=True, launches=3)
     assert 50.0 < worst <= mean <= best < 200.0
+
+
+def test_conv2d_trace_records_one_timeline_per_workgroup(hip):
+    """The measurement hook writes, per workgroup, four time stamps in order and where it ran; the output is unchanged."""
+    rng = np.random.default_rng(5)
+    x = hip.array(rng.standard_normal((8, 64, 28, 28), dtype=np.float32))
+    w = hip.array((rng.standard_normal((64, 64, 3, 3)) * 0.05).astype(np.float32))
+    O = hip.empty((8, 64, 28, 28))
+    hip.conv2D(x, w, None, O, 1, 1, 1, 1, relu=True)
+    plain = O.numpy()
+    buf = hip.conv_trace(4096)
+    try:
+        hip.conv2D(x, w, None, O, 1, 1, 1, 1, relu=True)
+        hip.synchronize()
+    finally:
+        hip.conv_trace(0)
+    assert np.array_equal(O.numpy(), plain)
+    rec = buf.numpy().view(np.uint64).reshape(-1, 8)
+    rec = rec[rec[:, 0] != 0].astype(np.int64)
+    assert len(rec) >= 8 * 28 * 28 // 128        # at least one workgroup per 64 x 128 tile of the largest tile shape
+    t = rec[:, 0:4]
+    assert np.all(np.diff(t, axis=1) >= 0)       # entry <= first operands in LDS <= end of the K loop <= stores drained
+    assert np.all(t[:, 3] - t[:, 0] < 100_000_000)   # under a second of the 100 MHz clock
+    assert np.all(rec[:, 6] > rec[:, 5])         # the shader clock advanced
+    xcd = (rec[:, 4] >> 32) & 0xf
+    assert len(np.unique(xcd)) == 8              # workgroups were dealt over all eight XCDs
+    hip.conv2D(x, w, None, O, 1, 1, 1, 1, relu=True)   # switched off again: nothing is written
+    hip.fill_(buf, 0.0)
+    hip.conv2D(x, w, None, O, 1, 1, 1, 1, relu=True)
+    hip.synchronize()
+    assert not buf.numpy().any()
+
+
+def test_conv2d_autotune_searches_once_per_geometry_and_stays_within_tolerance(hip, oracle):
+    """With the plan search on, the first call of a geometry measures the launch plans and later calls reuse the choice;
+    the result stays within the convolution's tolerance of the oracle and is the same from call to call, fused or not."""
+    rng = np.random.default_rng(11)
+    N, C, H, W, Kf = 8, 64, 28, 28, 64
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    w = (rng.standard_normal((Kf, C, 3, 3)) * 0.05).astype(np.float32)
+    g, b = rng.uniform(0.8, 1.2, Kf).astype(np.float32), (rng.standard_normal(Kf) * 0.1).astype(np.float32)
+    mean, var = (rng.standard_normal(Kf) * 0.1).astype(np.float32), rng.uniform(0.5, 1.5, Kf).astype(np.float32)
+    dx, dw = hip.array(x), hip.array(w)
+    bn = (hip.array(g), hip.array(b), hip.array(mean), hip.array(var), 1e-5)
+    O = hip.empty((N, Kf, H, W))
+    hip.conv_autotune(-1)
+    try:
+        hip.conv_autotune(True)
+        before = hip.conv_tuned_plans()
+        hip.conv2D(dx, dw, None, O, 1, 1, 1, 1)
+        assert hip.conv_tuned_plans() == before + 1
+        first = O.numpy()
+        hip.conv2D(dx, dw, None, O, 1, 1, 1, 1)
+        assert hip.conv_tuned_plans() == before + 1          # same geometry: no second search
+        assert np.array_equal(O.numpy(), first)
+        ref = oracle.conv2d(x, w, None, (1, 1), 1, 1, H, W, algo="im2col")
+        assert np.all(np.abs(first - ref) <= 1e-5 * float(np.abs(ref).max()) + 1e-4 * np.abs(ref))
+        # the epilogue is not part of the geometry: conv + stand-alone batch norm == the fused call, bit for bit
+        Y, opa, sd = hip.empty((N, Kf, H, W)), hip.empty((N, Kf, H, W)), hip.empty((Kf,))
+        hip.batchnorm_inference(O, Y, opa, bn[2], bn[3], bn[0], bn[1], sd, 1e-5)
+        F = hip.empty((N, Kf, H, W))
+        hip.conv2D(dx, dw, None, F, 1, 1, 1, 1, bn=bn)
+        assert hip.conv_tuned_plans() == before + 1
+        assert np.array_equal(F.numpy(), Y.numpy())
+    finally:
+        hip.conv_autotune(-1)
+    assert hip.conv_tuned_plans() == 0
