@@ -694,8 +694,15 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         }
     };
 
+    // A K range of exactly two steps (three or four input channels under a 3x3 filter) fits the two buffers: both are
+    // requested before the first wait, and the loop then runs without a trip to memory between its two steps.
+    const bool both = DIRECT && step_hi - step_lo == 2;
     load_a(step_lo, as_of(0));
     load_b(step_lo, bs_of(0), step_lo >= full_steps);
+    if (both) {
+        load_a(step_lo + 1, as_of(1));
+        load_b(step_lo + 1, bs_of(1), step_lo + 1 >= full_steps);
+    }
     store_a(as_of(0));
     store_b(bs_of(0));
     if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's LDS-direct loads have landed
@@ -704,7 +711,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
 
     for (int step = step_lo; step < step_hi; step++) {
         const int buf = (step - step_lo) & 1;
-        do_step(as_of(buf), bs_of(buf), as_of(buf ^ 1), bs_of(buf ^ 1), step, step + 1 < step_hi);
+        do_step(as_of(buf), bs_of(buf), as_of(buf ^ 1), bs_of(buf ^ 1), step, step + 1 < step_hi && !both);
         // The barrier publishes the next buffer to the other wavefronts, so this wavefront's
         // LDS-direct loads into it must be complete first.
         if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);

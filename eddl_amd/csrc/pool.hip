@@ -236,6 +236,93 @@ __global__ __launch_bounds__(TPB) void maxpool_3x3s2_kernel(const float *__restr
     }
 }
 
+// The same window on an even number of output rows: a thread produces a 2 x 2 patch of outputs (rows 2h, 2h+1) from five
+// input rows instead of two times three - the row the two windows share is loaded once - with five float4 loads in
+// flight.  Per output the scan order and the strict '>' are those of the kernel above.
+template <int PL>
+__global__ __launch_bounds__(TPB) void maxpool_3x3s2_rows_kernel(const float *__restrict__ I, float *__restrict__ O,
+                                                                 float *__restrict__ indX, float *__restrict__ indY,
+                                                                 size_t total_quads, int H, int W, int LP, int LQ, int pt) {
+    constexpr float OUTSIDE = -3.402823466e+38f;
+    const int LQ2 = LQ / 2, LP2 = LP / 2, lane = threadIdx.x & 63;
+    size_t t0 = (size_t)blockIdx.x * TPB + threadIdx.x, stride = (size_t)gridDim.x * TPB;
+    const size_t wave_first = t0 - lane;
+    for (size_t tw = wave_first; tw < total_quads; tw += stride) {
+        const size_t tt = tw + lane;
+        const bool live = tt < total_quads;
+        const size_t t = live ? tt : total_quads - 1;
+        const int m = (int)(t % LQ2);
+        const size_t r = t / LQ2;
+        const int oh = (int)(r % LP2);
+        const size_t plane = r / LP2;
+        const float *img = I + plane * (size_t)H * W;
+        const int i = 4 * oh - pt;  // first input row of the upper window
+        float4 c[5];
+        float e[5];
+#pragma unroll
+        for (int ki = 0; ki < 5; ki++) {
+            const int py = i + ki;
+            const bool rowin = (unsigned)py < (unsigned)H;
+            c[ki] = rowin ? *reinterpret_cast<const float4 *>(img + (size_t)py * W + 4 * m) : make_float4(OUTSIDE, OUTSIDE, OUTSIDE, OUTSIDE);
+        }
+#pragma unroll
+        for (int ki = 0; ki < 5; ki++) {
+            const int py = i + ki;
+            const bool rowin = (unsigned)py < (unsigned)H;
+            if (PL == 1) {
+                const float nb = __shfl_up(c[ki].w, 1, 64);
+                const bool own = lane == 0 || m == 0;
+                e[ki] = own ? ((rowin && m > 0) ? img[(size_t)py * W + 4 * m - 1] : OUTSIDE) : nb;
+            } else {
+                const float nb = __shfl_down(c[ki].x, 1, 64);
+                const bool own = lane == 63 || m == LQ2 - 1;
+                e[ki] = own ? ((rowin && 4 * m + 4 < W) ? img[(size_t)py * W + 4 * m + 4] : OUTSIDE) : nb;
+            }
+        }
+        const int j0 = 4 * m - PL;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {  // output rows 2*oh + half: input rows i + 2*half .. i + 2*half + 2
+            const size_t p = (plane * LP + 2 * oh + half) * LQ + 2 * m;
+            float2 o, ix, iy;
+            {
+                float mx = LOWEST, fx = 0.f, fy = 0.f;
+                bool found = false;
+#pragma unroll
+                for (int kk = 0; kk < 3; kk++) {
+                    const int ki = 2 * half + kk;
+                    const float w0 = PL ? e[ki] : c[ki].x, w1 = PL ? c[ki].x : c[ki].y, w2 = PL ? c[ki].y : c[ki].z;
+                    if (w0 > mx) { mx = w0; fx = (float)j0; fy = (float)(i + ki); found = true; }
+                    if (w1 > mx) { mx = w1; fx = (float)(j0 + 1); fy = (float)(i + ki); found = true; }
+                    if (w2 > mx) { mx = w2; fx = (float)(j0 + 2); fy = (float)(i + ki); found = true; }
+                }
+                o.x = mx;
+                if (!found && live) { fx = indX[p]; fy = indY[p]; }
+                ix.x = fx; iy.x = fy;
+            }
+            {
+                float mx = LOWEST, fx = 0.f, fy = 0.f;
+                bool found = false;
+#pragma unroll
+                for (int kk = 0; kk < 3; kk++) {
+                    const int ki = 2 * half + kk;
+                    const float w0 = PL ? c[ki].y : c[ki].z, w1 = PL ? c[ki].z : c[ki].w, w2 = PL ? c[ki].w : e[ki];
+                    if (w0 > mx) { mx = w0; fx = (float)(j0 + 2); fy = (float)(i + ki); found = true; }
+                    if (w1 > mx) { mx = w1; fx = (float)(j0 + 3); fy = (float)(i + ki); found = true; }
+                    if (w2 > mx) { mx = w2; fx = (float)(j0 + 4); fy = (float)(i + ki); found = true; }
+                }
+                o.y = mx;
+                if (!found && live) { fx = indX[p + 1]; fy = indY[p + 1]; }
+                ix.y = fx; iy.y = fy;
+            }
+            if (live) {
+                *reinterpret_cast<float2 *>(O + p) = o;
+                *reinterpret_cast<float2 *>(indX + p) = ix;
+                *reinterpret_cast<float2 *>(indY + p) = iy;
+            }
+        }
+    }
+}
+
 // One wavefront per output.  Lane l visits taps l, l+64, ... in scan order (tap = ki*kc + kj),
 // keeping its first maximum; the reduction keeps the larger value and, on equal values, the
 // lower tap index.
@@ -375,9 +462,15 @@ int eddlhip_maxpool2d(int dev, const float *I, float *O, float *indX, float *ind
     } else if (kr == 3 && kc == 3 && sr == 2 && sc == 2 && pad_left <= 1 && W % 4 == 0 && s.LQ % 2 == 0 && 2 * s.LQ <= W &&
                al(I, 16) && al(O, 8) && al(indX, 8) && al(indY, 8)) {
         size_t pairs = total / 2;
-        auto kern = pad_left ? maxpool_3x3s2_kernel<1> : maxpool_3x3s2_kernel<0>;
-        hipLaunchKernelGGL(kern, dim3(eh_blocks(pairs, TPB, 1u << 18)), dim3(TPB), 0, st, I, O, indX, indY, pairs, H, W, s.LP, s.LQ,
-                           pad_top);
+        if (s.LP % 2 == 0) {
+            auto kern = pad_left ? maxpool_3x3s2_rows_kernel<1> : maxpool_3x3s2_rows_kernel<0>;
+            hipLaunchKernelGGL(kern, dim3(eh_blocks(pairs / 2, TPB, 1u << 18)), dim3(TPB), 0, st, I, O, indX, indY, pairs / 2, H, W, s.LP,
+                               s.LQ, pad_top);
+        } else {
+            auto kern = pad_left ? maxpool_3x3s2_kernel<1> : maxpool_3x3s2_kernel<0>;
+            hipLaunchKernelGGL(kern, dim3(eh_blocks(pairs, TPB, 1u << 18)), dim3(TPB), 0, st, I, O, indX, indY, pairs, H, W, s.LP, s.LQ,
+                               pad_top);
+        }
     } else if (kr == 3 && kc == 3 && (long long)H * W < (1LL << 31)) {
         hipLaunchKernelGGL((maxpool_window_kernel<3, 3>), dim3(eh_blocks(total, TPB, 1u << 18)), dim3(TPB), 0, st, I, O, indX, indY,
                            total, s);
