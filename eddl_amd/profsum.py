@@ -92,13 +92,14 @@ def trace(workload, trace_dir, log, out, extra=""):
     bench = bench_line(log)
     o = ["rocprofv3 kernel trace of the %s benchmark (MI355X, gfx950)%s" % (workload, ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root):",
-         "  rocprofv3 --kernel-trace --stats --output-format csv -d %s -o %s -- python3 bench.py --workload %s --steps 10 --warmup 3 --no-cpu-baseline --no-device-probe --no-workloads%s > %s"
+         "  rocprofv3 --kernel-trace --stats --output-format csv -d %s -o %s -- python3 bench.py --workload %s --steps 10 --warmup 3 --no-cpu-baseline --no-device-probe --no-workloads --no-tune%s > %s"
          % (trace_dir, workload, workload, extra, log),
          "  python3 -m eddl_amd.profsum trace %s %s %s %s" % (workload, trace_dir, log, out),
          "",
          "columns: rocprofv3's own *_kernel_stats.csv, unchanged: Name, Calls, TotalDurationNs, AverageNs (= TotalDurationNs / Calls),",
          "Percentage (= TotalDurationNs / sum of TotalDurationNs over all kernels x 100).  The run holds 3 warm-up + 10 timed steps and",
-         "the repetitions bench.py uses to time the dominant kernel with HIP events.",
+         "the repetitions bench.py uses to time the dominant kernel with HIP events.  --no-tune keeps the launch planner's own plans: the",
+         "plan search of a default bench.py run would add its measurement launches (every plan of every layer) to the trace.",
          "",
          "%-100s %6s %14s %12s %7s" % ("kernel", "calls", "total ns", "average ns", "%")]
     for r in stats:
@@ -124,7 +125,7 @@ def traffic(workload, trace_dir, fetch_dir, write_dir, log, out, out_json=None, 
         raise SystemExit("the counter runs hold no copy probe: run bench.py with --copy-probe")
     sf, sw = COPY_PROBE_KIB / max(f[probe[0]]), COPY_PROBE_KIB / max(w[probe[0]])
     bench = bench_line(log)
-    args = "--workload %s%s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --copy-probe" % (workload, extra)
+    args = "--workload %s%s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --no-tune --copy-probe" % (workload, extra)
     o = ["HBM traffic per launch of the %s benchmark kernels%s (MI355X, gfx950)%s"
          % (workload, " run layer by layer" if "--unfused" in extra else "", ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root; one counter per run):",
@@ -180,7 +181,7 @@ def mfma(workload, directory, out):
     dur = durations(directory)
     o = ["Matrix-core counters of the %s benchmark kernels (MI355X, gfx950)%s" % (workload, ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root):",
-         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-workloads"
+         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-workloads --no-tune"
          % (MFMA_COUNTERS, directory, workload),
          "  python3 -m eddl_amd.profsum mfma %s %s %s" % (workload, directory, out),
          ""]
@@ -218,8 +219,8 @@ def stalls(workload, sq_dir, tcp_dir, out):
     dur = durations(sq_dir)
     o = ["Wavefront stall counters of the %s benchmark's convolution kernels (MI355X, gfx950)%s" % (workload, ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root; two passes, the hardware holds 8 SQ counters at a time):",
-         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads" % (STALL_SQ, sq_dir, workload),
-         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads" % (STALL_TCP, tcp_dir, workload),
+         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --no-tune" % (STALL_SQ, sq_dir, workload),
+         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --no-tune" % (STALL_TCP, tcp_dir, workload),
          "  python3 -m eddl_amd.profsum stalls %s %s %s %s" % (workload, sq_dir, tcp_dir, out),
          "",
          "columns (each counter: Counter_Value of a dispatch, averaged over the kernel's dispatches; SQ counters are sampled on one of the",
