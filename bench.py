@@ -176,7 +176,7 @@ def oracle_parity(workload, device_output, max_images):
 RIDGE_FLOP_PER_BYTE = PEAK_FP32_MFMA_TFLOPS * 1e3 / PEAK_HBM_GBS  # 19.7: below it a layer is bound by HBM, not by the matrix cores
 
 
-def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True):
+def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, plans=None):
     """Builds the workload, runs `warmup` + `steps` forwards with the input resident in HBM, then times every op.
     Returns (summary dict, per-op rows, device output of the last forward, model description)."""
     model, x, desc = build_workload(workload)
@@ -193,8 +193,12 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True):
             model.run()
             hip.synchronize()
         hip.conv_autotune(True)
+        if plans and os.path.exists(plans):
+            hip.conv_tuned_load(plans)   # what an earlier run found: nothing left to search for these geometries
         model.run()
         hip.synchronize()
+        if plans:
+            hip.conv_tuned_save(plans)
     step = model.run
     if graph:
         model.capture()
@@ -248,9 +252,13 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True):
     if os.path.exists(tpath) and fused:  # the committed counter runs are of the fused plan
         with open(tpath) as fh:
             t = json.load(fh)
-        if t.get("kernel", "").replace(" ", "") == dom_name.replace(" ", ""):
+        same_kernel = t.get("kernel", "").replace(" ", "") == dom_name.replace(" ", "")
+        if same_kernel and t.get("launches_per_step") in (None, dom_launches):
             roofline["traffic"] = t.get("hbm_bytes_per_launch")
             roofline["traffic_measured_at_commit"] = t.get("commit")
+        elif same_kernel:  # the plan search gave that kernel other layers in this run than in the counter runs
+            roofline["traffic_note"] = ("profiles/traffic_%s.json averages %s launches per step of this kernel, this run has %d"
+                                        % (workload, t.get("launches_per_step"), dom_launches))
         else:
             roofline["traffic_note"] = "profiles/traffic_%s.json is for %s, not this run's dominant kernel" % (workload, t.get("kernel"))
     # convolutions whose arithmetic intensity is below the ridge (first layers with 1-3 input channels, 1-filter
@@ -296,6 +304,9 @@ def main():
     ap.add_argument("--no-tune", action="store_true",
                     help="keep the launch planner's own choice for every convolution (without it the library searches the launch "
                          "plans of every convolution geometry once, before the timed region: eddlhip_conv2d_autotune)")
+    ap.add_argument("--plans", default=None, metavar="FILE",
+                    help="start the plan search from the plans in FILE (if it exists) and write what the run ends up with back to it: "
+                         "a second run with the same file launches no search (kernel traces then hold the workload only)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="after the timed region run one ReLU over 2^26 floats (reads 256 MiB, writes 256 MiB): the plain copy "
                          "kernel of known size that scales FETCH_SIZE / WRITE_SIZE counter readings")
@@ -306,7 +317,7 @@ def main():
     import eddl_amd
     hip = eddl_amd.Backend(0)
     hip.set_conv_algo(args.conv_algo)
-    summary, rows, out_host, desc = measure(hip, args.workload, args.steps, args.warmup, fused=not args.unfused, graph=args.graph, tune=not args.no_tune)
+    summary, rows, out_host, desc = measure(hip, args.workload, args.steps, args.warmup, fused=not args.unfused, graph=args.graph, tune=not args.no_tune, plans=args.plans)
     batch = summary["batch"]
     ms_per_step = summary["ms_per_step"]
     roofline = summary["roofline"]

@@ -62,6 +62,8 @@ PROTOTYPES = {
     "eddlhip_conv2d_trace": [P, ctypes.c_longlong],
     "eddlhip_conv2d_autotune": [c_int],
     "eddlhip_conv2d_tuned_plans": [c_int],
+    "eddlhip_conv2d_tuned_save": [c_int, ctypes.c_char_p],
+    "eddlhip_conv2d_tuned_load": [c_int, ctypes.c_char_p],
     "eddlhip_batchnorm_inference": [c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, c_float],
     "eddlhip_relu": [c_int, P, P, c_size_t],
     "eddlhip_sigmoid": [c_int, P, P, c_size_t],

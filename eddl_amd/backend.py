@@ -272,6 +272,14 @@ class Backend:
     def conv_tuned_plans(self):
         return self.lib.eddlhip_conv2d_tuned_plans(self.dev)
 
+    def conv_tuned_save(self, path):
+        """Write the plans found so far to a text file."""
+        self._check(self.lib.eddlhip_conv2d_tuned_save(self.dev, str(path).encode()))
+
+    def conv_tuned_load(self, path):
+        """Merge a file written by ``conv_tuned_save`` into the table (used while the plan search is on)."""
+        self._check(self.lib.eddlhip_conv2d_tuned_load(self.dev, str(path).encode()))
+
     def conv_trace(self, workgroups):
         """Per-workgroup timeline records of the next convolution launches (at most `workgroups` workgroups each);
         returns the device tensor that receives them (two floats hold one 64-bit word), or switches tracing off with 0."""

@@ -1414,6 +1414,53 @@ int eddlhip_conv2d_autotune(int on) {
     return 0;
 }
 
+int eddlhip_conv2d_tuned_save(int dev, const char *host_path) {
+    EH_REQUIRE(dev >= 0 && dev < EDDLHIP_MAX_DEVICES && host_path != nullptr, "conv2d_tuned_save: bad arguments");
+    FILE *f = fopen(host_path, "w");
+    EH_REQUIRE(f != nullptr, "conv2d_tuned_save: cannot write %s", host_path);
+    fprintf(f, "# eddlhip tuned convolution plans: N C H W Kf R S sr sc pad_top pad_left P Q two-tensor uh uw direct | tile slices\n");
+    for (const TunedPlan &t : g_tuned[dev]) {
+        for (int v : t.key) fprintf(f, "%d ", v);
+        fprintf(f, "| %d %d\n", t.tile, t.slices);
+    }
+    const bool ok = fclose(f) == 0;
+    EH_REQUIRE(ok, "conv2d_tuned_save: writing %s failed", host_path);
+    return 0;
+}
+
+int eddlhip_conv2d_tuned_load(int dev, const char *host_path) {
+    EH_REQUIRE(dev >= 0 && dev < EDDLHIP_MAX_DEVICES && host_path != nullptr, "conv2d_tuned_load: bad arguments");
+    FILE *f = fopen(host_path, "r");
+    EH_REQUIRE(f != nullptr, "conv2d_tuned_load: cannot read %s", host_path);
+    std::vector<TunedPlan> read;
+    char line[512];
+    bool bad = false;
+    while (fgets(line, sizeof(line), f) != nullptr) {
+        if (line[0] == '#' || line[0] == '\n') continue;
+        TunedPlan t;
+        int *k = t.key;
+        const int got = sscanf(line, "%d %d %d %d %d %d %d %d %d %d %d %d %d %d %d %d %d | %d %d", k, k + 1, k + 2, k + 3, k + 4, k + 5, k + 6, k + 7,
+                               k + 8, k + 9, k + 10, k + 11, k + 12, k + 13, k + 14, k + 15, k + 16, &t.tile, &t.slices);
+        if (got != 19 || t.tile < -1 || t.tile > 3 || t.slices < 1 || t.slices > 64) {
+            bad = true;
+            break;
+        }
+        read.push_back(t);
+    }
+    fclose(f);
+    EH_REQUIRE(!bad, "conv2d_tuned_load: %s holds a line that is not a plan", host_path);
+    for (const TunedPlan &t : read) {
+        bool known = false;
+        for (TunedPlan &have : g_tuned[dev])
+            if (memcmp(have.key, t.key, sizeof(t.key)) == 0) {
+                have = t;
+                known = true;
+            }
+        if (!known) g_tuned[dev].push_back(t);
+    }
+    return 0;
+}
+
 int eddlhip_conv2d_tuned_plans(int dev) {
     EH_REQUIRE(dev >= 0 && dev < EDDLHIP_MAX_DEVICES, "conv2d_tuned_plans: bad device %d", dev);
     return (int)g_tuned[dev].size();

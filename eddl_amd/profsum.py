@@ -81,7 +81,8 @@ def mean(values):
     return sum(values) / len(values)
 
 
-def write(path, lines):
+def write(path, lines, workload=""):
+    lines = [l.replace("WLTOKEN", workload) for l in lines]
     with open(path, "w") as fh:
         fh.write("\n".join(lines) + "\n")
     print("\n".join(lines))
@@ -92,14 +93,16 @@ def trace(workload, trace_dir, log, out, extra=""):
     bench = bench_line(log)
     o = ["rocprofv3 kernel trace of the %s benchmark (MI355X, gfx950)%s" % (workload, ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root):",
-         "  rocprofv3 --kernel-trace --stats --output-format csv -d %s -o %s -- python3 bench.py --workload %s --steps 10 --warmup 3 --no-cpu-baseline --no-device-probe --no-workloads --no-tune%s > %s"
+         "  rocprofv3 --kernel-trace --stats --output-format csv -d %s -o %s -- python3 bench.py --workload %s --steps 10 --warmup 3 --no-cpu-baseline --no-device-probe --no-workloads --plans gpurun_out/plans_WLTOKEN.txt%s > %s"
          % (trace_dir, workload, workload, extra, log),
          "  python3 -m eddl_amd.profsum trace %s %s %s %s" % (workload, trace_dir, log, out),
          "",
          "columns: rocprofv3's own *_kernel_stats.csv, unchanged: Name, Calls, TotalDurationNs, AverageNs (= TotalDurationNs / Calls),",
          "Percentage (= TotalDurationNs / sum of TotalDurationNs over all kernels x 100).  The run holds 3 warm-up + 10 timed steps and",
-         "the repetitions bench.py uses to time the dominant kernel with HIP events.  --no-tune keeps the launch planner's own plans: the",
-         "plan search of a default bench.py run would add its measurement launches (every plan of every layer) to the trace.",
+         "the repetitions bench.py uses to time the dominant kernel with HIP events.  The plans file comes from an earlier, unprofiled run",
+         "of the same workload (python3 bench.py --workload W --steps 3 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads",
+         "--plans gpurun_out/plans_W.txt), which searched the launch plans and saved what it found: the profiled run loads them and",
+         "launches no search, so the trace holds the workload only, under the plans a default bench.py run uses.",
          "",
          "%-100s %6s %14s %12s %7s" % ("kernel", "calls", "total ns", "average ns", "%")]
     for r in stats:
@@ -114,7 +117,7 @@ def trace(workload, trace_dir, log, out, extra=""):
         dom = [r for r in stats if key in r["Name"].replace(" ", "")]
         if dom:
             o.append("  same kernel in the trace above: average %.4f ms over %s calls" % (float(dom[0]["AverageNs"]) / 1e6, dom[0]["Calls"]))
-    write(out, o)
+    write(out, o, workload)
 
 
 def traffic(workload, trace_dir, fetch_dir, write_dir, log, out, out_json=None, extra=""):
@@ -125,7 +128,7 @@ def traffic(workload, trace_dir, fetch_dir, write_dir, log, out, out_json=None, 
         raise SystemExit("the counter runs hold no copy probe: run bench.py with --copy-probe")
     sf, sw = COPY_PROBE_KIB / max(f[probe[0]]), COPY_PROBE_KIB / max(w[probe[0]])
     bench = bench_line(log)
-    args = "--workload %s%s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --no-tune --copy-probe" % (workload, extra)
+    args = "--workload %s%s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --plans gpurun_out/plans_WLTOKEN.txt --copy-probe" % (workload, extra)
     o = ["HBM traffic per launch of the %s benchmark kernels%s (MI355X, gfx950)%s"
          % (workload, " run layer by layer" if "--unfused" in extra else "", ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root; one counter per run):",
@@ -162,14 +165,14 @@ def traffic(workload, trace_dir, fetch_dir, write_dir, log, out, out_json=None, 
         per_kernel[k] = b
     if bench:
         o += ["", "bench.py line of the traced run: %.1f %s, %.3f ms/step" % (bench["value"], bench["unit"], bench["ms_per_step"])]
-    write(out, o)
+    write(out, o, workload)
     if out_json and bench:
         key = bench["roofline"]["kernel"].replace(" ", "")
         m = [k for k in per_kernel if key in k.replace(" ", "")]
         if m:
             with open(out_json, "w") as fh:
                 json.dump({"kernel": bench["roofline"]["kernel"], "hbm_bytes_per_launch": per_kernel[m[0]], "fetch_scale": sf, "write_scale": sw,
-                           "source": out, "commit": commit()}, fh, indent=1)
+                           "launches_per_step": bench["roofline"].get("launches_per_step"), "source": out, "commit": commit()}, fh, indent=1)
                 fh.write("\n")
 
 
@@ -181,7 +184,7 @@ def mfma(workload, directory, out):
     dur = durations(directory)
     o = ["Matrix-core counters of the %s benchmark kernels (MI355X, gfx950)%s" % (workload, ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root):",
-         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-workloads --no-tune"
+         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-workloads --plans gpurun_out/plans_WLTOKEN.txt"
          % (MFMA_COUNTERS, directory, workload),
          "  python3 -m eddl_amd.profsum mfma %s %s %s" % (workload, directory, out),
          ""]
@@ -205,7 +208,7 @@ def mfma(workload, directory, out):
         cyc = mean(gui[k]) / 8.0
         o.append("%-88s %6d %9.1f %12.2f %9.1f %7.1f %7.1f %6.2f"
                  % (short(k, 88), len(dur[k]), us, fl / 1e9, fl / us / 1e6, fl / us / 1e6 / FP32_MFMA_PEAK_TFLOPS * 100, 100 * mean(busy[k]) / (cyc * 1024.0), cyc / us / 1e3))
-    write(out, o)
+    write(out, o, workload)
 
 
 STALL_SQ = "SQ_WAVES SQ_WAVE_CYCLES SQ_BUSY_CYCLES SQ_WAIT_INST_ANY SQ_VALU_MFMA_BUSY_CYCLES SQ_ACTIVE_INST_VALU SQ_ACTIVE_INST_LDS SQ_WAIT_INST_LDS GRBM_GUI_ACTIVE"
@@ -219,8 +222,8 @@ def stalls(workload, sq_dir, tcp_dir, out):
     dur = durations(sq_dir)
     o = ["Wavefront stall counters of the %s benchmark's convolution kernels (MI355X, gfx950)%s" % (workload, ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root; two passes, the hardware holds 8 SQ counters at a time):",
-         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --no-tune" % (STALL_SQ, sq_dir, workload),
-         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --no-tune" % (STALL_TCP, tcp_dir, workload),
+         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --plans gpurun_out/plans_WLTOKEN.txt" % (STALL_SQ, sq_dir, workload),
+         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --plans gpurun_out/plans_WLTOKEN.txt" % (STALL_TCP, tcp_dir, workload),
          "  python3 -m eddl_amd.profsum stalls %s %s %s %s" % (workload, sq_dir, tcp_dir, out),
          "",
          "columns (each counter: Counter_Value of a dispatch, averaged over the kernel's dispatches; SQ counters are sampled on one of the",
@@ -247,7 +250,7 @@ def stalls(workload, sq_dir, tcp_dir, out):
                  % (short(k, 64), len(dur[k]), mean(dur[k]), 100 * m(a, "SQ_VALU_MFMA_BUSY_CYCLES") / (cyc_a * 1024),
                     100 * m(a, "SQ_WAIT_INST_ANY") / wc, 100 * m(a, "SQ_WAIT_INST_LDS") / wc, 100 * m(b, "SQ_ACTIVE_INST_ANY") / wc_b,
                     100 * m(b, "TCP_PENDING_STALL_CYCLES_sum") / (cyc_b * 256), m(b, "SQ_INSTS_VALU") / (m(b, "SQ_INSTS_VMEM_RD") + m(b, "SQ_INSTS_VMEM_WR"))))
-    write(out, o)
+    write(out, o, workload)
 
 
 def counters(title, directory, out, wanted):

@@ -227,6 +227,12 @@ const char *eddlhip_conv2d_last_kernel(void);
  * search prints one line to stderr (geometry, the planner's time, the best time and plan). */
 int eddlhip_conv2d_autotune(int on);
 int eddlhip_conv2d_tuned_plans(int dev);
+/* The table as a text file (one geometry and its plan per line), so that a later process starts from what an earlier
+ * one found: _save writes the device's table, _load merges a file into it (a geometry already in the table takes the
+ * file's plan).  A loaded plan is used like a found one while eddlhip_conv2d_autotune(1) is in force.  A file from
+ * another device model is accepted (its plans are valid launches) but was not measured there. */
+int eddlhip_conv2d_tuned_save(int dev, const char *host_path);
+int eddlhip_conv2d_tuned_load(int dev, const char *host_path);
 
 /* Overrides the launch planner of the MFMA kernels (tuning and tests): tile = 0 (128x128 outputs per
  * workgroup), 1 (64x128), 2 (64x64), 3 (32x128) or -1 to give the choice back to the planner;

@@ -38,6 +38,34 @@ def test_version_and_argument_errors_without_a_device():
     assert lib.eddlhip_pool2d_out_dims(5, 5, 0, 3, 2, 2, 0, 1, 0, 1, ctypes.byref(lp), ctypes.byref(lq)) == -1
 
 
+def test_tuned_plan_table_round_trips_through_a_file(tmp_path):
+    """eddlhip_conv2d_tuned_save / _load need no device: a file of plans is merged into the table and written back."""
+    from eddl_amd import _lib
+    lib = _lib.load()
+    lib.eddlhip_conv2d_autotune(-1)
+    assert lib.eddlhip_conv2d_tuned_plans(0) == 0
+    src = tmp_path / "plans.txt"
+    src.write_text("# comment\n"
+                   "64 64 56 56 64 3 3 1 1 1 1 56 56 0 1 1 1 | 2 4\n"
+                   "32 512 28 28 512 3 3 1 1 1 1 28 28 0 1 1 1 | -1 1\n")
+    assert lib.eddlhip_conv2d_tuned_load(0, str(src).encode()) == 0
+    assert lib.eddlhip_conv2d_tuned_plans(0) == 2
+    assert lib.eddlhip_conv2d_tuned_load(0, str(src).encode()) == 0     # known geometries are replaced, not repeated
+    assert lib.eddlhip_conv2d_tuned_plans(0) == 2
+    dst = tmp_path / "out.txt"
+    assert lib.eddlhip_conv2d_tuned_save(0, str(dst).encode()) == 0
+    body = [l for l in dst.read_text().splitlines() if not l.startswith("#")]
+    assert body == ["64 64 56 56 64 3 3 1 1 1 1 56 56 0 1 1 1 | 2 4", "32 512 28 28 512 3 3 1 1 1 1 28 28 0 1 1 1 | -1 1"]
+    bad = tmp_path / "bad.txt"
+    bad.write_text("64 64 56 56 | 9 9\n")
+    assert lib.eddlhip_conv2d_tuned_load(0, str(bad).encode()) < 0
+    assert b"not a plan" in lib.eddlhip_last_error()
+    assert lib.eddlhip_conv2d_tuned_load(0, str(tmp_path / "missing.txt").encode()) < 0
+    assert lib.eddlhip_conv2d_tuned_plans(0) == 2
+    lib.eddlhip_conv2d_autotune(-1)
+    assert lib.eddlhip_conv2d_tuned_plans(0) == 0
+
+
 def test_descriptor_mirrors_match_the_oracle_geometry(oracle, golden):
     from eddl_amd.descriptors import ConvolDescriptor, PoolDescriptor
     t = golden["output_sizes"]
