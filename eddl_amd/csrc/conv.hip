@@ -953,51 +953,68 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_gen_kernel(c
 }
 
 // ---------------------------------------------------------------- finishing kernel of K-split tiles
-// One wavefront per 32x32 block of a divided tile (4 wavefronts x TM x TN blocks per tile), same
-// lane -> output mapping as the MFMA kernels: adds the slices in increasing K order (a fixed
-// order: results do not depend on scheduling), then applies the fused tail and stores.
+// One workgroup per 32x32 block of a divided tile (4 wavefronts x TM x TN blocks per tile), same lane -> output
+// mapping as the MFMA kernels, a quarter of the block's rows per wavefront (accumulator registers 4q .. 4q+3 of
+// wavefront q): adds the slices in increasing K order (a fixed order: results do not depend on scheduling), then
+// applies the fused tail and stores.  A wavefront has few values and therefore all slices' loads in flight at once
+// (fifteen slices at a time): the kernel lasts about one trip to memory.
 template <int WM, int WN, int TM, int TN>
-__global__ __launch_bounds__(64) void conv_reduce_kernel(const ConvParams p) {
+__global__ __launch_bounds__(256) void conv_reduce_kernel(const ConvParams p) {
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32, UNITS = 4 * TM * TN;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63, q = threadIdx.x >> 6, half = lane >> 5;
     const int unit = blockIdx.x % UNITS, local_tile = blockIdx.x / UNITS;
     const int wave = unit / (TM * TN), blk = unit % (TM * TN);
     const int wm = wave / WN, wn = wave % WN, tm = blk / TN, tn = blk % TN;
     const int tile = p.main_tiles + local_tile;
-    const int m0 = (tile % p.gm) * BM + (wm * TM + tm) * 32;
-    const long long n0 = (long long)(tile / p.gm) * BN + (wn * TN + tn) * 32;
+    const int m_first = (tile % p.gm) * BM + (wm * TM + tm) * 32 + 8 * q + 4 * half;  // this lane's rows: m_first + 0..3
+    const long long n = (long long)(tile / p.gm) * BN + (wn * TN + tn) * 32 + (lane & 31);
     const size_t tiles = gridDim.x / UNITS;
-    // the channel constants are asked for first; four slices' loads are in flight at a time, and the
-    // additions keep the slice order (starting from slice 0's value, not from zero)
-    const ChannelEpilogue chan = fetch_channel_constants<32>(p, m0, lane);
+    // the channel constants are asked for first, then the slices
+    ChannelEpilogue chan[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) chan[j] = load_channel(p, m_first + j < p.Kf ? m_first + j : p.Kf - 1);
     const size_t slice_stride = tiles * 4 * (TM * TN) * (16 * 64);
-    const float *src = p.partial + (((size_t)local_tile * 4 + wave) * (TM * TN) + blk) * (16 * 64) + lane;
-    floatx16 acc[1][1];
+    const float *src = p.partial + (((size_t)local_tile * 4 + wave) * (TM * TN) + blk) * (16 * 64) + (4 * q) * 64 + lane;
+    float acc[4];
 #pragma unroll
-    for (int v = 0; v < 16; v++) acc[0][0][v] = src[v * 64];
+    for (int j = 0; j < 4; j++) acc[j] = src[j * 64];  // the sum starts from slice 0's value, not from zero
     int sl = 1;
-    for (; sl + 4 <= p.nslices; sl += 4) {
-        float x[4][16];
+    for (; sl + 15 <= p.nslices; sl += 15) {
+        float x[15][4];
 #pragma unroll
-        for (int u = 0; u < 4; u++)
+        for (int u = 0; u < 15; u++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) x[u][v] = src[(size_t)(sl + u) * slice_stride + v * 64];
+            for (int j = 0; j < 4; j++) x[u][j] = src[(size_t)(sl + u) * slice_stride + j * 64];
 #pragma unroll
-        for (int u = 0; u < 4; u++)
+        for (int u = 0; u < 15; u++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[0][0][v] = __fadd_rn(acc[0][0][v], x[u][v]);
+            for (int j = 0; j < 4; j++) acc[j] = __fadd_rn(acc[j], x[u][j]);
     }
-    for (; sl < p.nslices; sl++) {
-        float x[16];
+    {
+        float x[14][4];
 #pragma unroll
-        for (int v = 0; v < 16; v++) x[v] = src[(size_t)sl * slice_stride + v * 64];
+        for (int u = 0; u < 14; u++)
+            if (sl + u < p.nslices) {
 #pragma unroll
-        for (int v = 0; v < 16; v++) acc[0][0][v] = __fadd_rn(acc[0][0][v], x[v]);
+                for (int j = 0; j < 4; j++) x[u][j] = src[(size_t)(sl + u) * slice_stride + j * 64];
+            }
+#pragma unroll
+        for (int u = 0; u < 14; u++)
+            if (sl + u < p.nslices) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[j] = __fadd_rn(acc[j], x[u][j]);
+            }
     }
-    __shared__ float epi[5 * 32];
-    put_channel_constants<32>(epi, chan, lane);
-    __syncthreads();
-    store_tile<1, 1, 32>(p, acc, epi, m0, 0, (int)n0, lane);
+    if (n >= p.npix) return;
+    const unsigned img = (unsigned)n / (unsigned)p.PQ, pq = (unsigned)n - img * (unsigned)p.PQ;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int m = m_first + j;
+        if (m < p.Kf) {
+            const size_t oidx = ((size_t)img * p.Kf + m) * p.PQ + pq;
+            p.O[oidx] = apply_epilogue(p, chan[j], acc[j], oidx);
+        }
+    }
 }
 
 // ---------------------------------------------------------------- 1x1 convolution onto a few filters
@@ -1408,7 +1425,7 @@ int eddlhip_conv2d_trace(unsigned long long *words, long long workgroups) {
 }
 
 int eddlhip_conv2d_autotune(int on) {
-    g_autotune = on != 0;
+    g_autotune = on > 0;
     if (on < 0)
         for (auto &t : g_tuned) t.clear();
     return 0;
@@ -1773,7 +1790,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
         EH_CHECK_LAUNCH();
         EH_TRY(prof_end(st));
         if (split_tiles > 0) {
-            hipLaunchKernelGGL(v->reduce, dim3((unsigned)(split_tiles * (v->bm / 32) * (v->bn / 32))), dim3(64), 0, st, q);
+            hipLaunchKernelGGL(v->reduce, dim3((unsigned)(split_tiles * (v->bm / 32) * (v->bn / 32))), dim3(256), 0, st, q);
             EH_CHECK_LAUNCH();
         }
     }

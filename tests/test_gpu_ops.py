@@ -745,3 +745,5 @@ def test_conv2d_autotune_searches_once_per_geometry_and_stays_within_tolerance(h
     finally:
         hip.conv_autotune(-1)
     assert hip.conv_tuned_plans() == 0
+    hip.conv2D(dx, dw, None, O, 1, 1, 1, 1)
+    assert hip.conv_tuned_plans() == 0                        # switched off: no search
