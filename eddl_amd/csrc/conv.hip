@@ -1138,10 +1138,12 @@ int g_force_tile = -1, g_force_slices = -1;  // eddlhip_conv2d_force_plan
 unsigned long long *g_trace = nullptr;       // eddlhip_conv2d_trace
 long long g_trace_wgs = 0;
 
-// eddlhip_conv2d_autotune: launch plans found by measurement, by device and geometry.  The epilogue is not part of the
-// key: a convolution sums in the same order whether its batch norm runs fused or as a launch of its own.
+// eddlhip_conv2d_autotune: launch plans found by measurement, by device and geometry.  Neither the epilogue nor the form of
+// the input is part of the key (image size and paddings - a folded Pad layer changes both -, one tensor or two, stored or
+// upsampled image): what a plan fixes, tile shape and K slices, meets the same channels, filter and output pixels either
+// way, and a convolution sums in the same order in a fused plan and in a layer-by-layer one.
 struct TunedPlan {
-    int key[17];       // N C H W Kf R S sr sc pad_top pad_left P Q two-tensor uh uw direct
+    int key[10];       // N C Kf R S sr sc P Q direct
     int tile, slices;  // tile -1: the planner's own choice was the fastest
 };
 bool g_autotune = false, g_tuning = false;
@@ -1435,7 +1437,7 @@ int eddlhip_conv2d_tuned_save(int dev, const char *host_path) {
     EH_REQUIRE(dev >= 0 && dev < EDDLHIP_MAX_DEVICES && host_path != nullptr, "conv2d_tuned_save: bad arguments");
     FILE *f = fopen(host_path, "w");
     EH_REQUIRE(f != nullptr, "conv2d_tuned_save: cannot write %s", host_path);
-    fprintf(f, "# eddlhip tuned convolution plans: N C H W Kf R S sr sc pad_top pad_left P Q two-tensor uh uw direct | tile slices\n");
+    fprintf(f, "# eddlhip tuned convolution plans: N C Kf R S sr sc P Q direct | tile slices\n");
     for (const TunedPlan &t : g_tuned[dev]) {
         for (int v : t.key) fprintf(f, "%d ", v);
         fprintf(f, "| %d %d\n", t.tile, t.slices);
@@ -1456,9 +1458,9 @@ int eddlhip_conv2d_tuned_load(int dev, const char *host_path) {
         if (line[0] == '#' || line[0] == '\n') continue;
         TunedPlan t;
         int *k = t.key;
-        const int got = sscanf(line, "%d %d %d %d %d %d %d %d %d %d %d %d %d %d %d %d %d | %d %d", k, k + 1, k + 2, k + 3, k + 4, k + 5, k + 6, k + 7,
-                               k + 8, k + 9, k + 10, k + 11, k + 12, k + 13, k + 14, k + 15, k + 16, &t.tile, &t.slices);
-        if (got != 19 || t.tile < -1 || t.tile > 3 || t.slices < 1 || t.slices > 64) {
+        const int got = sscanf(line, "%d %d %d %d %d %d %d %d %d %d | %d %d", k, k + 1, k + 2, k + 3, k + 4, k + 5, k + 6, k + 7, k + 8, k + 9, &t.tile,
+                               &t.slices);
+        if (got != 12 || t.tile < -1 || t.tile > 3 || t.slices < 1 || t.slices > 64) {
             bad = true;
             break;
         }
@@ -1647,7 +1649,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     Plan plan = plan_conv(family, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu, g_split != 0);
     if (g_force_tile >= 0) plan = forced_plan(family, g_force_tile, g_force_slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
     if (g_autotune && !g_tuning && g_force_tile < 0 && g_algo == 0 && g_split != 0) {
-        const int key[17] = {N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, two ? 1 : 0, uh, uw, direct};
+        const int key[10] = {N, C, Kf, R, S, sr, sc, P, Q, direct};
         const TunedPlan *found = nullptr;
         for (const TunedPlan &t : g_tuned[dev])
             if (memcmp(t.key, key, sizeof(key)) == 0) found = &t;

@@ -214,14 +214,15 @@ int eddlhip_conv2d_set_algo(int algo);
 const char *eddlhip_conv2d_last_kernel(void);
 
 /* Plan search on first use.  eddlhip_conv2d_autotune(1): from now on the first eddlhip_conv2d_fwd* call with a geometry the
- * device has not seen (N, C, H, W, Kf, R, S, strides, paddings, output size, input form) runs that convolution under
- * every launch plan (tile shape x K slices, three timed launches each, on the call's own tensors) and remembers the
- * fastest; later calls with that geometry take it.  The reference does the same on a layer's first forward, with
- * cudnnFindConvolutionForwardAlgorithm (src/hardware/gpu/nn/gpu_conv.cu:42-66, 211-213).  The epilogue is not part of
- * the geometry, so a layer computes the same sums whether its batch norm, residual and ReLU are fused or not; a plan
- * that divides tiles along K adds its slices in another order than an undivided one, so results with and without the
- * search agree to the convolution's tolerance, not bit for bit.  Calls that must not allocate or wait (graph
- * recording, eddlhip_conv2d_fwd_noalloc, eddlhip_conv2d_profile collecting) do not search; they use what was found.
+ * device has not seen (N, C, Kf, R, S, strides, output size P x Q) runs that convolution under every launch plan (tile
+ * shape x K slices, three timed launches each, on the call's own tensors) and remembers the fastest; later calls with
+ * that geometry take it.  The reference does the same on a layer's first forward, with
+ * cudnnFindConvolutionForwardAlgorithm (src/hardware/gpu/nn/gpu_conv.cu:42-66, 211-213).  Neither the epilogue, nor the
+ * image size and paddings (a folded Pad layer changes both), nor the form of the input (one tensor, two, upsampled) is
+ * part of the geometry, so a layer computes the same sums in a fused plan and layer by layer.  A plan that divides tiles
+ * along K adds its slices in another order than an undivided one, so results with and without the search agree to the
+ * convolution's tolerance, not bit for bit.  Calls that must not allocate or wait (graph recording,
+ * eddlhip_conv2d_fwd_noalloc, eddlhip_conv2d_profile collecting) do not search; they use what was found.
  * eddlhip_conv2d_autotune(0) stops searching and using the table, eddlhip_conv2d_autotune(-1) also empties it.
  * eddlhip_conv2d_tuned_plans(dev) = number of geometries in the table.  With EDDLHIP_TUNE_VERBOSE set in the environment every
  * search prints one line to stderr (geometry, the planner's time, the best time and plan). */

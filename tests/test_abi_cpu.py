@@ -46,8 +46,8 @@ def test_tuned_plan_table_round_trips_through_a_file(tmp_path):
     assert lib.eddlhip_conv2d_tuned_plans(0) == 0
     src = tmp_path / "plans.txt"
     src.write_text("# comment\n"
-                   "64 64 56 56 64 3 3 1 1 1 1 56 56 0 1 1 1 | 2 4\n"
-                   "32 512 28 28 512 3 3 1 1 1 1 28 28 0 1 1 1 | -1 1\n")
+                   "64 64 64 3 3 1 1 56 56 1 | 2 4\n"
+                   "32 512 512 3 3 1 1 28 28 1 | -1 1\n")
     assert lib.eddlhip_conv2d_tuned_load(0, str(src).encode()) == 0
     assert lib.eddlhip_conv2d_tuned_plans(0) == 2
     assert lib.eddlhip_conv2d_tuned_load(0, str(src).encode()) == 0     # known geometries are replaced, not repeated
@@ -55,7 +55,7 @@ def test_tuned_plan_table_round_trips_through_a_file(tmp_path):
     dst = tmp_path / "out.txt"
     assert lib.eddlhip_conv2d_tuned_save(0, str(dst).encode()) == 0
     body = [l for l in dst.read_text().splitlines() if not l.startswith("#")]
-    assert body == ["64 64 56 56 64 3 3 1 1 1 1 56 56 0 1 1 1 | 2 4", "32 512 28 28 512 3 3 1 1 1 1 28 28 0 1 1 1 | -1 1"]
+    assert body == ["64 64 64 3 3 1 1 56 56 1 | 2 4", "32 512 512 3 3 1 1 28 28 1 | -1 1"]
     bad = tmp_path / "bad.txt"
     bad.write_text("64 64 56 56 | 9 9\n")
     assert lib.eddlhip_conv2d_tuned_load(0, str(bad).encode()) < 0

@@ -113,6 +113,24 @@ def test_unet_small(hip, oracle):
     assert "pad" not in kinds and "batchnorm" not in kinds and "concat" not in kinds and kinds.count("conv2d") == 23
 
 
+def test_fused_plan_equals_layer_walk_with_the_plan_search_on(hip, oracle):
+    """The plan search keys on what a plan fixes (channels, filter, output pixels), not on paddings or the form of the input,
+    so a folded Pad / Concat / UpSampling and a fused epilogue still give the layer-by-layer result bit for bit."""
+    from eddl_amd import models
+    hip.conv_autotune(-1)
+    try:
+        hip.conv_autotune(True)
+        m = models.unet(batch=1, size=64, widths=(8, 16, 32, 64), bottleneck=128)
+        x = np.random.default_rng(5).uniform(0, 1, (1, 1, 64, 64)).astype(np.float32)
+        check_model(hip, oracle, m, x, 5)
+        m = models.resnet50(batch=2, size=64, num_classes=10, base=16)
+        x = np.random.default_rng(4).standard_normal((2, 3, 64, 64), dtype=np.float32)
+        check_model(hip, oracle, m, x, 4)
+        assert hip.conv_tuned_plans() > 10
+    finally:
+        hip.conv_autotune(-1)
+
+
 def test_batch_resize_and_asymmetric_padding_exception(hip, oracle):
     from eddl_amd import models, net as L
     m = models.conv_bn_relu_pool_block(batch=2, channels=8, size=12, filters=8)
