@@ -13,6 +13,7 @@
 #include <fstream>
 #include <iostream>
 
+#include "../../include/eddlhip.h"
 #include "eddl_hip_net.h"
 #include "eddl_hip_onnx.h"
 #include "eddl_hip_synth.h"
@@ -268,6 +269,14 @@ int main(int argc, char **argv) {
     }
     const string params = argv[2], in_path = argv[3], out_path = argv[4];
     const int batch = atoi(argv[5]), size = atoi(argv[6]);
+    // EDDLHIP_PLANS=<file>: the plan search of the library, started from the plans an earlier process found and saved
+    if (const char *plans = getenv("EDDLHIP_PLANS")) {
+        if (eddlhip_conv2d_tuned_load(0, plans) != 0 || eddlhip_conv2d_autotune(1) != 0) {
+            fprintf(stderr, "plans: %s\n", eddlhip_last_error());
+            return 2;
+        }
+        printf("plans: %d geometries loaded\n", eddlhip_conv2d_tuned_plans(0));
+    }
     vector<int> extra;
     for (int i = 7; i < argc; i++) extra.push_back(atoi(argv[i]));
     try {

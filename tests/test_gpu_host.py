@@ -168,6 +168,49 @@ def test_cpp_graphs_match_the_python_runner_bit_for_bit(hip, which, fused, tmp_p
     assert np.array_equal(got, want)
 
 
+def test_cpp_host_runs_the_plans_a_python_process_saved(hip, tmp_path):
+    """Plans travel between processes as a file: the Python host searches a block's convolution once, and the file it saves
+    is rewritten, once to an undivided plan and once to a four-way K-split (so that the plan in force is known).  The C++ host
+    started with either file must give what the Python host gives with that file, bit for bit; the two plans sum in different
+    orders, so the two results differ from each other in their last bits."""
+    from eddl_amd import models
+    batch, ch, size = 3, 64, 28
+    m = models.conv_bn_relu_pool_block(batch=batch, channels=ch, size=size, filters=ch)
+    models.init_he_normal(m, 43)
+    m.save(str(tmp_path / "params.bin"))
+    x = np.random.default_rng(43).standard_normal(m.lin[0].out_shape, dtype=np.float32)
+    x.tofile(tmp_path / "x.raw")
+    plans = str(tmp_path / "plans.txt")
+    assert os.path.exists(NET_DRIVER), "build the host layer first: make -C eddl_amd/host"
+    want = {}
+    hip.conv_autotune(-1)
+    try:
+        m.build(hip, fuse=True)
+        hip.conv_autotune(True)
+        m.predict([x])
+        assert hip.conv_tuned_plans() == 1
+        hip.conv_tuned_save(plans)
+        lines = open(plans).read().splitlines()
+        keys = [l.split("|")[0] for l in lines if l and not l.startswith("#")]
+        assert len(keys) == 1 and keys[0].split()[:3] == [str(batch), str(ch), str(ch)], lines
+        for plan in ("2 1", "2 4"):
+            with open(plans + plan[-1], "w") as f:
+                f.write("# rewritten by the test\n" + keys[0] + "| " + plan + "\n")
+            hip.conv_autotune(-1)
+            hip.conv_tuned_load(plans + plan[-1])
+            hip.conv_autotune(True)
+            want[plan] = m.predict([x])[0]
+    finally:
+        hip.conv_autotune(-1)
+    assert not np.array_equal(want["2 1"], want["2 4"]) and np.allclose(want["2 1"], want["2 4"], rtol=1e-4, atol=1e-5)
+    for plan in want:
+        res = subprocess.run([NET_DRIVER, "fused:block", str(tmp_path / "params.bin"), str(tmp_path / "x.raw"), str(tmp_path / "y.raw"), str(batch), str(size), str(ch), str(ch)],
+                             stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300, env=dict(os.environ, EDDLHIP_PLANS=plans + plan[-1]))
+        assert res.returncode == 0 and "plans: 1 geometries loaded" in res.stdout and "FAILED" not in res.stdout, (res.stdout[-2000:], res.stderr[-2000:])
+        got = np.fromfile(tmp_path / "y.raw", np.float32).reshape(want[plan].shape)
+        assert np.array_equal(got, want[plan]), plan
+
+
 @pytest.mark.parametrize("which", ["block", "resnet50", "unet"])
 def test_cpp_host_builds_a_configuration_from_seeds_alone(hip, which, tmp_path):
     """No parameter file and no input file: the C++ host draws both from the generator it shares with the Python host
