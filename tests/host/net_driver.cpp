@@ -270,7 +270,8 @@ int main(int argc, char **argv) {
     const string params = argv[2], in_path = argv[3], out_path = argv[4];
     const int batch = atoi(argv[5]), size = atoi(argv[6]);
     // EDDLHIP_PLANS=<file>: the plan search of the library, started from the plans an earlier process found and saved
-    if (const char *plans = getenv("EDDLHIP_PLANS")) {
+    const char *plans = getenv("EDDLHIP_PLANS");
+    if (plans != nullptr && plans[0] != 0) {
         if (eddlhip_conv2d_tuned_load(0, plans) != 0 || eddlhip_conv2d_autotune(1) != 0) {
             fprintf(stderr, "plans: %s\n", eddlhip_last_error());
             return 2;
@@ -341,7 +342,9 @@ int main(int argc, char **argv) {
         ofs.close();
         show_profile();
         if (timed) {  // forwards with the input already on the device
-            for (int i = 0; i < 5; i++) m->forward();
+            // warm-up: at least five forwards and 0.2 s, so that the device's clocks have settled
+            const auto w0 = std::chrono::steady_clock::now();
+            for (int i = 0; i < 5 || std::chrono::duration<double>(std::chrono::steady_clock::now() - w0).count() < 0.2; i++) m->forward();
             const auto t0 = std::chrono::steady_clock::now();
             const int reps = 20;
             for (int i = 0; i < reps; i++) m->forward();
