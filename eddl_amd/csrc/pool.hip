@@ -406,10 +406,30 @@ __global__ __launch_bounds__(64) void avgpool_plane_kernel(const float *__restri
     const size_t p0 = (size_t)blockIdx.x * 64;
     const int here = (int)(planes - p0 < 64 ? planes - p0 : 64);
     const float *src = I + p0 * hw;
-    for (int i = lane; i < here * hw; i += 64) plane_tile[(i / hw) * row + i % hw] = src[i];
+    // element i belongs to plane i / hw, position i % hw: both advance by fixed steps from one load to the next.
+    // Sixteen loads are requested before the first of them is stored, so a wavefront makes a handful of trips to memory.
+    int pl = lane / hw, k = lane - pl * hw;
+    const int dp = 64 / hw, dk = 64 - dp * hw;
+    const int n = here * hw;
+    for (int base = lane; base < n; base += 64 * 16) {
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; u++) v[u] = base + 64 * u < n ? src[base + 64 * u] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            if (base + 64 * u < n) plane_tile[pl * row + k] = v[u];
+            pl += dp;
+            k += dk;
+            if (k >= hw) {
+                k -= hw;
+                pl++;
+            }
+        }
+    }
     __syncthreads();
     if (lane < here) {
         float sum = 0.0f;
+#pragma unroll 8
         for (int k = 0; k < hw; k++) sum = __fadd_rn(sum, plane_tile[lane * row + k]);
         O[p0 + lane] = __fdiv_rn(sum, (float)hw);
     }
