@@ -85,6 +85,11 @@ struct ConvParams {
     // whose pixel (y, x) is the stored pixel (y / uh, x / uw).  uh == uw == 1: the stored image itself.
     int uh, uw;
     const float *Wp;  // packed filters [rows][Mp]
+    // Image n of the launch multiplies by the packed matrix at Wp + n * w_img_stride (floats): 0 for a convolution (one
+    // matrix for all images); the 16 products of a Winograd convolution run as ONE 1x1 launch over 16 "images", one
+    // transformed filter matrix each (an image's pixel count is then a multiple of every tile width, so that no tile
+    // holds pixels of two images).  conv_tap_kernel only.
+    size_t w_img_stride;
     const float *K;   // original OIHW filters (scalar kernel only)
     float *O;
     const float *bias, *bn_g, *bn_b, *bn_mean, *bn_var, *residual;
@@ -542,6 +547,8 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     // (plain 16-byte loads: the packed matrix is padded to whole steps and whole tiles, so every address exists)
     // Every thread loads in every round, without a condition: in a partial last round the lanes past
     // the end of the slice re-read their first element and park it behind the slice in LDS.
+    const float *wp = p.Wp;
+    if (p.w_img_stride != 0) wp += (size_t)((unsigned)n0 / (unsigned)p.PQ) * p.w_img_stride;  // the matrix of this tile's image
     const float *a_ptr[AV];
     int a_lds[AV];
 #pragma unroll
@@ -550,7 +557,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         const bool in_slice = f < A_VECS;
         const int fc = in_slice ? f : tid % A_VECS;
         const int kk = fc / (BM / 4), m4 = (fc % (BM / 4)) * 4;
-        a_ptr[j] = p.Wp + (size_t)kk * p.Mp + m0 + m4;
+        a_ptr[j] = wp + (size_t)kk * p.Mp + m0 + m4;
         a_lds[j] = in_slice ? kk * LDA + m4 : BK * LDA + lane * 4;
     }
     const int a_step = BK * p.Mp;
@@ -567,7 +574,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     constexpr int A_UNITS = (BK + RPI - 1) / RPI;
     constexpr int A_UPW = (A_UNITS + 3) / 4;
     static_assert((RPI - 1) * BM <= 256, "the parking area holds the surplus rows of the last unit");
-    const int32x4 dma_w = make_rsrc_words(p.Wp, p.wp_bytes), dma_in = make_rsrc_words(p.I, p.in_bytes);
+    const int32x4 dma_w = make_rsrc_words(wp, p.wp_bytes), dma_in = make_rsrc_words(p.I, p.in_bytes);
     const int32x4 dma_in2 = make_rsrc_words(p.I2, p.in_bytes);
     const int a_voff_direct = ((lane / (BM / 4)) * p.Mp + m0 + 4 * (lane % (BM / 4))) * 4;
 
@@ -1104,6 +1111,157 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvParams p) {
     }
 }
 
+// ---------------------------------------------------------------- Winograd F(2x2, 3x3)
+// A 3x3 stride-1 convolution as 16 independent products of [Kf x C] by [C x tiles] matrices (Lavin & Gray's minimal
+// filtering form): every 4x4 input patch d (stride 2, so neighbouring patches overlap by two pixels) becomes
+// V = B^T d B, every filter g becomes U = G g G^T, M = U (.) V summed over the channels - position by position, which is
+// what makes it 16 matrix products - and each 2x2 block of outputs is A^T M A.  2.25 times fewer multiplications than
+// the direct form.  The products run as ONE launch of the 1x1 tile kernel over 16 "images" (ConvParams::w_img_stride);
+// the two transforms are bandwidth kernels.  Sums are fp32 in a fixed order, so results are reproducible, and they
+// differ from the direct form's by rounding only (a few 1e-7 of the largest output on this path's layers).
+//   B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]   G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1]   A^T = [1 1 1 0; 0 1 -1 -1]
+struct WinoParams {
+    const float *I, *I2;  // input as ConvParams describes it (second tensor of a folded Concat, folded upsampling)
+    int Csplit, Cimg, uh, uw;
+    int C, H, W, pt, pl;
+    int th, tw;  // 2x2 output blocks per image, rows and columns
+    int T, Tp;   // blocks in the launch; Tp = T rounded up to the widest tile: one "image" of the product launch
+    float *V;    // [16][C][Tp]
+};
+constexpr int WINO_CH = 4;  // channels (input transform) or filters (output transform) per thread
+
+__global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restrict__ K, float *__restrict__ U, int Kf, int C, int Mp, int rows) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;  // (c, k), k fastest: row c of the packed matrices
+    if (idx >= rows * Mp) return;
+    const int c = idx / Mp, k = idx - c * Mp;
+    float g[9];
+#pragma unroll
+    for (int i = 0; i < 9; i++) g[i] = (c < C && k < Kf) ? K[((size_t)k * C + c) * 9 + i] : 0.0f;
+    float t[4][3];
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        t[0][j] = g[j];
+        t[1][j] = __fmul_rn(0.5f, __fadd_rn(__fadd_rn(g[j], g[3 + j]), g[6 + j]));
+        t[2][j] = __fmul_rn(0.5f, __fadd_rn(__fsub_rn(g[j], g[3 + j]), g[6 + j]));
+        t[3][j] = g[6 + j];
+    }
+    const size_t plane = (size_t)rows * Mp;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        U[(size_t)(4 * i + 0) * plane + idx] = t[i][0];
+        U[(size_t)(4 * i + 1) * plane + idx] = __fmul_rn(0.5f, __fadd_rn(__fadd_rn(t[i][0], t[i][1]), t[i][2]));
+        U[(size_t)(4 * i + 2) * plane + idx] = __fmul_rn(0.5f, __fadd_rn(__fsub_rn(t[i][0], t[i][1]), t[i][2]));
+        U[(size_t)(4 * i + 3) * plane + idx] = t[i][2];
+    }
+}
+
+// One thread: one 2x2 output block (its 4x4 input patch) for WINO_CH channels; lanes hold consecutive blocks, so the 16
+// stores of a channel are 16 coalesced rows.  The patch offsets and which of its pixels exist are worked out once.
+__global__ __launch_bounds__(256) void wino_input_kernel(const WinoParams w) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= w.T) return;
+    const int per_img = w.th * w.tw;
+    const int n = t / per_img, r = t - n * per_img, ty = r / w.tw, tx = r - ty * w.tw;
+    const int y0 = 2 * ty - w.pt, x0 = 2 * tx - w.pl;
+    const unsigned Hu = (unsigned)(w.H * w.uh), Wu = (unsigned)(w.W * w.uw);
+    int off[16];
+    unsigned mask = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const unsigned y = (unsigned)(y0 + i), x = (unsigned)(x0 + j);
+            const bool ok = y < Hu && x < Wu;
+            int o = 0;
+            if (ok) o = (w.uh == 1 && w.uw == 1) ? (int)(y * (unsigned)w.W + x) : (int)((y / (unsigned)w.uh) * (unsigned)w.W + x / (unsigned)w.uw);
+            off[4 * i + j] = o;
+            mask |= (ok ? 1u : 0u) << (4 * i + j);
+        }
+    const size_t hw = (size_t)w.H * w.W, plane = (size_t)w.C * w.Tp;
+    const int c0 = blockIdx.y * WINO_CH;
+#pragma unroll
+    for (int cc = 0; cc < WINO_CH; cc++) {
+        const int c = c0 + cc;
+        if (c >= w.C) break;
+        const float *src = c < w.Csplit ? w.I + ((size_t)n * w.Cimg + c) * hw : w.I2 + ((size_t)n * w.Cimg + (c - w.Csplit)) * hw;
+        float d[16];
+#pragma unroll
+        for (int e = 0; e < 16; e++) d[e] = ((mask >> e) & 1u) ? src[off[e]] : 0.0f;
+        float u[16];  // B^T d
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            u[0 + j] = __fsub_rn(d[0 + j], d[8 + j]);
+            u[4 + j] = __fadd_rn(d[4 + j], d[8 + j]);
+            u[8 + j] = __fsub_rn(d[8 + j], d[4 + j]);
+            u[12 + j] = __fsub_rn(d[4 + j], d[12 + j]);
+        }
+        float *dst = w.V + (size_t)c * w.Tp + t;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {  // (B^T d) B
+            dst[(size_t)(4 * i + 0) * plane] = __fsub_rn(u[4 * i + 0], u[4 * i + 2]);
+            dst[(size_t)(4 * i + 1) * plane] = __fadd_rn(u[4 * i + 1], u[4 * i + 2]);
+            dst[(size_t)(4 * i + 2) * plane] = __fsub_rn(u[4 * i + 2], u[4 * i + 1]);
+            dst[(size_t)(4 * i + 3) * plane] = __fsub_rn(u[4 * i + 1], u[4 * i + 3]);
+        }
+    }
+}
+
+// One thread: one 2x2 output block for WINO_CH filters: A^T M A, then the convolution's epilogue (the arithmetic of
+// apply_epilogue, value by value) and the stores - both values of a row at once where the row pair is aligned.
+__global__ __launch_bounds__(256) void wino_output_kernel(const ConvParams p, const float *__restrict__ M, int th, int tw, int T, int Tp) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= T) return;
+    const int per_img = th * tw;
+    const int n = t / per_img, r = t - n * per_img, ty = r / tw, tx = r - ty * tw;
+    const size_t plane = (size_t)p.Kf * Tp;
+    const bool pair = (p.Q % 2 == 0) && (((size_t)p.O | (size_t)(p.residual ? p.residual : p.O)) % 8 == 0);  // PQ is then even, too
+    const int k0 = blockIdx.y * WINO_CH;
+#pragma unroll
+    for (int cc = 0; cc < WINO_CH; cc++) {
+        const int k = k0 + cc;
+        if (k >= p.Kf) break;
+        const float *src = M + (size_t)k * Tp + t;
+        float m[16];
+#pragma unroll
+        for (int e = 0; e < 16; e++) m[e] = src[(size_t)e * plane];
+        float s[2][4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            s[0][j] = __fadd_rn(__fadd_rn(m[0 + j], m[4 + j]), m[8 + j]);
+            s[1][j] = __fsub_rn(__fsub_rn(m[4 + j], m[8 + j]), m[12 + j]);
+        }
+        const ChannelEpilogue e = load_channel(p, k);
+#pragma unroll
+        for (int a = 0; a < 2; a++) {
+            const int oy = 2 * ty + a, ox = 2 * tx;
+            if (oy >= p.P) break;
+            const float v0 = __fadd_rn(__fadd_rn(s[a][0], s[a][1]), s[a][2]);
+            const float v1 = __fsub_rn(__fsub_rn(s[a][1], s[a][2]), s[a][3]);
+            const size_t oidx = ((size_t)n * p.Kf + k) * p.PQ + (size_t)oy * p.Q + ox;
+            if (pair) {  // Q even: column ox + 1 exists
+                float r0 = 0.0f, r1 = 0.0f;
+                if (p.residual) {
+                    const float2 rr = *reinterpret_cast<const float2 *>(p.residual + oidx);
+                    r0 = rr.x;
+                    r1 = rr.y;
+                }
+                float x0 = v0, x1 = v1;
+                if (p.bias) x0 = __fadd_rn(x0, e.bias), x1 = __fadd_rn(x1, e.bias);
+                if (p.bn_mean) {
+                    x0 = __fdiv_rn(__fsub_rn(x0, e.mean), e.sd), x1 = __fdiv_rn(__fsub_rn(x1, e.mean), e.sd);
+                    if (p.bn_g) x0 = __fadd_rn(__fmul_rn(x0, e.g), e.b), x1 = __fadd_rn(__fmul_rn(x1, e.g), e.b);
+                }
+                if (p.residual) x0 = __fadd_rn(x0, r0), x1 = __fadd_rn(x1, r1);
+                if (p.relu) x0 = x0 > 0.0f ? x0 : 0.0f, x1 = x1 > 0.0f ? x1 : 0.0f;
+                *reinterpret_cast<float2 *>(p.O + oidx) = make_float2(x0, x1);
+            } else {
+                p.O[oidx] = apply_epilogue(p, e, v0, oidx);
+                if (ox + 1 < p.Q) p.O[oidx + 1] = apply_epilogue(p, e, v1, oidx + 1);
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------- host side
 int g_algo = 0;
 // Measurement: while collecting, every launch of a convolution kernel (not the filter repack, not
@@ -1134,6 +1292,7 @@ int prof_end(hipStream_t st) {
 }
 thread_local char g_last_kernel[128] = "";
 int g_split = 1;  // divide the tiles left over after a whole number per CU along K (set_algo 5 turns it off)
+bool g_wino = false;  // set_algo(7): the Winograd form wherever it applies (8: only where a searched plan asks for it)
 int g_force_tile = -1, g_force_slices = -1;  // eddlhip_conv2d_force_plan
 unsigned long long *g_trace = nullptr;       // eddlhip_conv2d_trace
 long long g_trace_wgs = 0;
@@ -1144,7 +1303,7 @@ long long g_trace_wgs = 0;
 // way, and a convolution sums in the same order in a fused plan and in a layer-by-layer one.
 struct TunedPlan {
     int key[10];       // N C Kf R S sr sc P Q direct
-    int tile, slices;  // tile -1: the planner's own choice was the fastest
+    int tile, slices;  // tile -1: the planner's own choice was the fastest; tile 4: the Winograd form
 };
 bool g_autotune = false, g_tuning = false;
 std::vector<TunedPlan> g_tuned[EDDLHIP_MAX_DEVICES];
@@ -1289,6 +1448,8 @@ struct CachedFilters {
     const float *K;
     int Kf, C, R, S, rows, Mp;
     float *Wp;
+    float *Wwino;  // 3x3 filters: the 16 transformed matrices of the Winograd form [16][wino_rows][Mp], made on first use
+    int wino_rows;
     bool stale;  // K was written through this library since the last repack
 };
 std::mutex g_cache_mutex;
@@ -1308,6 +1469,11 @@ int repack(int dev, CachedFilters &e) {
     hipLaunchKernelGGL(pack_filters_kernel, dim3((e.rows + 31) / 32, e.Mp / 32), dim3(256), 0, state(dev).stream, e.K, e.Wp, e.Kf,
                        e.C * e.R * e.S, e.Mp, e.rows);
     EH_CHECK_LAUNCH();
+    if (e.Wwino != nullptr) {
+        hipLaunchKernelGGL(wino_filter_kernel, dim3((unsigned)(((size_t)e.wino_rows * e.Mp + 255) / 256)), dim3(256), 0, state(dev).stream, e.K,
+                           e.Wwino, e.Kf, e.C, e.Mp, e.wino_rows);
+        EH_CHECK_LAUNCH();
+    }
     e.stale = false;
     return 0;
 }
@@ -1349,6 +1515,7 @@ void conv_filters_released(int dev, const void *base, size_t bytes) {
             // kernels still reading the packed copy finish first
             (void)hipStreamSynchronize(state(dev).stream);
             (void)hipFree(c[i].Wp);
+            if (c[i].Wwino) (void)hipFree(c[i].Wwino);
             c[i] = c.back();
             c.pop_back();
         } else {
@@ -1379,6 +1546,8 @@ int eddlhip_conv2d_cache_filters(int dev, const float *K, int Kf, int C, int R, 
     e.rows = cache_rows(C, R, S);
     e.Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
     e.Wp = nullptr;
+    e.Wwino = nullptr;
+    e.wino_rows = 0;
     e.stale = true;
     EH_REQUIRE((size_t)e.rows * e.Mp * sizeof(float) < ((size_t)1 << 31),
                "conv2d_cache_filters: the repacked filter matrix (%d taps x %d channels) exceeds the 2 GiB a buffer descriptor covers", e.rows, e.Mp);
@@ -1403,6 +1572,7 @@ int eddlhip_conv2d_uncache_filters(int dev, const float *K) {
             if (!synced) EH_TRY_HIP(hipStreamSynchronize(state(dev).stream));
             synced = true;
             EH_TRY_HIP(hipFree(c[i].Wp));
+            if (c[i].Wwino) EH_TRY_HIP(hipFree(c[i].Wwino));
             c[i] = c.back();
             c.pop_back();
         } else {
@@ -1413,7 +1583,7 @@ int eddlhip_conv2d_uncache_filters(int dev, const float *K) {
 }
 
 int eddlhip_conv2d_force_plan(int tile, int slices) {
-    EH_REQUIRE(tile >= -1 && tile <= 3, "conv2d_force_plan: tile is -1 (automatic) or 0..3");
+    EH_REQUIRE(tile >= -1 && tile <= 4, "conv2d_force_plan: tile is -1 (automatic), 0..3 or 4 (the Winograd form where it applies)");
     g_force_tile = tile;
     g_force_slices = slices;
     return 0;
@@ -1460,7 +1630,7 @@ int eddlhip_conv2d_tuned_load(int dev, const char *host_path) {
         int *k = t.key;
         const int got = sscanf(line, "%d %d %d %d %d %d %d %d %d %d | %d %d", k, k + 1, k + 2, k + 3, k + 4, k + 5, k + 6, k + 7, k + 8, k + 9, &t.tile,
                                &t.slices);
-        if (got != 12 || t.tile < -1 || t.tile > 3 || t.slices < 1 || t.slices > 64) {
+        if (got != 12 || t.tile < -1 || t.tile > 4 || t.slices < 1 || t.slices > 64) {
             bad = true;
             break;
         }
@@ -1486,9 +1656,13 @@ int eddlhip_conv2d_tuned_plans(int dev) {
 }
 
 int eddlhip_conv2d_set_algo(int algo) {
-    EH_REQUIRE(algo >= 0 && algo <= 6, "conv2d_set_algo: unknown algorithm %d", algo);
+    EH_REQUIRE(algo >= 0 && algo <= 8, "conv2d_set_algo: unknown algorithm %d", algo);
     if (algo == 5 || algo == 6) {
         g_split = (algo == 6);
+        return 0;
+    }
+    if (algo == 7 || algo == 8) {
+        g_wino = (algo == 7);
         return 0;
     }
     g_algo = algo;
@@ -1527,9 +1701,32 @@ namespace {
 // uh, uw > 1: the convolution runs over I enlarged uh x uw times by nearest-neighbour repetition (H, W stay the stored size).
 // no_alloc: take the scratch memory from the device's fixed array instead of the workspace, and refuse whatever
 // would allocate (an uninitialised device, a need beyond the array, event pairs for the measurement hook).
+// The 16 products of a Winograd convolution, run by conv2d_fwd_impl as a 1x1 convolution over 16 images: the packed
+// transformed filters (one matrix per image, `stride` floats apart) come from the caller instead of the filter tensor.
+struct GemmBatch {
+    const float *Wp;
+    size_t stride;
+};
+// Workspace a product launch may take for the partial tiles of a K-split plan: fewer than one tile per CU left over,
+// at most 16 slices each, 128 x 128 floats per tile.  The Winograd driver keeps its own buffers behind this much.
+constexpr size_t WINO_INNER_RESERVE = (size_t)16 * 255 * 128 * 128 * sizeof(float);
+
+int conv2d_winograd(int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C, int H, int W,
+                    int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
+                    const float *bn_var, float bn_eps, const float *residual, int relu);
+
+// Whether the Winograd form can run this convolution: 3x3, stride 1, and the product launch within the limits of
+// conv2d_fwd_impl (one "image" of transformed input or output below 1 GiB, fewer than 2^31 blocks).
+bool winograd_applies(int N, int C, int Kf, int R, int S, int sr, int sc, int P, int Q) {
+    if (R != 3 || S != 3 || sr != 1 || sc != 1) return false;
+    const long long T = (long long)N * ((P + 1) / 2) * ((Q + 1) / 2), Tp = (T + 127) / 128 * 128;
+    return Tp <= 0x3fffff80LL && (long long)C * Tp <= (1LL << 28) && (long long)Kf * Tp <= (1LL << 28);
+}
+
 int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
                     int H, int W, int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g,
-                    const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu) {
+                    const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu,
+                    const GemmBatch *gemm = nullptr) {
     EH_REQUIRE(N >= 0 && C > 0 && H > 0 && W > 0, "conv2d: bad input shape %dx%dx%dx%d", N, C, H, W);
     EH_REQUIRE(Kf > 0 && R > 0 && S > 0, "conv2d: bad filter shape %dx%dx%dx%d", Kf, C, R, S);
     EH_REQUIRE(sr > 0 && sc > 0, "conv2d: strides must be positive");
@@ -1597,6 +1794,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     p.in_bytes = p.wp_bytes = 0;
     p.main_tiles = 0; p.nslices = 1; p.slice_steps = 0; p.partial = nullptr;
     p.trace = nullptr;
+    p.w_img_stride = 0;
 
     if (g_algo == 2) {
         size_t total = (size_t)p.npix * Kf;
@@ -1609,7 +1807,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     }
 
     // ---- a 1x1 convolution onto at most four filters: a read stream, no tile
-    if (g_algo == 0 && g_force_tile < 0 && R == 1 && S == 1 && sr == 1 && sc == 1 && pad_top == 0 && pad_left == 0 && Kf <= 4 && !two &&
+    if (!gemm && g_algo == 0 && g_force_tile < 0 && R == 1 && S == 1 && sr == 1 && sc == 1 && pad_top == 0 && pad_left == 0 && Kf <= 4 && !two &&
         uh == 1 && uw == 1 && P == H && Q == W) {
         const bool vec4 = p.PQ % 4 == 0 && (((size_t)I | (size_t)O | (size_t)(residual ? residual : O)) & 15) == 0;
         void (*kern)(const ConvParams) = nullptr;
@@ -1647,13 +1845,22 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     EH_REQUIRE(max_imgs >= 1, "conv2d: one output plane of %d pixels is too large", p.PQ);
     const int chunk_imgs = (int)((N < max_imgs) ? N : max_imgs);
     Plan plan = plan_conv(family, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu, g_split != 0);
-    if (g_force_tile >= 0) plan = forced_plan(family, g_force_tile, g_force_slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
-    if (g_autotune && !g_tuning && g_force_tile < 0 && g_algo == 0 && g_split != 0) {
+    if (g_force_tile >= 0 && g_force_tile < 4)
+        plan = forced_plan(family, g_force_tile, g_force_slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
+    // the Winograd form: asked for (force_plan(4, .), set_algo(7)) or found faster by the plan search (below); never from the
+    // fixed scratch array, whose size it exceeds, and not for the scalar-order or register-staged algorithm switches
+    const bool wino_ok = !gemm && !no_alloc && g_algo == 0 && winograd_applies(N, C, Kf, R, S, sr, sc, P, Q);
+    if (wino_ok && (g_force_tile == 4 || (g_wino && g_force_tile < 0 && !g_tuning)))
+        return conv2d_winograd(dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean, bn_var,
+                               bn_eps, residual, relu);
+    if (g_autotune && g_force_tile < 0 && g_algo == 0 && g_split != 0) {
         const int key[10] = {N, C, Kf, R, S, sr, sc, P, Q, direct};
         const TunedPlan *found = nullptr;
         for (const TunedPlan &t : g_tuned[dev])
             if (memcmp(t.key, key, sizeof(key)) == 0) found = &t;
-        if (found == nullptr && !no_alloc && !state(dev).capturing && !g_prof_on) {
+        // (no search inside a search: a convolution being timed runs its product launch, a geometry of its own, under the
+        // plan already kept for it)
+        if (found == nullptr && !g_tuning && !no_alloc && !state(dev).capturing && !g_prof_on) {
             // First call with this geometry: run every plan on the call's own tensors (each writes the same output, up to
             // the rounding of its summation order) and keep the fastest.  The planner's choice stays unless another plan
             // beats it by more than the noise of the measurement.
@@ -1701,6 +1908,22 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
                     }
                 }
             }
+            if (rc == 0 && wino_ok) {
+                // the Winograd form; its product launch is a geometry of its own, searched first (one untimed call with the
+                // search open), then timed under what that search kept
+                g_tuning = false;
+                g_force_tile = 4;
+                int wrc = conv2d_fwd_impl(false, dev, I, I2, uh, uw, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
+                                          bn_mean, bn_var, bn_eps, residual, relu);
+                g_force_tile = -1;
+                g_tuning = true;
+                float ms = 0.0f;
+                if (wrc == 0 && measure(4, 1, &ms) == 0 && ms < best_ms && ms < 0.98f * planned_ms) {
+                    best_ms = ms;
+                    best.tile = 4;
+                    best.slices = 1;
+                }
+            }
             g_tuning = false;
             (void)hipEventDestroy(e0);
             (void)hipEventDestroy(e1);
@@ -1711,7 +1934,10 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
             g_tuned[dev].push_back(best);
             found = &g_tuned[dev].back();
         }
-        if (found != nullptr && found->tile >= 0)
+        if (found != nullptr && found->tile == 4 && wino_ok)
+            return conv2d_winograd(dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean, bn_var,
+                                   bn_eps, residual, relu);
+        if (found != nullptr && found->tile >= 0 && found->tile < 4)
             plan = forced_plan(family, found->tile, found->slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
     }
     const Variant *v = &family[plan.tile];
@@ -1729,8 +1955,8 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     // the kernels address the packed filters through a buffer descriptor with 32-bit byte offsets
     EH_REQUIRE((size_t)rows * p.Mp * sizeof(float) < ((size_t)1 << 31),
                "conv2d: the repacked filter matrix (%d taps x %d channels) exceeds the 2 GiB a buffer descriptor covers", rows, p.Mp);
-    const float *cached = nullptr;
-    {
+    const float *cached = gemm ? gemm->Wp : nullptr;
+    if (!gemm) {
         std::lock_guard<std::mutex> lock(g_cache_mutex);
         for (CachedFilters &e : g_cache[dev]) {
             if (e.K == K && e.Kf == Kf && e.C == C && e.R == R && e.S == S && rows <= e.rows) {
@@ -1756,6 +1982,12 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     }
     p.Wp = cached ? cached : (const float *)ws;
     p.wp_bytes = (unsigned)((size_t)rows * p.Mp * sizeof(float));
+    if (gemm) {
+        EH_REQUIRE(v->cpb != 0 && gemm->stride == (size_t)rows * p.Mp && p.PQ % v->bn == 0,
+                   "conv2d: internal error, the product launch of a Winograd convolution does not fit its operands");
+        EH_REQUIRE(wp_bytes + taps_bytes + partial_bytes <= WINO_INNER_RESERVE, "conv2d: internal error, workspace of a product launch");
+        p.w_img_stride = gemm->stride;
+    }
     p.taps = (const int32x4 *)((char *)ws + wp_bytes);
     p.partial = (float *)((char *)ws + wp_bytes + taps_bytes);
     if (taps_bytes) {
@@ -1774,6 +2006,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
         q.I = I + (size_t)b0 * img_elems;
         q.I2 = p.I2 + (size_t)b0 * img_elems;
         q.O = O + (size_t)b0 * Kf * p.PQ;
+        q.Wp = p.Wp + (size_t)b0 * p.w_img_stride;
         if (residual) q.residual = residual + (size_t)b0 * Kf * p.PQ;
         q.npix = (long long)nb * p.PQ;
         q.in_bytes = (unsigned)((size_t)nb * img_elems * sizeof(float));
@@ -1798,6 +2031,95 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     }
     if (leftover > 0) snprintf(g_last_kernel, sizeof(g_last_kernel), "%s +ksplit(%lld tiles x %d)", v->name, leftover, nslices);
     else snprintf(g_last_kernel, sizeof(g_last_kernel), "%s", v->name);
+    return 0;
+}
+
+// The Winograd form of a 3x3 stride-1 convolution (kernels and algebra above): filter transform (kept with a registered
+// filter tensor), input transform, ONE product launch through conv2d_fwd_impl (16 images of C channels and Tp pixels, a
+// planned or searched 1x1 launch like any other), output transform with the convolution's epilogue.
+// Workspace: [what the product launch may take][transformed filters unless kept][V][M].
+int conv2d_winograd(int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C, int H, int W,
+                    int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
+                    const float *bn_var, float bn_eps, const float *residual, int relu) {
+    hipStream_t st = state(dev).stream;
+    const int th = (P + 1) / 2, tw = (Q + 1) / 2;
+    const int T = N * th * tw, Tp = (T + 127) / 128 * 128;
+    const int rows = (C + 15) / 16 * 16, Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
+    const size_t u_floats = (size_t)16 * rows * Mp, v_floats = (size_t)16 * C * Tp, m_floats = (size_t)16 * Kf * Tp;
+    EH_REQUIRE((size_t)rows * Mp * sizeof(float) < ((size_t)1 << 31), "conv2d: the transformed filter matrix (%d x %d) exceeds 2 GiB", rows, Mp);
+
+    // ---- transformed filters: the registered copy (made here on first use, refreshed when the filters were written), or a
+    // transform into the workspace
+    const float *U = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_cache_mutex);
+        for (CachedFilters &e : g_cache[dev]) {
+            if (e.K == K && e.Kf == Kf && e.C == C && e.R == 3 && e.S == 3) {
+                if (e.Wwino == nullptr && !state(dev).capturing) {
+                    if (hipMalloc((void **)&e.Wwino, u_floats * sizeof(float)) != hipSuccess) {
+                        e.Wwino = nullptr;
+                        (void)hipGetLastError();
+                        break;  // no room to keep them: transform per call
+                    }
+                    e.wino_rows = rows;
+                    e.stale = true;
+                }
+                if (e.Wwino != nullptr) {
+                    if (e.stale) EH_TRY(repack(dev, e));
+                    U = e.Wwino;
+                }
+                break;
+            }
+        }
+    }
+    const size_t u_bytes = U ? 0 : ((u_floats * sizeof(float) + 255) & ~(size_t)255);
+    const size_t v_bytes = (v_floats * sizeof(float) + 255) & ~(size_t)255, m_bytes = (m_floats * sizeof(float) + 255) & ~(size_t)255;
+    void *ws = nullptr;
+    EH_TRY(get_workspace(dev, WINO_INNER_RESERVE + u_bytes + v_bytes + m_bytes, &ws));
+    char *base = (char *)ws + WINO_INNER_RESERVE;
+    float *Uw = (float *)base, *V = (float *)(base + u_bytes), *M = (float *)(base + u_bytes + v_bytes);
+    if (U == nullptr) {
+        hipLaunchKernelGGL(wino_filter_kernel, dim3((unsigned)(((size_t)rows * Mp + 255) / 256)), dim3(256), 0, st, K, Uw, Kf, C, Mp, rows);
+        EH_CHECK_LAUNCH();
+        U = Uw;
+    }
+
+    // ---- input transform
+    WinoParams w;
+    w.I = I; w.I2 = I2 ? I2 : I; w.Csplit = I2 ? C / 2 : C; w.Cimg = I2 ? C / 2 : C;
+    w.uh = uh; w.uw = uw;
+    w.C = C; w.H = H; w.W = W; w.pt = pad_top; w.pl = pad_left;
+    w.th = th; w.tw = tw; w.T = T; w.Tp = Tp;
+    w.V = V;
+    hipLaunchKernelGGL(wino_input_kernel, dim3((unsigned)((T + 255) / 256), (unsigned)((C + WINO_CH - 1) / WINO_CH)), dim3(256), 0, st, w);
+    EH_CHECK_LAUNCH();
+
+    // ---- the 16 products: M[xi] = U[xi] x V[xi]
+    {
+        const GemmBatch gb = {U, (size_t)rows * Mp};
+        const int ft = g_force_tile, fs = g_force_slices;
+        g_force_tile = -1;
+        g_force_slices = -1;
+        const int rc = conv2d_fwd_impl(false, dev, V, nullptr, 1, 1, K, nullptr, M, 16, C, 1, Tp, Kf, 1, 1, 1, 1, 0, 0, 1, Tp, nullptr, nullptr, nullptr,
+                                       nullptr, 0.0f, nullptr, 0, &gb);
+        g_force_tile = ft;
+        g_force_slices = fs;
+        if (rc != 0) return rc;
+    }
+
+    // ---- output transform + epilogue
+    ConvParams p;
+    memset(&p, 0, sizeof(p));
+    p.O = O;
+    p.bias = bias; p.bn_g = bn_g; p.bn_b = bn_b; p.bn_mean = bn_mean; p.bn_var = bn_var; p.residual = residual;
+    p.bn_eps = bn_eps; p.relu = relu;
+    p.N = N; p.Kf = Kf; p.P = P; p.Q = Q; p.PQ = P * Q;
+    hipLaunchKernelGGL(wino_output_kernel, dim3((unsigned)((T + 255) / 256), (unsigned)((Kf + WINO_CH - 1) / WINO_CH)), dim3(256), 0, st, p,
+                       (const float *)M, th, tw, T, Tp);
+    EH_CHECK_LAUNCH();
+    char inner[sizeof(g_last_kernel)];
+    snprintf(inner, sizeof(inner), "%s", g_last_kernel);
+    snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%.100s, %d blocks]", inner, Tp);
     return 0;
 }
 

@@ -207,9 +207,22 @@ int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const fl
  * 3 = MFMA with the operand slices staged through registers; 4 = MFMA with the operand slices
  * written by the load unit straight into LDS (what 0 and 1 select); 5 / 6 = switch off / on the
  * division along K of the tiles left over after a whole number of tiles per CU (on by default;
- * independent of 0-4).
+ * independent of 0-4); 7 / 8 = switch on / off the Winograd form for every convolution it applies to
+ * (off by default; independent of 5 / 6; only under 0).
+ *
+ * The Winograd form, F(2x2, 3x3): a 3x3 stride-1 convolution (any paddings, one or two input tensors, stored or
+ * upsampled image) computed as an input transform, 16 products of [Kf x C] by [C x blocks of 2x2 outputs] matrices -
+ * one launch of the 1x1 MFMA kernel - and an output transform that carries the fused epilogue: 2.25 times fewer
+ * multiplications, the role of the WINOGRAD algorithms among those the reference lets cuDNN choose from
+ * (src/hardware/gpu/nn/gpu_conv.cu:42-66).  Sums run in a fixed order (reproducible) and differ from the direct form's
+ * by rounding: the result meets the same tolerance against the reference's CPU convolution, it is not bit-identical to
+ * the direct form.  It takes workspace (16/4 of the input and of the output, plus 256 MB for its product launch), so
+ * eddlhip_conv2d_fwd_noalloc never uses it.  Chosen per geometry by the plan search (below) where it is faster, or
+ * everywhere by 7, or by eddlhip_conv2d_force_plan(4, .).
+ *
  * eddlhip_conv2d_last_kernel() names the kernel the calling thread's last eddlhip_conv2d_fwd
- * launched, followed by " +ksplit(T tiles x S)" when T tiles were divided into S slices. */
+ * launched, followed by " +ksplit(T tiles x S)" when T tiles were divided into S slices; for the Winograd form
+ * "winograd[<kernel and plan of the product launch>, <blocks per product> blocks]". */
 int eddlhip_conv2d_set_algo(int algo);
 const char *eddlhip_conv2d_last_kernel(void);
 
@@ -238,7 +251,8 @@ int eddlhip_conv2d_tuned_load(int dev, const char *host_path);
 /* Overrides the launch planner of the MFMA kernels (tuning and tests): tile = 0 (128x128 outputs per
  * workgroup), 1 (64x128), 2 (64x64), 3 (32x128) or -1 to give the choice back to the planner;
  * slices = number of K slices the tiles left over after a whole number per CU are divided into
- * (1 = none). */
+ * (1 = none).  tile = 4: the Winograd form wherever it applies (its product launch is planned or searched as usual),
+ * the planner's choice elsewhere. */
 int eddlhip_conv2d_force_plan(int tile, int slices);
 
 /* Filters that stay fixed between calls (inference).  Every eddlhip_conv2d_fwd first repacks its

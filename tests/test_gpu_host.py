@@ -188,11 +188,12 @@ def test_cpp_host_runs_the_plans_a_python_process_saved(hip, tmp_path):
         m.build(hip, fuse=True)
         hip.conv_autotune(True)
         m.predict([x])
-        assert hip.conv_tuned_plans() == 1
+        assert hip.conv_tuned_plans() in (1, 2)      # the convolution, and the product launch of its Winograd form
         hip.conv_tuned_save(plans)
         lines = open(plans).read().splitlines()
         keys = [l.split("|")[0] for l in lines if l and not l.startswith("#")]
-        assert len(keys) == 1 and keys[0].split()[:3] == [str(batch), str(ch), str(ch)], lines
+        keys = [k for k in keys if k.split()[:5] == [str(batch), str(ch), str(ch), "3", "3"]]
+        assert len(keys) == 1, lines
         for plan in ("2 1", "2 4"):
             with open(plans + plan[-1], "w") as f:
                 f.write("# rewritten by the test\n" + keys[0] + "| " + plan + "\n")

@@ -346,6 +346,106 @@ def test_conv2d_upsampled_input_equals_conv_of_the_resized_tensor(hip, oracle, a
         hip.conv2D(x, hip.array(np.zeros((6, 4, 3, 3), np.float32)), None, hip.empty((1, 6, 4, 4)), 1, 1, 0, 0, upsample=(0, 2))
 
 
+WINOGRAD_CASES = [
+    # N, C (all input channels), H, W (stored), Kf, (pad top, pad left), (P, Q) or None, bias, bn, residual, relu, two tensors, upsampling
+    (2, 16, 8, 8, 32, (1, 1), None, False, False, False, False, False, None),
+    (1, 5, 9, 7, 7, (1, 1), None, True, False, False, True, False, None),            # odd output sizes, ragged channels and filters
+    (3, 32, 14, 14, 64, (1, 1), None, False, True, True, True, False, None),         # the whole fused epilogue
+    (2, 24, 13, 17, 40, (0, 0), None, True, False, False, False, False, None),       # no padding
+    (2, 24, 12, 16, 40, (2, 1), None, False, True, False, False, False, None),       # a folded Pad layer: unequal paddings
+    (2, 8, 10, 10, 16, (0, 0), (9, 9), False, False, False, False, False, None),     # zero rows below and right of the image only
+    (2, 32, 12, 12, 48, (1, 1), None, False, True, False, True, True, None),         # a folded Concat
+    (2, 16, 6, 5, 24, (1, 1), None, True, False, False, False, False, (2, 2)),       # a folded UpSampling2D
+    (1, 16, 6, 6, 24, (0, 0), (11, 11), False, False, False, False, False, (2, 3)),
+    (4, 256, 28, 28, 256, (1, 1), None, False, True, False, True, False, None),      # a long channel sum
+]
+
+
+@pytest.mark.parametrize("case", WINOGRAD_CASES, ids=lambda c: "x".join(str(v) for v in c[:5]))
+def test_conv2d_winograd_form_against_oracle(hip, oracle, case):
+    """The Winograd form (force_conv_plan(4, .)) against the CPU oracle's direct convolution of the same logical input
+    (concatenated / resized / zero-padded on the host), to the convolution tolerance; the epilogue after it is the
+    oracle's, step by step."""
+    N, C, H, W, Kf, (pt, pl), out, use_bias, use_bn, use_res, relu, two, up = case
+    rng = np.random.default_rng(77)
+    Ci = C // 2 if two else C
+    a = rng.standard_normal((N, Ci, H, W), dtype=np.float32)
+    b = rng.standard_normal((N, Ci, H, W), dtype=np.float32) if two else None
+    w = (rng.standard_normal((Kf, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32)
+    logical = np.concatenate([a, b], axis=1) if two else a
+    if up:
+        logical = np.repeat(np.repeat(logical, up[0], axis=2), up[1], axis=3)
+    Hu, Wu = logical.shape[2:]
+    P, Q = out or (Hu + 2 * pt - 2, Wu + 2 * pl - 2)
+    # the output size fixes how many zero rows / columns follow the image
+    padded = np.zeros((N, C, P + 2, Q + 2), np.float32)
+    ys, xs = min(Hu, P + 2 - pt), min(Wu, Q + 2 - pl)
+    padded[:, :, pt:pt + ys, pl:pl + xs] = logical[:, :, :ys, :xs]
+    bias = rng.standard_normal(Kf, dtype=np.float32) if use_bias else None
+    bn = _bn_params(rng, Kf) if use_bn else None
+    res = rng.standard_normal((N, Kf, P, Q), dtype=np.float32) if use_res else None
+    ref = oracle.conv2d(padded, w, bias, (1, 1), 0, 0, P, Q)
+    if bn is not None:
+        g, bb, mean, var, eps = bn
+        ref, _, _ = oracle.batchnorm_inference(ref, mean, var, g, bb, eps)
+    if res is not None:
+        ref = oracle.add(ref, res)
+    if relu:
+        ref = oracle.relu(ref)
+    O = hip.full((N, Kf, P, Q), 3.0)
+    dbn = (hip.array(bn[0]), hip.array(bn[1]), hip.array(bn[2]), hip.array(bn[3]), bn[4]) if bn else None
+    hip.force_conv_plan(4, 1)
+    try:
+        hip.conv2D(hip.array(a), hip.array(w), hip.array(bias) if use_bias else None, O, 1, 1, pt, pl, bn=dbn,
+                   residual=hip.array(res) if use_res else None, relu=relu, second=hip.array(b) if two else None, upsample=up)
+        name = hip.last_conv_kernel()
+    finally:
+        hip.force_conv_plan(-1, 1)
+    assert name.startswith("winograd["), name
+    assert_conv_close(ref, O.numpy(), "winograd %s" % (case,))
+
+
+def test_conv2d_winograd_form_only_where_it_applies_and_with_kept_filters(hip, oracle):
+    """Strides other than one and filters other than 3x3 keep the direct form under force_conv_plan(4, .) and set_conv_algo
+    ("winograd"); registered filters keep their transformed copy, which follows writes to the filter tensor; the call that
+    cannot allocate never takes the Winograd form."""
+    rng = np.random.default_rng(78)
+    x = rng.standard_normal((2, 16, 12, 12), dtype=np.float32)
+    w3 = (rng.standard_normal((32, 16, 3, 3)) * 0.1).astype(np.float32)
+    w1 = (rng.standard_normal((32, 16, 1, 1)) * 0.1).astype(np.float32)
+    hip.set_conv_algo("winograd")
+    try:
+        ref, out = run_conv(hip, oracle, x, w3, None, (2, 2), "same", algo=7)
+        assert not hip.last_conv_kernel().startswith("winograd") and (assert_conv_close(ref, out, "stride 2") is None)
+        ref, out = run_conv(hip, oracle, x, w1, None, (1, 1), "valid", algo=7)
+        assert not hip.last_conv_kernel().startswith("winograd") and (assert_conv_close(ref, out, "1x1") is None)
+        ref, out = run_conv(hip, oracle, x, w3, None, (1, 1), "same", algo=7)
+        assert hip.last_conv_kernel().startswith("winograd") and (assert_conv_close(ref, out, "3x3") is None)
+        # kept filters: the transformed copy is made on first use and redone after a write
+        X, Wd, O = hip.array(x), hip.array(w3), hip.empty((2, 32, 12, 12))
+        hip.cache_conv_filters(Wd)
+        hip.set_conv_algo(7)
+        hip.conv2D(X, Wd, None, O, 1, 1, 1, 1)
+        assert hip.last_conv_kernel().startswith("winograd")
+        first = O.numpy()
+        assert_conv_close(oracle.conv2d(x, w3, None, (1, 1), 1, 1, 12, 12), first, "kept filters")
+        Wd.copy_from(2.0 * w3)
+        hip.conv2D(X, Wd, None, O, 1, 1, 1, 1)
+        assert np.array_equal(O.numpy(), 2.0 * first)      # doubling is exact in every step of the transforms
+        # the entry point over the fixed scratch array keeps the direct form
+        O2, O3 = hip.empty((2, 32, 12, 12)), hip.empty((2, 32, 12, 12))
+        hip._check(hip.lib.eddlhip_conv2d_fwd_noalloc(hip.dev, X.ptr, Wd.ptr, None, O2.ptr, 2, 16, 12, 12, 32, 3, 3, 1, 1, 1, 1, 12, 12,
+                                                      None, None, None, None, 0.0, None, 0))
+        assert not hip.last_conv_kernel().startswith("winograd")
+        hip.set_conv_algo("winograd_off")
+        hip.conv2D(X, Wd, None, O3, 1, 1, 1, 1)
+        assert np.array_equal(O2.numpy(), O3.numpy())
+        hip.uncache_conv_filters(Wd)
+    finally:
+        hip.set_conv_algo("winograd_off")
+        hip.set_conv_algo("auto")
+
+
 def test_conv2d_linearity_and_empty_batch(hip, oracle):
     from eddl_amd.descriptors import ConvolDescriptor
     rng = np.random.default_rng(301)
@@ -728,10 +828,11 @@ def test_conv2d_autotune_searches_once_per_geometry_and_stays_within_tolerance(h
         hip.conv_autotune(True)
         before = hip.conv_tuned_plans()
         hip.conv2D(dx, dw, None, O, 1, 1, 1, 1)
-        assert hip.conv_tuned_plans() == before + 1
+        after = hip.conv_tuned_plans()
+        assert after in (before + 1, before + 2)             # the geometry itself, and the product launch of its Winograd form
         first = O.numpy()
         hip.conv2D(dx, dw, None, O, 1, 1, 1, 1)
-        assert hip.conv_tuned_plans() == before + 1          # same geometry: no second search
+        assert hip.conv_tuned_plans() == after               # same geometry: no second search
         assert np.array_equal(O.numpy(), first)
         ref = oracle.conv2d(x, w, None, (1, 1), 1, 1, H, W, algo="im2col")
         assert np.all(np.abs(first - ref) <= 1e-5 * float(np.abs(ref).max()) + 1e-4 * np.abs(ref))
@@ -740,7 +841,7 @@ def test_conv2d_autotune_searches_once_per_geometry_and_stays_within_tolerance(h
         hip.batchnorm_inference(O, Y, opa, bn[2], bn[3], bn[0], bn[1], sd, 1e-5)
         F = hip.empty((N, Kf, H, W))
         hip.conv2D(dx, dw, None, F, 1, 1, 1, 1, bn=bn)
-        assert hip.conv_tuned_plans() == before + 1
+        assert hip.conv_tuned_plans() == after
         assert np.array_equal(F.numpy(), Y.numpy())
     finally:
         hip.conv_autotune(-1)
