@@ -44,6 +44,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <mutex>
 #include <utility>
 #include <vector>
@@ -1155,8 +1156,104 @@ __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restric
     }
 }
 
+// V = B^T d B of one patch, written to the 16 planes (`plane` floats apart) at dst
+__device__ __forceinline__ void wino_input_store(const float (&d)[16], float *dst, size_t plane) {
+    float u[16];  // B^T d
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        u[0 + j] = __fsub_rn(d[0 + j], d[8 + j]);
+        u[4 + j] = __fadd_rn(d[4 + j], d[8 + j]);
+        u[8 + j] = __fsub_rn(d[8 + j], d[4 + j]);
+        u[12 + j] = __fsub_rn(d[4 + j], d[12 + j]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {  // (B^T d) B
+        dst[(size_t)(4 * i + 0) * plane] = __fsub_rn(u[4 * i + 0], u[4 * i + 2]);
+        dst[(size_t)(4 * i + 1) * plane] = __fadd_rn(u[4 * i + 1], u[4 * i + 2]);
+        dst[(size_t)(4 * i + 2) * plane] = __fsub_rn(u[4 * i + 2], u[4 * i + 1]);
+        dst[(size_t)(4 * i + 3) * plane] = __fsub_rn(u[4 * i + 1], u[4 * i + 3]);
+    }
+}
+
+// The input transform with the image rows staged through LDS.  A workgroup takes 256 consecutive blocks, i.e. a run of
+// whole rows of blocks in one image or a few small images, and `chans` channels.  Once per workgroup it writes, for every
+// LDS slot (a pixel of the zero-padded, possibly upsampled rows its blocks touch; a row holds 2 tw + 2 pixels, the
+// first being column -pad_left), where that pixel lies in a channel plane, or that it does not exist.  Then per channel:
+// the slots are filled with coalesced loads - every pixel once, where the kernel below reads each four times through
+// the cache with half of every line unused -, a thread reads its 4x4 patch from LDS, transforms and stores as below.
+template <int KMAX>  // a thread fills at most KMAX slots: slots <= 256 * KMAX
+__global__ __launch_bounds__(256) void wino_input_lds_kernel(const WinoParams w, int slots, int chans) {
+    extern __shared__ int wino_lds[];
+    int *soff = wino_lds;
+    float *sval = reinterpret_cast<float *>(wino_lds + slots);
+    const int tid = threadIdx.x;
+    const int t0 = blockIdx.x * 256, t1 = min(t0 + 256, w.T), t = t0 + tid;
+    const int per_img = w.th * w.tw, LW = 2 * w.tw + 2;
+    const unsigned Hu = (unsigned)(w.H * w.uh), Wu = (unsigned)(w.W * w.uw);
+    const int n_first = t0 / per_img;
+    const int img_elems = w.Cimg * w.H * w.W;
+    const int my_n = t / per_img, my_r = t - my_n * per_img, my_ty = my_r / w.tw, my_tx = my_r - my_ty * w.tw;
+    int my_base = 0, total = 0;
+    for (int n = n_first; n * per_img < t1; n++) {  // the images this workgroup's blocks lie in (uniform)
+        const int a = max(t0, n * per_img) - n * per_img, b = min(t1, (n + 1) * per_img) - n * per_img;
+        const int ty_a = a / w.tw, ty_b = (b - 1) / w.tw;
+        const int cells = (2 * (ty_b - ty_a) + 4) * LW;
+        const int y_first = 2 * ty_a - w.pt, img_off = (n - n_first) * img_elems;
+        for (int i = tid; i < cells; i += 256) {
+            const int r = i / LW, xl = i - r * LW;
+            const unsigned y = (unsigned)(y_first + r), x = (unsigned)(xl - w.pl);
+            soff[total + i] = (y < Hu && x < Wu) ? img_off + (int)(y / (unsigned)w.uh) * w.W + (int)(x / (unsigned)w.uw) : -1;
+        }
+        if (my_n == n) my_base = total + 2 * (my_ty - ty_a) * LW + 2 * my_tx;
+        total += cells;
+    }
+    __syncthreads();
+    const size_t hw = (size_t)w.H * w.W, plane = (size_t)w.C * w.Tp;
+    const int c0 = blockIdx.y * chans, c1 = min(c0 + chans, w.C);
+    auto plane_of = [&](int c) {
+        return c < w.Csplit ? w.I + ((size_t)n_first * w.Cimg + c) * hw : w.I2 + ((size_t)n_first * w.Cimg + (c - w.Csplit)) * hw;
+    };
+    // the next channel's pixels are requested while this channel's patches are transformed and stored
+    float pre[KMAX];
+    auto fetch = [&](int c) {
+        const float *src = plane_of(c);
+#pragma unroll
+        for (int k = 0; k < KMAX; k++) {
+            const int i = tid + 256 * k;
+            pre[k] = 0.0f;
+            if (i < total) {
+                const int o = soff[i];
+                if (o >= 0) pre[k] = src[o];
+            }
+        }
+    };
+    fetch(c0);
+    for (int c = c0; c < c1; c++) {
+#pragma unroll
+        for (int k = 0; k < KMAX; k++)
+            if (tid + 256 * k < total) sval[tid + 256 * k] = pre[k];
+        __syncthreads();
+        if (c + 1 < c1) fetch(c + 1);
+        if (t < t1) {
+            float d[16];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {  // (rows and the patch's first column are at even slots)
+                const float2 lo = *reinterpret_cast<const float2 *>(sval + my_base + i * LW);
+                const float2 hi = *reinterpret_cast<const float2 *>(sval + my_base + i * LW + 2);
+                d[4 * i + 0] = lo.x;
+                d[4 * i + 1] = lo.y;
+                d[4 * i + 2] = hi.x;
+                d[4 * i + 3] = hi.y;
+            }
+            wino_input_store(d, w.V + (size_t)c * w.Tp + t, plane);
+        }
+        __syncthreads();
+    }
+}
+
 // One thread: one 2x2 output block (its 4x4 input patch) for WINO_CH channels; lanes hold consecutive blocks, so the 16
 // stores of a channel are 16 coalesced rows.  The patch offsets and which of its pixels exist are worked out once.
+// (The general form: taken where the staged kernel's tables would not fit.)
 __global__ __launch_bounds__(256) void wino_input_kernel(const WinoParams w) {
     const int t = blockIdx.x * 256 + threadIdx.x;
     if (t >= w.T) return;
@@ -1187,22 +1284,7 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const WinoParams w) {
         float d[16];
 #pragma unroll
         for (int e = 0; e < 16; e++) d[e] = ((mask >> e) & 1u) ? src[off[e]] : 0.0f;
-        float u[16];  // B^T d
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            u[0 + j] = __fsub_rn(d[0 + j], d[8 + j]);
-            u[4 + j] = __fadd_rn(d[4 + j], d[8 + j]);
-            u[8 + j] = __fsub_rn(d[8 + j], d[4 + j]);
-            u[12 + j] = __fsub_rn(d[4 + j], d[12 + j]);
-        }
-        float *dst = w.V + (size_t)c * w.Tp + t;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {  // (B^T d) B
-            dst[(size_t)(4 * i + 0) * plane] = __fsub_rn(u[4 * i + 0], u[4 * i + 2]);
-            dst[(size_t)(4 * i + 1) * plane] = __fadd_rn(u[4 * i + 1], u[4 * i + 2]);
-            dst[(size_t)(4 * i + 2) * plane] = __fsub_rn(u[4 * i + 2], u[4 * i + 1]);
-            dst[(size_t)(4 * i + 3) * plane] = __fsub_rn(u[4 * i + 1], u[4 * i + 3]);
-        }
+        wino_input_store(d, w.V + (size_t)c * w.Tp + t, plane);
     }
 }
 
@@ -2091,7 +2173,24 @@ int conv2d_winograd(int dev, const float *I, const float *I2, int uh, int uw, co
     w.C = C; w.H = H; w.W = W; w.pt = pad_top; w.pl = pad_left;
     w.th = th; w.tw = tw; w.T = T; w.Tp = Tp;
     w.V = V;
-    hipLaunchKernelGGL(wino_input_kernel, dim3((unsigned)((T + 255) / 256), (unsigned)((C + WINO_CH - 1) / WINO_CH)), dim3(256), 0, st, w);
+    {
+        // LDS slots of the staged kernel, an upper bound over its workgroups: 256 blocks lie in at most `segs` images and
+        // 256 / tw whole rows of blocks, plus a partial row at either end of every image's run; a run of r rows of blocks
+        // touches 2 r + 2 pixel rows of 2 tw + 2 slots
+        const long long per_img = (long long)th * tw;
+        const long long segs = std::min<long long>(N, 256 / per_img + 2);
+        const long long block_rows = 256 / tw + 2 * segs;
+        const long long slots = ((2 * block_rows + 2 * segs) * (2 * tw + 2) + 1) & ~1LL;
+        const long long img_elems = (long long)w.Cimg * H * W;
+        constexpr int chans = 8;
+        if (slots <= 256 * 16 && segs * img_elems < 0x7fffffffLL) {
+            const dim3 grid((unsigned)((T + 255) / 256), (unsigned)((C + chans - 1) / chans));
+            if (slots <= 256 * 8) hipLaunchKernelGGL(wino_input_lds_kernel<8>, grid, dim3(256), (size_t)slots * 8, st, w, (int)slots, chans);
+            else hipLaunchKernelGGL(wino_input_lds_kernel<16>, grid, dim3(256), (size_t)slots * 8, st, w, (int)slots, chans);
+        } else {
+            hipLaunchKernelGGL(wino_input_kernel, dim3((unsigned)((T + 255) / 256), (unsigned)((C + WINO_CH - 1) / WINO_CH)), dim3(256), 0, st, w);
+        }
+    }
     EH_CHECK_LAUNCH();
 
     // ---- the 16 products: M[xi] = U[xi] x V[xi]
