@@ -114,6 +114,10 @@ struct ConvParams {
     const int32x4 *taps;
     // eddlhip_conv2d_trace: eight 64-bit words per workgroup (see trace_mark), or nullptr
     unsigned long long *trace;
+    // conv_tap_kernel<..., WINO = true> (the 16 products of a Winograd convolution and its output transform in one
+    // launch): the K range is 16 runs of wspx steps, one per patch position; a pixel of the launch is a 2x2 block of the
+    // wP x wQ output planes, wth x wtw of them per image, wT in all (see wino_fold / wino_store_tile).
+    int wspx, wth, wtw, wT, wP, wQ;
 };
 
 // Timeline of a workgroup for eddlhip_conv2d_trace: words 0..3 = the device's constant 100 MHz clock at the marks (entry,
@@ -468,13 +472,92 @@ __global__ __launch_bounds__(256) void pack_filters_kernel(const float *__restri
     }
 }
 
+// ---------------------------------------------------------------- Winograd output transform inside the product launch
+// Y = A^T M A with A^T = [1 1 1 0; 0 1 -1 -1]: the product M of patch position xi = 4 i + j reaches output (a, b) of the
+// 2x2 block with the factor A^T[a][i] * A^T[b][j], which is 0, 1 or -1.  A workgroup that walks through all 16 positions
+// therefore needs no M tensor: after the K run of a position it adds the accumulator into four running outputs, with
+// those signs, and clears it.  Positions are taken in the order 0..15, so the sums are reproducible.
+__device__ __forceinline__ void wino_fold(floatx16 (&y)[2][2], floatx16 &acc, int xi) {
+    const int i = xi >> 2, j = xi & 3;
+    const int ca[2] = {i < 3 ? 1 : 0, i == 0 ? 0 : (i == 1 ? 1 : -1)};
+    const int cb[2] = {j < 3 ? 1 : 0, j == 0 ? 0 : (j == 1 ? 1 : -1)};
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const int f = ca[a] * cb[b];  // the same for every lane
+            if (f > 0) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) y[a][b][v] = __fadd_rn(y[a][b][v], acc[v]);
+            } else if (f < 0) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) y[a][b][v] = __fsub_rn(y[a][b][v], acc[v]);
+            }
+        }
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+}
+
+// A wavefront's 32 filters x 32 blocks: lane = block (column) lane % 32, filter rows 8 * (v / 4) + 4 * (lane / 32) + v % 4.
+// The convolution's epilogue value by value (the arithmetic of apply_epilogue), two outputs of a row per store where
+// the rows are aligned for it.  `epi`: the tile's channel constants (stage_channel_constants); m_local: the
+// wavefront's first row in the tile.
+template <int BM>
+__device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&y)[2][2], const float *epi, int m0, int m_local, int n_base,
+                                                int lane) {
+    const int n = n_base + (lane & 31);
+    if (n >= p.wT) return;
+    const int per_img = p.wth * p.wtw;
+    const int img = n / per_img, r = n - img * per_img, ty = r / p.wtw, tx = r - ty * p.wtw;
+    const size_t plane = (size_t)p.wP * p.wQ;
+    const bool pair = (p.wQ % 2 == 0) && (((size_t)p.O | (size_t)(p.residual ? p.residual : p.O)) % 8 == 0);
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const int ml = m_local + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+        if (m0 + ml >= p.Kf) continue;
+        const float bias = epi[ml], mean = epi[BM + ml], sd = epi[2 * BM + ml], g = epi[3 * BM + ml], b = epi[4 * BM + ml];
+#pragma unroll
+        for (int a = 0; a < 2; a++) {
+            const int oy = 2 * ty + a, ox = 2 * tx;
+            if (oy >= p.wP) continue;
+            const size_t oidx = ((size_t)img * p.Kf + (size_t)(m0 + ml)) * plane + (size_t)oy * p.wQ + ox;
+            float x0 = y[a][0][v], x1 = y[a][1][v];
+            float r0 = 0.0f, r1 = 0.0f;
+            if (p.residual) {
+                if (pair) {
+                    const float2 rr = *reinterpret_cast<const float2 *>(p.residual + oidx);
+                    r0 = rr.x;
+                    r1 = rr.y;
+                } else {
+                    r0 = p.residual[oidx];
+                    if (ox + 1 < p.wQ) r1 = p.residual[oidx + 1];
+                }
+            }
+            if (p.bias) x0 = __fadd_rn(x0, bias), x1 = __fadd_rn(x1, bias);
+            if (p.bn_mean) {
+                x0 = __fdiv_rn(__fsub_rn(x0, mean), sd), x1 = __fdiv_rn(__fsub_rn(x1, mean), sd);
+                if (p.bn_g) x0 = __fadd_rn(__fmul_rn(x0, g), b), x1 = __fadd_rn(__fmul_rn(x1, g), b);
+            }
+            if (p.residual) x0 = __fadd_rn(x0, r0), x1 = __fadd_rn(x1, r1);
+            if (p.relu) x0 = x0 > 0.0f ? x0 : 0.0f, x1 = x1 > 0.0f ? x1 : 0.0f;
+            if (pair) {
+                *reinterpret_cast<float2 *>(p.O + oidx) = make_float2(x0, x1);
+            } else {
+                p.O[oidx] = x0;
+                if (ox + 1 < p.wQ) p.O[oidx + 1] = x1;
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------- MFMA kernel, compile-time filter shape
 // K-step = CPB input channels x (R*S) taps.  Gather work is split by wavefront: a wavefront
 // serves one 64-pixel segment of the tile (its lanes = 64 consecutive output pixels) and CPW of
 // the step's channels; each of its loads is one (channel, tap) row segment of 64 floats.
-template <int WM, int WN, int TM, int TN, int R, int S, int CPB, bool DIRECT>
+template <int WM, int WN, int TM, int TN, int R, int S, int CPB, bool DIRECT, bool WINO = false>
 __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(const ConvParams p) {  // registers for 3 (4) workgroups per CU
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
+    static_assert(!WINO || (TM == 1 && TN == 1 && R == 1 && S == 1), "the Winograd products run on one 32x32 block per wavefront");
     constexpr int RS = R * S, BK = CPB * RS;
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
     constexpr int NS = BN / 64;     // 64-pixel segments in a tile row
@@ -717,9 +800,26 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     __syncthreads();
     trace_mark(p, 1);
 
+    floatx16 wy[WINO ? 2 : 1][WINO ? 2 : 1];  // WINO: the four outputs of every 2x2 block of this wavefront
+    int wino_left = p.wspx, wino_xi = 0;        // steps left in the current patch position's run
+    if constexpr (WINO) {
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) wy[a][b][v] = 0.0f;
+    }
     for (int step = step_lo; step < step_hi; step++) {
         const int buf = (step - step_lo) & 1;
         do_step(as_of(buf), bs_of(buf), as_of(buf ^ 1), bs_of(buf ^ 1), step, step + 1 < step_hi && !both);
+        if constexpr (WINO) {
+            if (--wino_left == 0) {  // this position's product is complete
+                wino_fold(wy, acc[0][0], wino_xi);
+                wino_xi++;
+                wino_left = p.wspx;
+            }
+        }
         // The barrier publishes the next buffer to the other wavefronts, so this wavefront's
         // LDS-direct loads into it must be complete first.
         if constexpr (DIRECT) __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -727,7 +827,13 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     }
 
     trace_mark(p, 2);
-    if (split) {
+    if constexpr (WINO) {
+        // (launched with whole tiles only)
+        float *epi = &As[0][0];
+        put_channel_constants<BM>(epi, chan, tid);
+        __syncthreads();
+        wino_store_tile<BM>(p, wy, epi, m0, wm * 32, (int)n0 + wn * 32, lane);
+    } else if (split) {
         store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
     } else {
         float *epi = &As[0][0];  // the K loop ended with a barrier: the filter buffers are free
@@ -1665,7 +1771,7 @@ int eddlhip_conv2d_uncache_filters(int dev, const float *K) {
 }
 
 int eddlhip_conv2d_force_plan(int tile, int slices) {
-    EH_REQUIRE(tile >= -1 && tile <= 4, "conv2d_force_plan: tile is -1 (automatic), 0..3 or 4 (the Winograd form where it applies)");
+    EH_REQUIRE(tile >= -1 && tile <= 5, "conv2d_force_plan: tile is -1 (automatic), 0..3, or 4 / 5 (the Winograd forms where they apply)");
     g_force_tile = tile;
     g_force_slices = slices;
     return 0;
@@ -1712,7 +1818,7 @@ int eddlhip_conv2d_tuned_load(int dev, const char *host_path) {
         int *k = t.key;
         const int got = sscanf(line, "%d %d %d %d %d %d %d %d %d %d | %d %d", k, k + 1, k + 2, k + 3, k + 4, k + 5, k + 6, k + 7, k + 8, k + 9, &t.tile,
                                &t.slices);
-        if (got != 12 || t.tile < -1 || t.tile > 4 || t.slices < 1 || t.slices > 64) {
+        if (got != 12 || t.tile < -1 || t.tile > 5 || t.slices < 1 || t.slices > 64) {
             bad = true;
             break;
         }
@@ -1793,8 +1899,8 @@ struct GemmBatch {
 // at most 16 slices each, 128 x 128 floats per tile.  The Winograd driver keeps its own buffers behind this much.
 constexpr size_t WINO_INNER_RESERVE = (size_t)16 * 255 * 128 * 128 * sizeof(float);
 
-int conv2d_winograd(int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C, int H, int W,
-                    int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
+int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C, int H,
+                    int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
                     const float *bn_var, float bn_eps, const float *residual, int relu);
 
 // Whether the Winograd form can run this convolution: 3x3, stride 1, and the product launch within the limits of
@@ -1803,6 +1909,13 @@ bool winograd_applies(int N, int C, int Kf, int R, int S, int sr, int sc, int P,
     if (R != 3 || S != 3 || sr != 1 || sc != 1) return false;
     const long long T = (long long)N * ((P + 1) / 2) * ((Q + 1) / 2), Tp = (T + 127) / 128 * 128;
     return Tp <= 0x3fffff80LL && (long long)C * Tp <= (1LL << 28) && (long long)Kf * Tp <= (1LL << 28);
+}
+// ... with the output transform folded into the product launch (one launch over all 16 positions: the transformed input is
+// then ONE image of 16 C channels, which a buffer descriptor must cover, and the channel runs must be whole K-steps)
+bool winograd_fold_applies(int N, int C, int Kf, int R, int S, int sr, int sc, int P, int Q) {
+    if (!winograd_applies(N, C, Kf, R, S, sr, sc, P, Q) || C % 16 != 0) return false;
+    const long long T = (long long)N * ((P + 1) / 2) * ((Q + 1) / 2), Tp = (T + 127) / 128 * 128;
+    return 16LL * C * Tp * 4 < (1LL << 31) && 16LL * C * ((Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN) * 4 < (1LL << 31);
 }
 
 int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
@@ -1932,9 +2045,10 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     // the Winograd form: asked for (force_plan(4, .), set_algo(7)) or found faster by the plan search (below); never from the
     // fixed scratch array, whose size it exceeds, and not for the scalar-order or register-staged algorithm switches
     const bool wino_ok = !gemm && !no_alloc && g_algo == 0 && winograd_applies(N, C, Kf, R, S, sr, sc, P, Q);
-    if (wino_ok && (g_force_tile == 4 || (g_wino && g_force_tile < 0 && !g_tuning)))
-        return conv2d_winograd(dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean, bn_var,
-                               bn_eps, residual, relu);
+    const bool fold_ok = wino_ok && winograd_fold_applies(N, C, Kf, R, S, sr, sc, P, Q);
+    if ((wino_ok && (g_force_tile == 4 || (g_wino && g_force_tile < 0 && !g_tuning))) || (fold_ok && g_force_tile == 5))
+        return conv2d_winograd(g_force_tile == 5, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b,
+                               bn_mean, bn_var, bn_eps, residual, relu);
     if (g_autotune && g_force_tile < 0 && g_algo == 0 && g_split != 0) {
         const int key[10] = {N, C, Kf, R, S, sr, sc, P, Q, direct};
         const TunedPlan *found = nullptr;
@@ -2005,6 +2119,11 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
                     best.tile = 4;
                     best.slices = 1;
                 }
+                if (fold_ok && measure(5, 1, &ms) == 0 && ms < best_ms && ms < 0.98f * planned_ms) {
+                    best_ms = ms;
+                    best.tile = 5;
+                    best.slices = 1;
+                }
             }
             g_tuning = false;
             (void)hipEventDestroy(e0);
@@ -2016,9 +2135,9 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
             g_tuned[dev].push_back(best);
             found = &g_tuned[dev].back();
         }
-        if (found != nullptr && found->tile == 4 && wino_ok)
-            return conv2d_winograd(dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean, bn_var,
-                                   bn_eps, residual, relu);
+        if (found != nullptr && ((found->tile == 4 && wino_ok) || (found->tile == 5 && fold_ok)))
+            return conv2d_winograd(found->tile == 5, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b,
+                                   bn_mean, bn_var, bn_eps, residual, relu);
         if (found != nullptr && found->tile >= 0 && found->tile < 4)
             plan = forced_plan(family, found->tile, found->slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
     }
@@ -2120,8 +2239,8 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
 // filter tensor), input transform, ONE product launch through conv2d_fwd_impl (16 images of C channels and Tp pixels, a
 // planned or searched 1x1 launch like any other), output transform with the convolution's epilogue.
 // Workspace: [what the product launch may take][transformed filters unless kept][V][M].
-int conv2d_winograd(int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C, int H, int W,
-                    int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
+int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C, int H,
+                    int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
                     const float *bn_var, float bn_eps, const float *residual, int relu) {
     hipStream_t st = state(dev).stream;
     const int th = (P + 1) / 2, tw = (Q + 1) / 2;
@@ -2155,7 +2274,8 @@ int conv2d_winograd(int dev, const float *I, const float *I2, int uh, int uw, co
         }
     }
     const size_t u_bytes = U ? 0 : ((u_floats * sizeof(float) + 255) & ~(size_t)255);
-    const size_t v_bytes = (v_floats * sizeof(float) + 255) & ~(size_t)255, m_bytes = (m_floats * sizeof(float) + 255) & ~(size_t)255;
+    const size_t v_bytes = (v_floats * sizeof(float) + 255) & ~(size_t)255;
+    const size_t m_bytes = fold ? 0 : ((m_floats * sizeof(float) + 255) & ~(size_t)255);  // folded: M is never written
     void *ws = nullptr;
     EH_TRY(get_workspace(dev, WINO_INNER_RESERVE + u_bytes + v_bytes + m_bytes, &ws));
     char *base = (char *)ws + WINO_INNER_RESERVE;
@@ -2192,6 +2312,33 @@ int conv2d_winograd(int dev, const float *I, const float *I2, int uh, int uw, co
         }
     }
     EH_CHECK_LAUNCH();
+
+    if (fold) {
+        // ---- the 16 products and the output transform in one launch: a 1x1 "convolution" of ONE image of 16 C channels
+        // and Tp pixels whose K range is 16 runs of C / 16 steps; conv_tap_kernel<..., WINO> folds each run's product
+        // into the four outputs of a block and finishes with the convolution's epilogue (64x64 tiles, whole tiles only)
+        ConvParams q;
+        memset(&q, 0, sizeof(q));
+        q.I = V; q.I2 = V; q.Csplit = 16 * C; q.Cimg = 16 * C; q.uh = 1; q.uw = 1;
+        q.Wp = U; q.w_img_stride = 0; q.K = K; q.O = O;
+        q.bias = bias; q.bn_g = bn_g; q.bn_b = bn_b; q.bn_mean = bn_mean; q.bn_var = bn_var; q.residual = residual;
+        q.bn_eps = bn_eps; q.relu = relu;
+        q.N = 1; q.C = 16 * C; q.H = 1; q.W = Tp; q.Kf = Kf; q.R = 1; q.S = 1; q.sr = 1; q.sc = 1; q.P = 1; q.Q = Tp;
+        q.CRS = 16 * C; q.Mp = Mp; q.nsteps = C; q.PQ = Tp; q.npix = Tp;
+        q.gm = (Kf + 63) / 64; q.gn = Tp / 64;
+        q.in_bytes = (unsigned)((size_t)16 * C * Tp * sizeof(float));
+        q.wp_bytes = (unsigned)((size_t)16 * rows * Mp * sizeof(float));
+        q.main_tiles = q.gm * q.gn; q.nslices = 1; q.slice_steps = q.nsteps;
+        q.wspx = C / 16; q.wth = th; q.wtw = tw; q.wT = T; q.wP = P; q.wQ = Q;
+        EH_REQUIRE(rows == C && (long long)q.gm * q.gn <= 0x3fffffffLL, "conv2d: internal error, folded Winograd launch");
+        q.trace = (g_trace != nullptr && q.main_tiles <= g_trace_wgs) ? g_trace : nullptr;
+        EH_TRY(prof_begin(st));
+        hipLaunchKernelGGL((conv_tap_kernel<2, 2, 1, 1, 1, 1, 16, true, true>), dim3((unsigned)q.main_tiles), dim3(256), 0, st, q);
+        EH_CHECK_LAUNCH();
+        EH_TRY(prof_end(st));
+        snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[conv_tap_kernel<2,2,1,1,1,1,16,true,true>, %d blocks]", Tp);
+        return 0;
+    }
 
     // ---- the 16 products: M[xi] = U[xi] x V[xi]
     {

@@ -218,7 +218,10 @@ int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const fl
  * by rounding: the result meets the same tolerance against the reference's CPU convolution, it is not bit-identical to
  * the direct form.  It takes workspace (16/4 of the input and of the output, plus 256 MB for its product launch), so
  * eddlhip_conv2d_fwd_noalloc never uses it.  Chosen per geometry by the plan search (below) where it is faster, or
- * everywhere by 7, or by eddlhip_conv2d_force_plan(4, .).
+ * everywhere by 7, or by eddlhip_conv2d_force_plan(4, .).  A second form, for input channel counts that are multiples of
+ * 16 (force_plan(5, .), or the search): one product launch walks through all 16 patch positions and folds each product
+ * into the outputs as it completes, so the products are never written and there is no output-transform launch; it sums
+ * the 16 positions in another order than the first form (same tolerance, not the same bits).
  *
  * eddlhip_conv2d_last_kernel() names the kernel the calling thread's last eddlhip_conv2d_fwd
  * launched, followed by " +ksplit(T tiles x S)" when T tiles were divided into S slices; for the Winograd form
@@ -252,7 +255,7 @@ int eddlhip_conv2d_tuned_load(int dev, const char *host_path);
  * workgroup), 1 (64x128), 2 (64x64), 3 (32x128) or -1 to give the choice back to the planner;
  * slices = number of K slices the tiles left over after a whole number per CU are divided into
  * (1 = none).  tile = 4: the Winograd form wherever it applies (its product launch is planned or searched as usual),
- * the planner's choice elsewhere. */
+ * 5: its folded form wherever that applies; the planner's choice elsewhere. */
 int eddlhip_conv2d_force_plan(int tile, int slices);
 
 /* Filters that stay fixed between calls (inference).  Every eddlhip_conv2d_fwd first repacks its

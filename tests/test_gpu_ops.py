@@ -351,9 +351,9 @@ WINOGRAD_CASES = [
     (2, 16, 8, 8, 32, (1, 1), None, False, False, False, False, False, None),
     (1, 5, 9, 7, 7, (1, 1), None, True, False, False, True, False, None),            # odd output sizes, ragged channels and filters
     (3, 32, 14, 14, 64, (1, 1), None, False, True, True, True, False, None),         # the whole fused epilogue
-    (2, 24, 13, 17, 40, (0, 0), None, True, False, False, False, False, None),       # no padding
-    (2, 24, 12, 16, 40, (2, 1), None, False, True, False, False, False, None),       # a folded Pad layer: unequal paddings
-    (2, 8, 10, 10, 16, (0, 0), (9, 9), False, False, False, False, False, None),     # zero rows below and right of the image only
+    (2, 48, 13, 17, 40, (0, 0), None, True, False, False, False, False, None),       # no padding
+    (2, 32, 12, 16, 40, (2, 1), None, False, True, False, False, False, None),       # a folded Pad layer: unequal paddings
+    (2, 16, 10, 10, 16, (0, 0), (9, 9), False, False, False, False, False, None),    # zero rows below and right of the image only
     (2, 32, 12, 12, 48, (1, 1), None, False, True, False, True, True, None),         # a folded Concat
     (2, 16, 6, 5, 24, (1, 1), None, True, False, False, False, False, (2, 2)),       # a folded UpSampling2D
     (1, 16, 6, 6, 24, (0, 0), (11, 11), False, False, False, False, False, (2, 3)),
@@ -361,11 +361,13 @@ WINOGRAD_CASES = [
 ]
 
 
+@pytest.mark.parametrize("form", [4, 5], ids=["three-kernels", "folded"])
 @pytest.mark.parametrize("case", WINOGRAD_CASES, ids=lambda c: "x".join(str(v) for v in c[:5]))
-def test_conv2d_winograd_form_against_oracle(hip, oracle, case):
-    """The Winograd form (force_conv_plan(4, .)) against the CPU oracle's direct convolution of the same logical input
-    (concatenated / resized / zero-padded on the host), to the convolution tolerance; the epilogue after it is the
-    oracle's, step by step."""
+def test_conv2d_winograd_form_against_oracle(hip, oracle, case, form):
+    """The Winograd forms (force_conv_plan(4, .): transforms and products as separate launches; 5: the output transform
+    folded into the one product launch, for channel counts that are whole K-steps) against the CPU oracle's direct
+    convolution of the same logical input (concatenated / resized / zero-padded on the host), to the convolution
+    tolerance; the epilogue after it is the oracle's, step by step."""
     N, C, H, W, Kf, (pt, pl), out, use_bias, use_bn, use_res, relu, two, up = case
     rng = np.random.default_rng(77)
     Ci = C // 2 if two else C
@@ -394,14 +396,17 @@ def test_conv2d_winograd_form_against_oracle(hip, oracle, case):
         ref = oracle.relu(ref)
     O = hip.full((N, Kf, P, Q), 3.0)
     dbn = (hip.array(bn[0]), hip.array(bn[1]), hip.array(bn[2]), hip.array(bn[3]), bn[4]) if bn else None
-    hip.force_conv_plan(4, 1)
+    hip.force_conv_plan(form, 1)
     try:
         hip.conv2D(hip.array(a), hip.array(w), hip.array(bias) if use_bias else None, O, 1, 1, pt, pl, bn=dbn,
                    residual=hip.array(res) if use_res else None, relu=relu, second=hip.array(b) if two else None, upsample=up)
         name = hip.last_conv_kernel()
     finally:
         hip.force_conv_plan(-1, 1)
-    assert name.startswith("winograd["), name
+    if form == 4 or C % 16 == 0:
+        assert name.startswith("winograd[") and ("true,true>" in name) == (form == 5), name
+    else:
+        assert not name.startswith("winograd["), name       # the folded form needs whole K-steps of channels: the direct form ran
     assert_conv_close(ref, O.numpy(), "winograd %s" % (case,))
 
 
