@@ -2332,11 +2332,20 @@ int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh,
         q.wspx = C / 16; q.wth = th; q.wtw = tw; q.wT = T; q.wP = P; q.wQ = Q;
         EH_REQUIRE(rows == C && (long long)q.gm * q.gn <= 0x3fffffffLL, "conv2d: internal error, folded Winograd launch");
         q.trace = (g_trace != nullptr && q.main_tiles <= g_trace_wgs) ? g_trace : nullptr;
+        // K-steps of 32 channels where the runs divide into them: a workgroup's K loop is long here (16 C channels), few
+        // workgroups share a CU (64 output registers per lane), and a step's matrix work then covers a trip to memory
+        const bool wide = C % 32 == 0;
+        if (wide) {
+            q.nsteps = C / 2;
+            q.slice_steps = q.nsteps;
+            q.wspx = C / 32;
+        }
         EH_TRY(prof_begin(st));
-        hipLaunchKernelGGL((conv_tap_kernel<2, 2, 1, 1, 1, 1, 16, true, true>), dim3((unsigned)q.main_tiles), dim3(256), 0, st, q);
+        if (wide) hipLaunchKernelGGL((conv_tap_kernel<2, 2, 1, 1, 1, 1, 32, true, true>), dim3((unsigned)q.main_tiles), dim3(256), 0, st, q);
+        else hipLaunchKernelGGL((conv_tap_kernel<2, 2, 1, 1, 1, 1, 16, true, true>), dim3((unsigned)q.main_tiles), dim3(256), 0, st, q);
         EH_CHECK_LAUNCH();
         EH_TRY(prof_end(st));
-        snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[conv_tap_kernel<2,2,1,1,1,1,16,true,true>, %d blocks]", Tp);
+        snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[conv_tap_kernel<2,2,1,1,1,1,%d,true,true>, %d blocks]", wide ? 32 : 16, Tp);
         return 0;
     }
 
