@@ -114,7 +114,8 @@ def trace(workload, trace_dir, log, out, extra=""):
               "  roofline kernel %s: %s launches/step, avg launch %.4f ms (HIP events inside bench.py), achieved %.2f %s = %.1f%% of %.1f"
               % (rf["kernel"], rf.get("launches_per_step"), rf.get("avg_launch_ms", 0.0), rf["achieved"], rf["unit"], 100 * rf["frac"], rf["peak"])]
         key = rf["kernel"].replace(" ", "")
-        dom = [r for r in stats if key in r["Name"].replace(" ", "")]
+        # (the trace spells out a kernel's defaulted last template argument, the library's name for it does not)
+        dom = [r for r in stats if key in r["Name"].replace(" ", "").replace(",false>", ">")]
         if dom:
             o.append("  same kernel in the trace above: average %.4f ms over %s calls" % (float(dom[0]["AverageNs"]) / 1e6, dom[0]["Calls"]))
     write(out, o, workload)
@@ -168,7 +169,7 @@ def traffic(workload, trace_dir, fetch_dir, write_dir, log, out, out_json=None, 
     write(out, o, workload)
     if out_json and bench:
         key = bench["roofline"]["kernel"].replace(" ", "")
-        m = [k for k in per_kernel if key in k.replace(" ", "")]
+        m = [k for k in per_kernel if key in k.replace(" ", "").replace(",false>", ">")]
         if m:
             with open(out_json, "w") as fh:
                 json.dump({"kernel": bench["roofline"]["kernel"], "hbm_bytes_per_launch": per_kernel[m[0]], "fetch_scale": sf, "write_scale": sw,
