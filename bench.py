@@ -230,9 +230,11 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, pl
             if kern.startswith("winograd["):
                 blocks = int(kern[kern.rindex(",") + 1:].split()[0])
                 kern = kern[len("winograd["):kern.rindex(",")]
+                conv = [l for l in op.layers if "cd" in l.attrs][0].attrs["cd"]
                 n_out, kf = op.layers[-1].out_shape[0] * op.layers[-1].out_shape[2] * op.layers[-1].out_shape[3], op.layers[-1].out_shape[1]
-                c_in = op.flops // (18 * n_out * kf)
-                kernel_flops, form = 32 * kf * c_in * blocks, "winograd_f2x2_3x3"
+                c_in = op.flops // (2 * conv.kr * conv.kc * n_out * kf)
+                positions = (conv.kr + 1) * (conv.kc + 1)          # 16 products for a 3x3 filter, 9 for a 2x2 one
+                kernel_flops, form = 2 * positions * kf * c_in * blocks, "winograd"
             row.update(kernel=kern.split(" +ksplit")[0], kernel_ms=kms, kernel_launches=kl, kernel_flops=kernel_flops, form=form)
         if op.kind in ("conv2d", "dense") and ms > 0:
             row["tflops"] = op.flops / ms / 1e9
@@ -288,7 +290,7 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, pl
                "conv_total": {"tflops": conv_flops / conv_ms / 1e9 if conv_ms else 0.0, "ms": conv_ms, "gflop": conv_flops / 1e9,
                               "frac_fp32_mfma_peak": (conv_flops / conv_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS) if conv_ms else 0.0,
                               "flops_counted": "direct form", "layers": len(conv_rows),
-                              "winograd_layers": sum(1 for r in conv_rows if r.get("form") == "winograd_f2x2_3x3")},
+                              "winograd_layers": sum(1 for r in conv_rows if r.get("form") == "winograd")},
                "device_ms_sum_of_ops": sum(op_ms)}
     del model
     return summary, rows, out_host, desc
@@ -419,7 +421,7 @@ def main():
         table.append("%-44s %9.4f %9s %8s %9.1f %7.2f  %s" % (
             r["name"][:44], r["ms"], "%.2f" % r["tflops"] if "tflops" in r else "-",
             "%.1f" % (100 * r["frac_fp32_mfma_peak"]) if "tflops" in r else "-", r.get("gbs", 0.0), 100 * r.get("frac_hbm_peak", 0.0),
-            ("winograd: " if r.get("form") == "winograd_f2x2_3x3" else "") + r.get("kernel", "")))
+            ("winograd: " if r.get("form") == "winograd" else "") + r.get("kernel", "")))
     if args.layers:
         print("\n".join(table), file=sys.stderr)
     out_dir = args.out

@@ -118,6 +118,7 @@ struct ConvParams {
     // launch): the K range is 16 runs of wspx steps, one per patch position; a pixel of the launch is a 2x2 block of the
     // wP x wQ output planes, wth x wtw of them per image, wT in all (see wino_fold / wino_store_tile).
     int wspx, wth, wtw, wT, wP, wQ;
+    int wps;  // patch side: 4 (3x3 filters, 16 positions) or 3 (2x2 filters, 9 positions)
 };
 
 // Timeline of a workgroup for eddlhip_conv2d_trace: words 0..3 = the device's constant 100 MHz clock at the marks (entry,
@@ -477,10 +478,11 @@ __global__ __launch_bounds__(256) void pack_filters_kernel(const float *__restri
 // 2x2 block with the factor A^T[a][i] * A^T[b][j], which is 0, 1 or -1.  A workgroup that walks through all 16 positions
 // therefore needs no M tensor: after the K run of a position it adds the accumulator into four running outputs, with
 // those signs, and clears it.  Positions are taken in the order 0..15, so the sums are reproducible.
-__device__ __forceinline__ void wino_fold(floatx16 (&y)[2][2], floatx16 &acc, int xi) {
-    const int i = xi >> 2, j = xi & 3;
-    const int ca[2] = {i < 3 ? 1 : 0, i == 0 ? 0 : (i == 1 ? 1 : -1)};
-    const int cb[2] = {j < 3 ? 1 : 0, j == 0 ? 0 : (j == 1 ? 1 : -1)};
+__device__ __forceinline__ void wino_fold(floatx16 (&y)[2][2], floatx16 &acc, int xi, int ps) {
+    // ps = 4: A^T = [1 1 1 0; 0 1 -1 -1]; ps = 3 (2x2 filters): A^T = [1 1 0; 0 1 -1]
+    const int i = xi / ps, j = xi - i * ps;
+    const int ca[2] = {i < ps - 1 ? 1 : 0, i == 0 ? 0 : (i == 1 ? 1 : -1)};
+    const int cb[2] = {j < ps - 1 ? 1 : 0, j == 0 ? 0 : (j == 1 ? 1 : -1)};
 #pragma unroll
     for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -815,7 +817,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         do_step(as_of(buf), bs_of(buf), as_of(buf ^ 1), bs_of(buf ^ 1), step, step + 1 < step_hi && !both);
         if constexpr (WINO) {
             if (--wino_left == 0) {  // this position's product is complete
-                wino_fold(wy, acc[0][0], wino_xi);
+                wino_fold(wy, acc[0][0], wino_xi, p.wps);
                 wino_xi++;
                 wino_left = p.wspx;
             }
@@ -1218,7 +1220,7 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvParams p) {
     }
 }
 
-// ---------------------------------------------------------------- Winograd F(2x2, 3x3)
+// ---------------------------------------------------------------- Winograd F(2x2, 3x3) and F(2x2, 2x2)
 // A 3x3 stride-1 convolution as 16 independent products of [Kf x C] by [C x tiles] matrices (Lavin & Gray's minimal
 // filtering form): every 4x4 input patch d (stride 2, so neighbouring patches overlap by two pixels) becomes
 // V = B^T d B, every filter g becomes U = G g G^T, M = U (.) V summed over the channels - position by position, which is
@@ -1227,57 +1229,95 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvParams p) {
 // the two transforms are bandwidth kernels.  Sums are fp32 in a fixed order, so results are reproducible, and they
 // differ from the direct form's by rounding only (a few 1e-7 of the largest output on this path's layers).
 //   B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1]   G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1]   A^T = [1 1 1 0; 0 1 -1 -1]
+// The same for a 2x2 filter (U-Net's convolutions behind its upsamplings): 3x3 patches, 9 products where the direct form
+// multiplies 16 times, every factor 1 or -1:
+//   B^T = [1 -1 0; 0 1 0; 0 1 -1]   G = [1 0; 1 1; 0 1]   A^T = [1 1 0; 0 1 -1]
+// PS below is the patch side (filter size + 1), PS * PS the number of products ("positions").
 struct WinoParams {
     const float *I, *I2;  // input as ConvParams describes it (second tensor of a folded Concat, folded upsampling)
     int Csplit, Cimg, uh, uw;
     int C, H, W, pt, pl;
     int th, tw;  // 2x2 output blocks per image, rows and columns
     int T, Tp;   // blocks in the launch; Tp = T rounded up to the widest tile: one "image" of the product launch
-    float *V;    // [16][C][Tp]
+    float *V;    // [PS * PS][C][Tp]
 };
 constexpr int WINO_CH = 4;  // channels (input transform) or filters (output transform) per thread
 
+template <int PS>
 __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restrict__ K, float *__restrict__ U, int Kf, int C, int Mp, int rows) {
+    constexpr int R = PS - 1;
     const int idx = blockIdx.x * 256 + threadIdx.x;  // (c, k), k fastest: row c of the packed matrices
     if (idx >= rows * Mp) return;
     const int c = idx / Mp, k = idx - c * Mp;
-    float g[9];
+    float g[R * R];
 #pragma unroll
-    for (int i = 0; i < 9; i++) g[i] = (c < C && k < Kf) ? K[((size_t)k * C + c) * 9 + i] : 0.0f;
-    float t[4][3];
-#pragma unroll
-    for (int j = 0; j < 3; j++) {
-        t[0][j] = g[j];
-        t[1][j] = __fmul_rn(0.5f, __fadd_rn(__fadd_rn(g[j], g[3 + j]), g[6 + j]));
-        t[2][j] = __fmul_rn(0.5f, __fadd_rn(__fsub_rn(g[j], g[3 + j]), g[6 + j]));
-        t[3][j] = g[6 + j];
-    }
+    for (int i = 0; i < R * R; i++) g[i] = (c < C && k < Kf) ? K[((size_t)k * C + c) * (R * R) + i] : 0.0f;
     const size_t plane = (size_t)rows * Mp;
+    if constexpr (PS == 4) {
+        float t[4][3];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        U[(size_t)(4 * i + 0) * plane + idx] = t[i][0];
-        U[(size_t)(4 * i + 1) * plane + idx] = __fmul_rn(0.5f, __fadd_rn(__fadd_rn(t[i][0], t[i][1]), t[i][2]));
-        U[(size_t)(4 * i + 2) * plane + idx] = __fmul_rn(0.5f, __fadd_rn(__fsub_rn(t[i][0], t[i][1]), t[i][2]));
-        U[(size_t)(4 * i + 3) * plane + idx] = t[i][2];
+        for (int j = 0; j < 3; j++) {
+            t[0][j] = g[j];
+            t[1][j] = __fmul_rn(0.5f, __fadd_rn(__fadd_rn(g[j], g[3 + j]), g[6 + j]));
+            t[2][j] = __fmul_rn(0.5f, __fadd_rn(__fsub_rn(g[j], g[3 + j]), g[6 + j]));
+            t[3][j] = g[6 + j];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            U[(size_t)(4 * i + 0) * plane + idx] = t[i][0];
+            U[(size_t)(4 * i + 1) * plane + idx] = __fmul_rn(0.5f, __fadd_rn(__fadd_rn(t[i][0], t[i][1]), t[i][2]));
+            U[(size_t)(4 * i + 2) * plane + idx] = __fmul_rn(0.5f, __fadd_rn(__fsub_rn(t[i][0], t[i][1]), t[i][2]));
+            U[(size_t)(4 * i + 3) * plane + idx] = t[i][2];
+        }
+    } else {
+        float t[3][2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            t[0][j] = g[j];
+            t[1][j] = __fadd_rn(g[j], g[2 + j]);
+            t[2][j] = g[2 + j];
+        }
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            U[(size_t)(3 * i + 0) * plane + idx] = t[i][0];
+            U[(size_t)(3 * i + 1) * plane + idx] = __fadd_rn(t[i][0], t[i][1]);
+            U[(size_t)(3 * i + 2) * plane + idx] = t[i][1];
+        }
     }
 }
 
-// V = B^T d B of one patch, written to the 16 planes (`plane` floats apart) at dst
-__device__ __forceinline__ void wino_input_store(const float (&d)[16], float *dst, size_t plane) {
-    float u[16];  // B^T d
+// V = B^T d B of one PS x PS patch, written to the PS * PS planes (`plane` floats apart) at dst
+template <int PS>
+__device__ __forceinline__ void wino_input_store(const float (&d)[PS * PS], float *dst, size_t plane) {
+    float u[PS * PS];  // B^T d
+    if constexpr (PS == 4) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        u[0 + j] = __fsub_rn(d[0 + j], d[8 + j]);
-        u[4 + j] = __fadd_rn(d[4 + j], d[8 + j]);
-        u[8 + j] = __fsub_rn(d[8 + j], d[4 + j]);
-        u[12 + j] = __fsub_rn(d[4 + j], d[12 + j]);
-    }
+        for (int j = 0; j < 4; j++) {
+            u[0 + j] = __fsub_rn(d[0 + j], d[8 + j]);
+            u[4 + j] = __fadd_rn(d[4 + j], d[8 + j]);
+            u[8 + j] = __fsub_rn(d[8 + j], d[4 + j]);
+            u[12 + j] = __fsub_rn(d[4 + j], d[12 + j]);
+        }
 #pragma unroll
-    for (int i = 0; i < 4; i++) {  // (B^T d) B
-        dst[(size_t)(4 * i + 0) * plane] = __fsub_rn(u[4 * i + 0], u[4 * i + 2]);
-        dst[(size_t)(4 * i + 1) * plane] = __fadd_rn(u[4 * i + 1], u[4 * i + 2]);
-        dst[(size_t)(4 * i + 2) * plane] = __fsub_rn(u[4 * i + 2], u[4 * i + 1]);
-        dst[(size_t)(4 * i + 3) * plane] = __fsub_rn(u[4 * i + 1], u[4 * i + 3]);
+        for (int i = 0; i < 4; i++) {  // (B^T d) B
+            dst[(size_t)(4 * i + 0) * plane] = __fsub_rn(u[4 * i + 0], u[4 * i + 2]);
+            dst[(size_t)(4 * i + 1) * plane] = __fadd_rn(u[4 * i + 1], u[4 * i + 2]);
+            dst[(size_t)(4 * i + 2) * plane] = __fsub_rn(u[4 * i + 2], u[4 * i + 1]);
+            dst[(size_t)(4 * i + 3) * plane] = __fsub_rn(u[4 * i + 1], u[4 * i + 3]);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            u[0 + j] = __fsub_rn(d[0 + j], d[3 + j]);
+            u[3 + j] = d[3 + j];
+            u[6 + j] = __fsub_rn(d[3 + j], d[6 + j]);
+        }
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            dst[(size_t)(3 * i + 0) * plane] = __fsub_rn(u[3 * i + 0], u[3 * i + 1]);
+            dst[(size_t)(3 * i + 1) * plane] = u[3 * i + 1];
+            dst[(size_t)(3 * i + 2) * plane] = __fsub_rn(u[3 * i + 1], u[3 * i + 2]);
+        }
     }
 }
 
@@ -1287,14 +1327,14 @@ __device__ __forceinline__ void wino_input_store(const float (&d)[16], float *ds
 // first being column -pad_left), where that pixel lies in a channel plane, or that it does not exist.  Then per channel:
 // the slots are filled with coalesced loads - every pixel once, where the kernel below reads each four times through
 // the cache with half of every line unused -, a thread reads its 4x4 patch from LDS, transforms and stores as below.
-template <int KMAX>  // a thread fills at most KMAX slots: slots <= 256 * KMAX
+template <int KMAX, int PS>  // a thread fills at most KMAX slots: slots <= 256 * KMAX
 __global__ __launch_bounds__(256) void wino_input_lds_kernel(const WinoParams w, int slots, int chans) {
     extern __shared__ int wino_lds[];
     int *soff = wino_lds;
     float *sval = reinterpret_cast<float *>(wino_lds + slots);
     const int tid = threadIdx.x;
     const int t0 = blockIdx.x * 256, t1 = min(t0 + 256, w.T), t = t0 + tid;
-    const int per_img = w.th * w.tw, LW = 2 * w.tw + 2;
+    const int per_img = w.th * w.tw, LW = 2 * w.tw + PS - 2;
     const unsigned Hu = (unsigned)(w.H * w.uh), Wu = (unsigned)(w.W * w.uw);
     const int n_first = t0 / per_img;
     const int img_elems = w.Cimg * w.H * w.W;
@@ -1303,7 +1343,7 @@ __global__ __launch_bounds__(256) void wino_input_lds_kernel(const WinoParams w,
     for (int n = n_first; n * per_img < t1; n++) {  // the images this workgroup's blocks lie in (uniform)
         const int a = max(t0, n * per_img) - n * per_img, b = min(t1, (n + 1) * per_img) - n * per_img;
         const int ty_a = a / w.tw, ty_b = (b - 1) / w.tw;
-        const int cells = (2 * (ty_b - ty_a) + 4) * LW;
+        const int cells = (2 * (ty_b - ty_a) + PS) * LW;
         const int y_first = 2 * ty_a - w.pt, img_off = (n - n_first) * img_elems;
         for (int i = tid; i < cells; i += 256) {
             const int r = i / LW, xl = i - r * LW;
@@ -1341,17 +1381,24 @@ __global__ __launch_bounds__(256) void wino_input_lds_kernel(const WinoParams w,
         __syncthreads();
         if (c + 1 < c1) fetch(c + 1);
         if (t < t1) {
-            float d[16];
+            float d[PS * PS];
+            if constexpr (PS == 4) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {  // (rows and the patch's first column are at even slots)
-                const float2 lo = *reinterpret_cast<const float2 *>(sval + my_base + i * LW);
-                const float2 hi = *reinterpret_cast<const float2 *>(sval + my_base + i * LW + 2);
-                d[4 * i + 0] = lo.x;
-                d[4 * i + 1] = lo.y;
-                d[4 * i + 2] = hi.x;
-                d[4 * i + 3] = hi.y;
+                for (int i = 0; i < 4; i++) {  // (rows and the patch's first column are at even slots)
+                    const float2 lo = *reinterpret_cast<const float2 *>(sval + my_base + i * LW);
+                    const float2 hi = *reinterpret_cast<const float2 *>(sval + my_base + i * LW + 2);
+                    d[4 * i + 0] = lo.x;
+                    d[4 * i + 1] = lo.y;
+                    d[4 * i + 2] = hi.x;
+                    d[4 * i + 3] = hi.y;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < PS; i++)
+#pragma unroll
+                    for (int j = 0; j < PS; j++) d[PS * i + j] = sval[my_base + i * LW + j];
             }
-            wino_input_store(d, w.V + (size_t)c * w.Tp + t, plane);
+            wino_input_store<PS>(d, w.V + (size_t)c * w.Tp + t, plane);
         }
         __syncthreads();
     }
@@ -1360,6 +1407,7 @@ __global__ __launch_bounds__(256) void wino_input_lds_kernel(const WinoParams w,
 // One thread: one 2x2 output block (its 4x4 input patch) for WINO_CH channels; lanes hold consecutive blocks, so the 16
 // stores of a channel are 16 coalesced rows.  The patch offsets and which of its pixels exist are worked out once.
 // (The general form: taken where the staged kernel's tables would not fit.)
+template <int PS>
 __global__ __launch_bounds__(256) void wino_input_kernel(const WinoParams w) {
     const int t = blockIdx.x * 256 + threadIdx.x;
     if (t >= w.T) return;
@@ -1367,18 +1415,18 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const WinoParams w) {
     const int n = t / per_img, r = t - n * per_img, ty = r / w.tw, tx = r - ty * w.tw;
     const int y0 = 2 * ty - w.pt, x0 = 2 * tx - w.pl;
     const unsigned Hu = (unsigned)(w.H * w.uh), Wu = (unsigned)(w.W * w.uw);
-    int off[16];
+    int off[PS * PS];
     unsigned mask = 0;
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < PS; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < PS; j++) {
             const unsigned y = (unsigned)(y0 + i), x = (unsigned)(x0 + j);
             const bool ok = y < Hu && x < Wu;
             int o = 0;
             if (ok) o = (w.uh == 1 && w.uw == 1) ? (int)(y * (unsigned)w.W + x) : (int)((y / (unsigned)w.uh) * (unsigned)w.W + x / (unsigned)w.uw);
-            off[4 * i + j] = o;
-            mask |= (ok ? 1u : 0u) << (4 * i + j);
+            off[PS * i + j] = o;
+            mask |= (ok ? 1u : 0u) << (PS * i + j);
         }
     const size_t hw = (size_t)w.H * w.W, plane = (size_t)w.C * w.Tp;
     const int c0 = blockIdx.y * WINO_CH;
@@ -1387,15 +1435,16 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const WinoParams w) {
         const int c = c0 + cc;
         if (c >= w.C) break;
         const float *src = c < w.Csplit ? w.I + ((size_t)n * w.Cimg + c) * hw : w.I2 + ((size_t)n * w.Cimg + (c - w.Csplit)) * hw;
-        float d[16];
+        float d[PS * PS];
 #pragma unroll
-        for (int e = 0; e < 16; e++) d[e] = ((mask >> e) & 1u) ? src[off[e]] : 0.0f;
-        wino_input_store(d, w.V + (size_t)c * w.Tp + t, plane);
+        for (int e = 0; e < PS * PS; e++) d[e] = ((mask >> e) & 1u) ? src[off[e]] : 0.0f;
+        wino_input_store<PS>(d, w.V + (size_t)c * w.Tp + t, plane);
     }
 }
 
 // One thread: one 2x2 output block for WINO_CH filters: A^T M A, then the convolution's epilogue (the arithmetic of
 // apply_epilogue, value by value) and the stores - both values of a row at once where the row pair is aligned.
+template <int PS>
 __global__ __launch_bounds__(256) void wino_output_kernel(const ConvParams p, const float *__restrict__ M, int th, int tw, int T, int Tp) {
     const int t = blockIdx.x * 256 + threadIdx.x;
     if (t >= T) return;
@@ -1409,22 +1458,33 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const ConvParams p, co
         const int k = k0 + cc;
         if (k >= p.Kf) break;
         const float *src = M + (size_t)k * Tp + t;
-        float m[16];
+        float m[PS * PS];
 #pragma unroll
-        for (int e = 0; e < 16; e++) m[e] = src[(size_t)e * plane];
-        float s[2][4];
+        for (int e = 0; e < PS * PS; e++) m[e] = src[(size_t)e * plane];
+        float s[2][PS];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            s[0][j] = __fadd_rn(__fadd_rn(m[0 + j], m[4 + j]), m[8 + j]);
-            s[1][j] = __fsub_rn(__fsub_rn(m[4 + j], m[8 + j]), m[12 + j]);
+        for (int j = 0; j < PS; j++) {
+            if constexpr (PS == 4) {
+                s[0][j] = __fadd_rn(__fadd_rn(m[0 + j], m[4 + j]), m[8 + j]);
+                s[1][j] = __fsub_rn(__fsub_rn(m[4 + j], m[8 + j]), m[12 + j]);
+            } else {
+                s[0][j] = __fadd_rn(m[0 + j], m[3 + j]);
+                s[1][j] = __fsub_rn(m[3 + j], m[6 + j]);
+            }
         }
         const ChannelEpilogue e = load_channel(p, k);
 #pragma unroll
         for (int a = 0; a < 2; a++) {
             const int oy = 2 * ty + a, ox = 2 * tx;
             if (oy >= p.P) break;
-            const float v0 = __fadd_rn(__fadd_rn(s[a][0], s[a][1]), s[a][2]);
-            const float v1 = __fsub_rn(__fsub_rn(s[a][1], s[a][2]), s[a][3]);
+            float v0, v1;
+            if constexpr (PS == 4) {
+                v0 = __fadd_rn(__fadd_rn(s[a][0], s[a][1]), s[a][2]);
+                v1 = __fsub_rn(__fsub_rn(s[a][1], s[a][2]), s[a][3]);
+            } else {
+                v0 = __fadd_rn(s[a][0], s[a][1]);
+                v1 = __fsub_rn(s[a][1], s[a][2]);
+            }
             const size_t oidx = ((size_t)n * p.Kf + k) * p.PQ + (size_t)oy * p.Q + ox;
             if (pair) {  // Q even: column ox + 1 exists
                 float r0 = 0.0f, r1 = 0.0f;
@@ -1636,7 +1696,7 @@ struct CachedFilters {
     const float *K;
     int Kf, C, R, S, rows, Mp;
     float *Wp;
-    float *Wwino;  // 3x3 filters: the 16 transformed matrices of the Winograd form [16][wino_rows][Mp], made on first use
+    float *Wwino;  // 3x3 (2x2) filters: the 16 (9) transformed matrices of the Winograd form [16][wino_rows][Mp], made on first use
     int wino_rows;
     bool stale;  // K was written through this library since the last repack
 };
@@ -1658,8 +1718,9 @@ int repack(int dev, CachedFilters &e) {
                        e.C * e.R * e.S, e.Mp, e.rows);
     EH_CHECK_LAUNCH();
     if (e.Wwino != nullptr) {
-        hipLaunchKernelGGL(wino_filter_kernel, dim3((unsigned)(((size_t)e.wino_rows * e.Mp + 255) / 256)), dim3(256), 0, state(dev).stream, e.K,
-                           e.Wwino, e.Kf, e.C, e.Mp, e.wino_rows);
+        const dim3 grid((unsigned)(((size_t)e.wino_rows * e.Mp + 255) / 256));
+        if (e.R == 3) hipLaunchKernelGGL(wino_filter_kernel<4>, grid, dim3(256), 0, state(dev).stream, e.K, e.Wwino, e.Kf, e.C, e.Mp, e.wino_rows);
+        else hipLaunchKernelGGL(wino_filter_kernel<3>, grid, dim3(256), 0, state(dev).stream, e.K, e.Wwino, e.Kf, e.C, e.Mp, e.wino_rows);
         EH_CHECK_LAUNCH();
     }
     e.stale = false;
@@ -1899,14 +1960,14 @@ struct GemmBatch {
 // at most 16 slices each, 128 x 128 floats per tile.  The Winograd driver keeps its own buffers behind this much.
 constexpr size_t WINO_INNER_RESERVE = (size_t)16 * 255 * 128 * 128 * sizeof(float);
 
-int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C, int H,
-                    int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
+int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
+                    int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
                     const float *bn_var, float bn_eps, const float *residual, int relu);
 
 // Whether the Winograd form can run this convolution: 3x3, stride 1, and the product launch within the limits of
 // conv2d_fwd_impl (one "image" of transformed input or output below 1 GiB, fewer than 2^31 blocks).
 bool winograd_applies(int N, int C, int Kf, int R, int S, int sr, int sc, int P, int Q) {
-    if (R != 3 || S != 3 || sr != 1 || sc != 1) return false;
+    if (R != S || (R != 3 && R != 2) || sr != 1 || sc != 1) return false;
     const long long T = (long long)N * ((P + 1) / 2) * ((Q + 1) / 2), Tp = (T + 127) / 128 * 128;
     return Tp <= 0x3fffff80LL && (long long)C * Tp <= (1LL << 28) && (long long)Kf * Tp <= (1LL << 28);
 }
@@ -1915,7 +1976,8 @@ bool winograd_applies(int N, int C, int Kf, int R, int S, int sr, int sc, int P,
 bool winograd_fold_applies(int N, int C, int Kf, int R, int S, int sr, int sc, int P, int Q) {
     if (!winograd_applies(N, C, Kf, R, S, sr, sc, P, Q) || C % 16 != 0) return false;
     const long long T = (long long)N * ((P + 1) / 2) * ((Q + 1) / 2), Tp = (T + 127) / 128 * 128;
-    return 16LL * C * Tp * 4 < (1LL << 31) && 16LL * C * ((Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN) * 4 < (1LL << 31);
+    const long long np = (R + 1) * (R + 1);
+    return np * C * Tp * 4 < (1LL << 31) && np * C * ((Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN) * 4 < (1LL << 31);
 }
 
 int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
@@ -2047,7 +2109,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     const bool wino_ok = !gemm && !no_alloc && g_algo == 0 && winograd_applies(N, C, Kf, R, S, sr, sc, P, Q);
     const bool fold_ok = wino_ok && winograd_fold_applies(N, C, Kf, R, S, sr, sc, P, Q);
     if ((wino_ok && (g_force_tile == 4 || (g_wino && g_force_tile < 0 && !g_tuning))) || (fold_ok && g_force_tile == 5))
-        return conv2d_winograd(g_force_tile == 5, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b,
+        return conv2d_winograd(g_force_tile == 5, R, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b,
                                bn_mean, bn_var, bn_eps, residual, relu);
     if (g_autotune && g_force_tile < 0 && g_algo == 0 && g_split != 0) {
         const int key[10] = {N, C, Kf, R, S, sr, sc, P, Q, direct};
@@ -2136,8 +2198,8 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
             found = &g_tuned[dev].back();
         }
         if (found != nullptr && ((found->tile == 4 && wino_ok) || (found->tile == 5 && fold_ok)))
-            return conv2d_winograd(found->tile == 5, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b,
-                                   bn_mean, bn_var, bn_eps, residual, relu);
+            return conv2d_winograd(found->tile == 5, R, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g,
+                                   bn_b, bn_mean, bn_var, bn_eps, residual, relu);
         if (found != nullptr && found->tile >= 0 && found->tile < 4)
             plan = forced_plan(family, found->tile, found->slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
     }
@@ -2239,14 +2301,15 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
 // filter tensor), input transform, ONE product launch through conv2d_fwd_impl (16 images of C channels and Tp pixels, a
 // planned or searched 1x1 launch like any other), output transform with the convolution's epilogue.
 // Workspace: [what the product launch may take][transformed filters unless kept][V][M].
-int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C, int H,
-                    int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
+int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
+                    int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
                     const float *bn_var, float bn_eps, const float *residual, int relu) {
     hipStream_t st = state(dev).stream;
+    const int ps = fs + 1, np = ps * ps;  // patch side and positions: 4 and 16 for 3x3 filters, 3 and 9 for 2x2
     const int th = (P + 1) / 2, tw = (Q + 1) / 2;
     const int T = N * th * tw, Tp = (T + 127) / 128 * 128;
     const int rows = (C + 15) / 16 * 16, Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
-    const size_t u_floats = (size_t)16 * rows * Mp, v_floats = (size_t)16 * C * Tp, m_floats = (size_t)16 * Kf * Tp;
+    const size_t u_floats = (size_t)np * rows * Mp, v_floats = (size_t)np * C * Tp, m_floats = (size_t)np * Kf * Tp;
     EH_REQUIRE((size_t)rows * Mp * sizeof(float) < ((size_t)1 << 31), "conv2d: the transformed filter matrix (%d x %d) exceeds 2 GiB", rows, Mp);
 
     // ---- transformed filters: the registered copy (made here on first use, refreshed when the filters were written), or a
@@ -2255,7 +2318,7 @@ int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh,
     {
         std::lock_guard<std::mutex> lock(g_cache_mutex);
         for (CachedFilters &e : g_cache[dev]) {
-            if (e.K == K && e.Kf == Kf && e.C == C && e.R == 3 && e.S == 3) {
+            if (e.K == K && e.Kf == Kf && e.C == C && e.R == fs && e.S == fs) {
                 if (e.Wwino == nullptr && !state(dev).capturing) {
                     if (hipMalloc((void **)&e.Wwino, u_floats * sizeof(float)) != hipSuccess) {
                         e.Wwino = nullptr;
@@ -2281,7 +2344,9 @@ int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh,
     char *base = (char *)ws + WINO_INNER_RESERVE;
     float *Uw = (float *)base, *V = (float *)(base + u_bytes), *M = (float *)(base + u_bytes + v_bytes);
     if (U == nullptr) {
-        hipLaunchKernelGGL(wino_filter_kernel, dim3((unsigned)(((size_t)rows * Mp + 255) / 256)), dim3(256), 0, st, K, Uw, Kf, C, Mp, rows);
+        const dim3 grid((unsigned)(((size_t)rows * Mp + 255) / 256));
+        if (ps == 4) hipLaunchKernelGGL(wino_filter_kernel<4>, grid, dim3(256), 0, st, K, Uw, Kf, C, Mp, rows);
+        else hipLaunchKernelGGL(wino_filter_kernel<3>, grid, dim3(256), 0, st, K, Uw, Kf, C, Mp, rows);
         EH_CHECK_LAUNCH();
         U = Uw;
     }
@@ -2300,15 +2365,20 @@ int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh,
         const long long per_img = (long long)th * tw;
         const long long segs = std::min<long long>(N, 256 / per_img + 2);
         const long long block_rows = 256 / tw + 2 * segs;
-        const long long slots = ((2 * block_rows + 2 * segs) * (2 * tw + 2) + 1) & ~1LL;
+        const long long slots = ((2 * block_rows + (ps - 2) * segs) * (2 * tw + ps - 2) + 1) & ~1LL;
         const long long img_elems = (long long)w.Cimg * H * W;
         constexpr int chans = 8;
         if (slots <= 256 * 16 && segs * img_elems < 0x7fffffffLL) {
             const dim3 grid((unsigned)((T + 255) / 256), (unsigned)((C + chans - 1) / chans));
-            if (slots <= 256 * 8) hipLaunchKernelGGL(wino_input_lds_kernel<8>, grid, dim3(256), (size_t)slots * 8, st, w, (int)slots, chans);
-            else hipLaunchKernelGGL(wino_input_lds_kernel<16>, grid, dim3(256), (size_t)slots * 8, st, w, (int)slots, chans);
+            const size_t lds = (size_t)slots * 8;
+            if (ps == 4 && slots <= 256 * 8) hipLaunchKernelGGL((wino_input_lds_kernel<8, 4>), grid, dim3(256), lds, st, w, (int)slots, chans);
+            else if (ps == 4) hipLaunchKernelGGL((wino_input_lds_kernel<16, 4>), grid, dim3(256), lds, st, w, (int)slots, chans);
+            else if (slots <= 256 * 8) hipLaunchKernelGGL((wino_input_lds_kernel<8, 3>), grid, dim3(256), lds, st, w, (int)slots, chans);
+            else hipLaunchKernelGGL((wino_input_lds_kernel<16, 3>), grid, dim3(256), lds, st, w, (int)slots, chans);
         } else {
-            hipLaunchKernelGGL(wino_input_kernel, dim3((unsigned)((T + 255) / 256), (unsigned)((C + WINO_CH - 1) / WINO_CH)), dim3(256), 0, st, w);
+            const dim3 grid((unsigned)((T + 255) / 256), (unsigned)((C + WINO_CH - 1) / WINO_CH));
+            if (ps == 4) hipLaunchKernelGGL(wino_input_kernel<4>, grid, dim3(256), 0, st, w);
+            else hipLaunchKernelGGL(wino_input_kernel<3>, grid, dim3(256), 0, st, w);
         }
     }
     EH_CHECK_LAUNCH();
@@ -2319,24 +2389,24 @@ int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh,
         // into the four outputs of a block and finishes with the convolution's epilogue (64x64 tiles, whole tiles only)
         ConvParams q;
         memset(&q, 0, sizeof(q));
-        q.I = V; q.I2 = V; q.Csplit = 16 * C; q.Cimg = 16 * C; q.uh = 1; q.uw = 1;
+        q.I = V; q.I2 = V; q.Csplit = np * C; q.Cimg = np * C; q.uh = 1; q.uw = 1;
         q.Wp = U; q.w_img_stride = 0; q.K = K; q.O = O;
         q.bias = bias; q.bn_g = bn_g; q.bn_b = bn_b; q.bn_mean = bn_mean; q.bn_var = bn_var; q.residual = residual;
         q.bn_eps = bn_eps; q.relu = relu;
-        q.N = 1; q.C = 16 * C; q.H = 1; q.W = Tp; q.Kf = Kf; q.R = 1; q.S = 1; q.sr = 1; q.sc = 1; q.P = 1; q.Q = Tp;
-        q.CRS = 16 * C; q.Mp = Mp; q.nsteps = C; q.PQ = Tp; q.npix = Tp;
+        q.N = 1; q.C = np * C; q.H = 1; q.W = Tp; q.Kf = Kf; q.R = 1; q.S = 1; q.sr = 1; q.sc = 1; q.P = 1; q.Q = Tp;
+        q.CRS = np * C; q.Mp = Mp; q.nsteps = np * C / 16; q.PQ = Tp; q.npix = Tp;
         q.gm = (Kf + 63) / 64; q.gn = Tp / 64;
-        q.in_bytes = (unsigned)((size_t)16 * C * Tp * sizeof(float));
-        q.wp_bytes = (unsigned)((size_t)16 * rows * Mp * sizeof(float));
+        q.in_bytes = (unsigned)((size_t)np * C * Tp * sizeof(float));
+        q.wp_bytes = (unsigned)((size_t)np * rows * Mp * sizeof(float));
         q.main_tiles = q.gm * q.gn; q.nslices = 1; q.slice_steps = q.nsteps;
-        q.wspx = C / 16; q.wth = th; q.wtw = tw; q.wT = T; q.wP = P; q.wQ = Q;
+        q.wspx = C / 16; q.wth = th; q.wtw = tw; q.wT = T; q.wP = P; q.wQ = Q; q.wps = ps;
         EH_REQUIRE(rows == C && (long long)q.gm * q.gn <= 0x3fffffffLL, "conv2d: internal error, folded Winograd launch");
         q.trace = (g_trace != nullptr && q.main_tiles <= g_trace_wgs) ? g_trace : nullptr;
         // K-steps of 32 channels where the runs divide into them: a workgroup's K loop is long here (16 C channels), few
         // workgroups share a CU (64 output registers per lane), and a step's matrix work then covers a trip to memory
         const bool wide = C % 32 == 0;
         if (wide) {
-            q.nsteps = C / 2;
+            q.nsteps = np * C / 32;
             q.slice_steps = q.nsteps;
             q.wspx = C / 32;
         }
@@ -2355,7 +2425,7 @@ int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh,
         const int ft = g_force_tile, fs = g_force_slices;
         g_force_tile = -1;
         g_force_slices = -1;
-        const int rc = conv2d_fwd_impl(false, dev, V, nullptr, 1, 1, K, nullptr, M, 16, C, 1, Tp, Kf, 1, 1, 1, 1, 0, 0, 1, Tp, nullptr, nullptr, nullptr,
+        const int rc = conv2d_fwd_impl(false, dev, V, nullptr, 1, 1, K, nullptr, M, np, C, 1, Tp, Kf, 1, 1, 1, 1, 0, 0, 1, Tp, nullptr, nullptr, nullptr,
                                        nullptr, 0.0f, nullptr, 0, &gb);
         g_force_tile = ft;
         g_force_slices = fs;
@@ -2369,8 +2439,11 @@ int conv2d_winograd(bool fold, int dev, const float *I, const float *I2, int uh,
     p.bias = bias; p.bn_g = bn_g; p.bn_b = bn_b; p.bn_mean = bn_mean; p.bn_var = bn_var; p.residual = residual;
     p.bn_eps = bn_eps; p.relu = relu;
     p.N = N; p.Kf = Kf; p.P = P; p.Q = Q; p.PQ = P * Q;
-    hipLaunchKernelGGL(wino_output_kernel, dim3((unsigned)((T + 255) / 256), (unsigned)((Kf + WINO_CH - 1) / WINO_CH)), dim3(256), 0, st, p,
-                       (const float *)M, th, tw, T, Tp);
+    {
+        const dim3 grid((unsigned)((T + 255) / 256), (unsigned)((Kf + WINO_CH - 1) / WINO_CH));
+        if (ps == 4) hipLaunchKernelGGL(wino_output_kernel<4>, grid, dim3(256), 0, st, p, (const float *)M, th, tw, T, Tp);
+        else hipLaunchKernelGGL(wino_output_kernel<3>, grid, dim3(256), 0, st, p, (const float *)M, th, tw, T, Tp);
+    }
     EH_CHECK_LAUNCH();
     char inner[sizeof(g_last_kernel)];
     snprintf(inner, sizeof(inner), "%s", g_last_kernel);

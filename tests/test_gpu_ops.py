@@ -410,6 +410,39 @@ def test_conv2d_winograd_form_against_oracle(hip, oracle, case, form):
     assert_conv_close(ref, O.numpy(), "winograd %s" % (case,))
 
 
+@pytest.mark.parametrize("form", [4, 5], ids=["three-kernels", "folded"])
+def test_conv2d_winograd_form_of_2x2_filters_against_oracle(hip, oracle, form):
+    """F(2x2, 2x2): the convolutions behind U-Net's upsamplings (a folded UpSampling2D and a folded Pad of one row below and
+    one column right), plain 2x2 'valid' convolutions, odd sizes, the fused epilogue - against the oracle's direct form."""
+    rng = np.random.default_rng(79)
+    cases = [(2, 32, 8, 8, 48, (0, 0), None, None), (1, 16, 9, 11, 24, (0, 0), None, None), (2, 32, 6, 6, 16, (0, 0), (12, 12), (2, 2)),
+             (2, 64, 5, 7, 40, (1, 0), None, None), (1, 48, 7, 5, 32, (0, 0), (14, 10), (2, 2))]
+    for (N, C, H, W, Kf, (pt, pl), out, up) in cases:
+        a = rng.standard_normal((N, C, H, W), dtype=np.float32)
+        w = (rng.standard_normal((Kf, C, 2, 2)) * np.sqrt(2.0 / (C * 4))).astype(np.float32)
+        logical = np.repeat(np.repeat(a, up[0], axis=2), up[1], axis=3) if up else a
+        Hu, Wu = logical.shape[2:]
+        P, Q = out or (Hu + 2 * pt - 1, Wu + 2 * pl - 1)
+        padded = np.zeros((N, C, P + 1, Q + 1), np.float32)
+        ys, xs = min(Hu, P + 1 - pt), min(Wu, Q + 1 - pl)
+        padded[:, :, pt:pt + ys, pl:pl + xs] = logical[:, :, :ys, :xs]
+        bias = rng.standard_normal(Kf, dtype=np.float32)
+        bn = _bn_params(rng, Kf)
+        ref = oracle.conv2d(padded, w, bias, (1, 1), 0, 0, P, Q)
+        ref, _, _ = oracle.batchnorm_inference(ref, bn[2], bn[3], bn[0], bn[1], bn[4])
+        ref = oracle.relu(ref)
+        O = hip.full((N, Kf, P, Q), 3.0)
+        dbn = (hip.array(bn[0]), hip.array(bn[1]), hip.array(bn[2]), hip.array(bn[3]), bn[4])
+        hip.force_conv_plan(form, 1)
+        try:
+            hip.conv2D(hip.array(a), hip.array(w), hip.array(bias), O, 1, 1, pt, pl, bn=dbn, relu=True, upsample=up)
+            name = hip.last_conv_kernel()
+        finally:
+            hip.force_conv_plan(-1, 1)
+        assert name.startswith("winograd[") and ("true,true>" in name) == (form == 5), name
+        assert_conv_close(ref, O.numpy(), "winograd 2x2 %s" % ((N, C, H, W, Kf, pt, pl, out, up),))
+
+
 def test_conv2d_winograd_form_only_where_it_applies_and_with_kept_filters(hip, oracle):
     """Strides other than one and filters other than 3x3 keep the direct form under force_conv_plan(4, .) and set_conv_algo
     ("winograd"); registered filters keep their transformed copy, which follows writes to the filter tensor; the call that
