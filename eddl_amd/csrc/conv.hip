@@ -2368,13 +2368,16 @@ int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2,
         const long long slots = ((2 * block_rows + (ps - 2) * segs) * (2 * tw + ps - 2) + 1) & ~1LL;
         const long long img_elems = (long long)w.Cimg * H * W;
         constexpr int chans = 8;
-        if (slots <= 256 * 16 && segs * img_elems < 0x7fffffffLL) {
+        if (slots <= 256 * 30 && segs * img_elems < 0x7fffffffLL) {  // (offsets and values of 7680 slots: 60 KB of LDS)
             const dim3 grid((unsigned)((T + 255) / 256), (unsigned)((C + chans - 1) / chans));
             const size_t lds = (size_t)slots * 8;
-            if (ps == 4 && slots <= 256 * 8) hipLaunchKernelGGL((wino_input_lds_kernel<8, 4>), grid, dim3(256), lds, st, w, (int)slots, chans);
-            else if (ps == 4) hipLaunchKernelGGL((wino_input_lds_kernel<16, 4>), grid, dim3(256), lds, st, w, (int)slots, chans);
-            else if (slots <= 256 * 8) hipLaunchKernelGGL((wino_input_lds_kernel<8, 3>), grid, dim3(256), lds, st, w, (int)slots, chans);
-            else hipLaunchKernelGGL((wino_input_lds_kernel<16, 3>), grid, dim3(256), lds, st, w, (int)slots, chans);
+            const int kmax = slots <= 256 * 8 ? 8 : (slots <= 256 * 16 ? 16 : 30);
+            if (ps == 4 && kmax == 8) hipLaunchKernelGGL((wino_input_lds_kernel<8, 4>), grid, dim3(256), lds, st, w, (int)slots, chans);
+            else if (ps == 4 && kmax == 16) hipLaunchKernelGGL((wino_input_lds_kernel<16, 4>), grid, dim3(256), lds, st, w, (int)slots, chans);
+            else if (ps == 4) hipLaunchKernelGGL((wino_input_lds_kernel<30, 4>), grid, dim3(256), lds, st, w, (int)slots, chans);
+            else if (kmax == 8) hipLaunchKernelGGL((wino_input_lds_kernel<8, 3>), grid, dim3(256), lds, st, w, (int)slots, chans);
+            else if (kmax == 16) hipLaunchKernelGGL((wino_input_lds_kernel<16, 3>), grid, dim3(256), lds, st, w, (int)slots, chans);
+            else hipLaunchKernelGGL((wino_input_lds_kernel<30, 3>), grid, dim3(256), lds, st, w, (int)slots, chans);
         } else {
             const dim3 grid((unsigned)((T + 255) / 256), (unsigned)((C + WINO_CH - 1) / WINO_CH));
             if (ps == 4) hipLaunchKernelGGL(wino_input_kernel<4>, grid, dim3(256), 0, st, w);
