@@ -37,7 +37,7 @@ def assert_conv_bar(ref, got, scale, what):
     assert np.all(err <= tol), "%s: worst error %g (allowed %g)" % (what, err.max(), tol[np.argmax(err - tol)])
 
 
-def check_fullsize(hip, ora, model, x, seed):
+def check_fullsize(hip, ora, model, x, seed, only_convs=False):
     from eddl_amd import models
     rng = np.random.default_rng(seed + 1000)
     models.init_he_normal(model, seed)
@@ -45,7 +45,7 @@ def check_fullsize(hip, ora, model, x, seed):
     out_unfused = [o.numpy() for o in model.forward([x])]
     checked = {"conv2d": 0, "dense": 0, "exact": 0}
     for l in model.layers:
-        if l.kind == "input":
+        if l.kind == "input" or (only_convs and l.kind != "conv2d"):
             continue
         ins = [model.output_of(p).numpy() for p in l.parents]
         got = model.output_of(l).numpy()
@@ -125,6 +125,31 @@ def test_unet_4x1x512x512(hip, oracle):
     x = np.random.default_rng(5).uniform(0, 1, (4, 1, 512, 512)).astype(np.float32)
     got = check_fullsize(hip, oracle, m, x, 5)
     assert got["conv2d"] == 23
+
+
+@pytest.mark.parametrize("workload,form", [("vgg16", "three kernels"), ("vgg16", "folded"), ("resnet50", "three kernels"), ("unet", "three kernels")])
+def test_winograd_forms_at_full_size(hip, oracle, workload, form):
+    """The same sampled check of every convolution with the Winograd forms forced wherever they apply (3x3 and 2x2
+    filters at stride 1; the folded form also needs channels in sixteens): the forms the plan search may pick at the
+    benchmark sizes meet the convolution bar there, on the device's own layer inputs, and fuse bit for bit."""
+    from eddl_amd import models
+    m, x, seed, convs = {
+        "vgg16": lambda: (models.vgg16(batch=32), np.random.default_rng(3).uniform(0, 1, (32, 3, 224, 224)).astype(np.float32), 3, 13),
+        "resnet50": lambda: (models.resnet50(batch=64), np.random.default_rng(4).standard_normal((64, 3, 224, 224), dtype=np.float32), 4, 53),
+        "unet": lambda: (models.unet(batch=4), np.random.default_rng(5).uniform(0, 1, (4, 1, 512, 512)).astype(np.float32), 5, 23),
+    }[workload]()
+    try:
+        if form == "folded":
+            hip.force_conv_plan(5, 1)
+        else:
+            hip.set_conv_algo("winograd")
+        got = check_fullsize(hip, oracle, m, x, seed, only_convs=True)
+        assert got["conv2d"] == convs
+        if workload == "vgg16":  # its last convolution is 3x3 at stride 1 over 512 channels: both forms apply
+            assert hip.last_conv_kernel().startswith("winograd["), hip.last_conv_kernel()
+    finally:
+        hip.force_conv_plan(-1, 1)
+        hip.set_conv_algo("auto")
 
 
 def test_conv_scaling_by_powers_of_two_is_exact_at_full_size(hip):
