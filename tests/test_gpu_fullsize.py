@@ -127,7 +127,7 @@ def test_unet_4x1x512x512(hip, oracle):
     assert got["conv2d"] == 23
 
 
-@pytest.mark.parametrize("workload,form", [("vgg16", "three kernels"), ("vgg16", "folded"), ("resnet50", "three kernels"), ("unet", "three kernels")])
+@pytest.mark.parametrize("workload,form", [("vgg16", "three kernels"), ("vgg16", "folded"), ("resnet50", "three kernels"), ("resnet50", "folded"), ("unet", "three kernels"), ("unet", "folded")])
 def test_winograd_forms_at_full_size(hip, oracle, workload, form):
     """The same sampled check of every convolution with the Winograd forms forced wherever they apply (3x3 and 2x2
     filters at stride 1; the folded form also needs channels in sixteens): the forms the plan search may pick at the
