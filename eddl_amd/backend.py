@@ -245,7 +245,7 @@ class Backend:
         return t
 
     def set_conv_algo(self, algo):
-        self._check(self.lib.eddlhip_conv2d_set_algo({"auto": 0, "mfma": 1, "direct": 2, "mfma_staged": 3, "mfma_lds": 4, "ksplit_off": 5, "ksplit_on": 6, "winograd": 7, "winograd_off": 8}.get(algo, algo)))
+        self._check(self.lib.eddlhip_conv2d_set_algo({"auto": 0, "mfma": 1, "direct": 2, "mfma_staged": 3, "mfma_lds": 4, "ksplit_off": 5, "ksplit_on": 6, "winograd": 7, "winograd_off": 8, "winograd_never": 9}.get(algo, algo)))
 
     def force_conv_plan(self, tile=-1, slices=1):
         """Override the convolution launch planner (tile 0..3, K slices; tile 4 / 5: the Winograd forms where they apply);

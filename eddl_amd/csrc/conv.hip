@@ -1541,6 +1541,7 @@ int prof_end(hipStream_t st) {
 thread_local char g_last_kernel[128] = "";
 int g_split = 1;  // divide the tiles left over after a whole number per CU along K (set_algo 5 turns it off)
 bool g_wino = false;  // set_algo(7): the Winograd form wherever it applies (8: only where a searched plan asks for it)
+bool g_wino_never = false;  // set_algo(9): no Winograd form at all, not in the plan search and not from a kept plan
 int g_force_tile = -1, g_force_slices = -1;  // eddlhip_conv2d_force_plan
 unsigned long long *g_trace = nullptr;       // eddlhip_conv2d_trace
 long long g_trace_wgs = 0;
@@ -1905,13 +1906,14 @@ int eddlhip_conv2d_tuned_plans(int dev) {
 }
 
 int eddlhip_conv2d_set_algo(int algo) {
-    EH_REQUIRE(algo >= 0 && algo <= 8, "conv2d_set_algo: unknown algorithm %d", algo);
+    EH_REQUIRE(algo >= 0 && algo <= 9, "conv2d_set_algo: unknown algorithm %d", algo);
     if (algo == 5 || algo == 6) {
         g_split = (algo == 6);
         return 0;
     }
-    if (algo == 7 || algo == 8) {
+    if (algo >= 7 && algo <= 9) {
         g_wino = (algo == 7);
+        g_wino_never = (algo == 9);
         return 0;
     }
     g_algo = algo;
@@ -2106,7 +2108,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
         plan = forced_plan(family, g_force_tile, g_force_slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
     // the Winograd form: asked for (force_plan(4, .), set_algo(7)) or found faster by the plan search (below); never from the
     // fixed scratch array, whose size it exceeds, and not for the scalar-order or register-staged algorithm switches
-    const bool wino_ok = !gemm && !no_alloc && g_algo == 0 && winograd_applies(N, C, Kf, R, S, sr, sc, P, Q);
+    const bool wino_ok = !gemm && !no_alloc && g_algo == 0 && !g_wino_never && winograd_applies(N, C, Kf, R, S, sr, sc, P, Q);
     const bool fold_ok = wino_ok && winograd_fold_applies(N, C, Kf, R, S, sr, sc, P, Q);
     if ((wino_ok && (g_force_tile == 4 || (g_wino && g_force_tile < 0 && !g_tuning))) || (fold_ok && g_force_tile == 5))
         return conv2d_winograd(g_force_tile == 5, R, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b,

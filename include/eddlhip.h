@@ -208,7 +208,8 @@ int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const fl
  * written by the load unit straight into LDS (what 0 and 1 select); 5 / 6 = switch off / on the
  * division along K of the tiles left over after a whole number of tiles per CU (on by default;
  * independent of 0-4); 7 / 8 = switch on / off the Winograd form for every convolution it applies to
- * (off by default; independent of 5 / 6; only under 0).
+ * (off by default; independent of 5 / 6; only under 0); 9 = no Winograd form at all: the plan search does not try
+ * it and a kept plan that names it runs the planner's own choice instead (8 returns to the default).
  *
  * The Winograd form, F(2x2, 3x3): a 3x3 stride-1 convolution (any paddings, one or two input tensors, stored or
  * upsampled image) computed as an input transform, 16 products of [Kf x C] by [C x blocks of 2x2 outputs] matrices -
@@ -221,7 +222,10 @@ int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const fl
  * everywhere by 7, or by eddlhip_conv2d_force_plan(4, .).  A second form, for input channel counts that are multiples of
  * 16 (force_plan(5, .), or the search): one product launch walks through all 16 patch positions and folds each product
  * into the outputs as it completes, so the products are never written and there is no output-transform launch; it sums
- * the 16 positions in another order than the first form (same tolerance, not the same bits).
+ * the 16 positions in another order than the first form (same tolerance, not the same bits).  Non-finite inputs: the
+ * transforms take differences of neighbouring pixels, so an infinity in the input can turn into NaN in outputs where the
+ * direct form yields an infinity (all finite inputs give finite outputs as in the direct form); a caller that relies on
+ * the propagation of infinities keeps the plan search off or calls eddlhip_conv2d_set_algo(9).
  *
  * eddlhip_conv2d_last_kernel() names the kernel the calling thread's last eddlhip_conv2d_fwd
  * launched, followed by " +ksplit(T tiles x S)" when T tiles were divided into S slices; for the Winograd form

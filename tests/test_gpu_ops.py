@@ -484,6 +484,43 @@ def test_conv2d_winograd_form_only_where_it_applies_and_with_kept_filters(hip, o
         hip.set_conv_algo("auto")
 
 
+def test_conv2d_winograd_never_keeps_infinities_where_the_direct_form_has_them(hip):
+    """set_conv_algo("winograd_never"): neither a forced plan nor the plan search takes a Winograd form, so an infinity in
+    the input stays an infinity in exactly the outputs whose window holds it (the transforms would subtract it from itself)."""
+    rng = np.random.default_rng(91)
+    x = rng.standard_normal((4, 64, 28, 28), dtype=np.float32)
+    x[1, 3, 5, 7] = np.inf
+    w = (rng.standard_normal((64, 64, 3, 3)) * 0.05).astype(np.float32)
+    X, Wd, O = hip.array(x), hip.array(w), hip.empty((4, 64, 28, 28))
+    hip.conv2D(X, Wd, None, O, 1, 1, 1, 1)
+    direct = O.numpy()
+    window = np.zeros((4, 64, 28, 28), bool)
+    window[1, :, 4:7, 6:9] = True
+    assert np.array_equal(np.isinf(direct), window) and not np.isnan(direct).any()
+    hip.conv_autotune(-1)
+    try:
+        hip.set_conv_algo("winograd_never")
+        hip.force_conv_plan(4, 1)
+        hip.conv2D(X, Wd, None, O, 1, 1, 1, 1)
+        assert not hip.last_conv_kernel().startswith("winograd")
+        hip.force_conv_plan(-1, 1)
+        hip.conv_autotune(True)
+        hip.conv2D(X, Wd, None, O, 1, 1, 1, 1)      # searched, without the Winograd candidates
+        assert hip.conv_tuned_plans() == 1 and not hip.last_conv_kernel().startswith("winograd")
+        got = O.numpy()
+        assert np.array_equal(np.isinf(got), window) and not np.isnan(got).any()
+        finite = ~window
+        assert np.allclose(got[finite], direct[finite], rtol=1e-4, atol=1e-5)
+        hip.set_conv_algo("winograd_off")            # back to the default: a forced Winograd plan applies again
+        hip.force_conv_plan(4, 1)
+        hip.conv2D(X, Wd, None, O, 1, 1, 1, 1)
+        assert hip.last_conv_kernel().startswith("winograd")
+    finally:
+        hip.force_conv_plan(-1, 1)
+        hip.set_conv_algo("winograd_off")
+        hip.conv_autotune(-1)
+
+
 def test_conv2d_linearity_and_empty_batch(hip, oracle):
     from eddl_amd.descriptors import ConvolDescriptor
     rng = np.random.default_rng(301)
