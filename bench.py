@@ -231,7 +231,7 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, pl
                 blocks = int(kern[kern.rindex(",") + 1:].split()[0])
                 kern = kern[len("winograd["):kern.rindex(",")]
                 conv = [l for l in op.layers if "cd" in l.attrs][0].attrs["cd"]
-                n_out, kf = op.layers[-1].out_shape[0] * op.layers[-1].out_shape[2] * op.layers[-1].out_shape[3], op.layers[-1].out_shape[1]
+                n_out, kf = conv.out_shape[0] * conv.out_shape[2] * conv.out_shape[3], conv.out_shape[1]
                 c_in = op.flops // (2 * conv.kr * conv.kc * n_out * kf)
                 positions = (conv.kr + 1) * (conv.kc + 1)          # 16 products for a 3x3 filter, 9 for a 2x2 one
                 kernel_flops, form = 2 * positions * kf * c_in * blocks, "winograd"

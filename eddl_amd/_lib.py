@@ -52,6 +52,7 @@ PROTOTYPES = {
     "eddlhip_conv2d_fwd_noalloc": [c_int, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_fwd_concat": [c_int, P, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_fwd_upsampled": [c_int, P, c_int, c_int, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
+    "eddlhip_conv2d_fwd_maxpool": [c_int, P, P, c_int, c_int, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int, P, P, P, c_int],
     "eddlhip_conv2d_cache_filters": [c_int, P, c_int, c_int, c_int, c_int],
     "eddlhip_conv2d_uncache_filters": [c_int, P],
     "eddlhip_conv2d_set_algo": [c_int],

@@ -320,11 +320,14 @@ class Backend:
     def add_scalar(self, A, B, v):
         self._check(self.lib.eddlhip_add_scalar(self.dev, A.ptr, B.ptr, A.size, v))
 
-    def conv2D(self, I, K, bias, O, sr, sc, padrt, padcl, bn=None, residual=None, relu=False, second=None, upsample=None):
+    def conv2D(self, I, K, bias, O, sr, sc, padrt, padcl, bn=None, residual=None, relu=False, second=None, upsample=None, pool=None,
+               keep=True):
         """``bn`` = (g, b, mean, var, eps) device tensors (g, b may be None) or None.  ``second``: the other half
         of the input channels as a tensor of its own (a channel Concat of ``I`` and ``second`` folded into the call).
         ``upsample`` = (rows, columns): whole factors of a nearest-neighbour UpSampling2D of ``I`` folded into the call
-        (paddings and the output size then refer to the enlarged image)."""
+        (paddings and the output size then refer to the enlarged image).  ``pool`` = (pooled, indX, indY): the 2x2,
+        stride-2 max-pool of the output in the same call (``eddlhip_conv2d_fwd_maxpool``); ``keep=False``: the
+        unpooled output ``O`` is scratch space whose contents nobody reads afterwards."""
         N, C, H, W = I.shape
         Kf, C2, R, S = K.shape
         if second is not None:
@@ -343,7 +346,14 @@ class Backend:
                 _ptr(mean), _ptr(var), eps, _ptr(residual), int(relu))
         if second is not None and upsample is not None:
             raise ValueError("a two-tensor input and an upsampled input do not combine")
-        if upsample is not None:
+        if pool is not None:
+            up = upsample if upsample is not None else (1, 1)
+            PO, IX, IY = pool
+            if tuple(PO.shape) != (N, Kf, O.shape[2] // 2, O.shape[3] // 2) or tuple(IX.shape) != tuple(PO.shape) or tuple(IY.shape) != tuple(PO.shape):
+                raise ValueError("pooled shapes %s %s %s do not match output %s" % (PO.shape, IX.shape, IY.shape, O.shape))
+            self._check(self.lib.eddlhip_conv2d_fwd_maxpool(self.dev, I.ptr, _ptr(second), int(up[0]), int(up[1]), *tail, PO.ptr, IX.ptr, IY.ptr,
+                                                            int(bool(keep))))
+        elif upsample is not None:
             self._check(self.lib.eddlhip_conv2d_fwd_upsampled(self.dev, I.ptr, int(upsample[0]), int(upsample[1]), *tail))
         elif second is None:
             self._check(self.lib.eddlhip_conv2d_fwd(self.dev, I.ptr, *tail))

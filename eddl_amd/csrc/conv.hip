@@ -119,7 +119,29 @@ struct ConvParams {
     // wP x wQ output planes, wth x wtw of them per image, wT in all (see wino_fold / wino_store_tile).
     int wspx, wth, wtw, wT, wP, wQ;
     int wps;  // patch side: 4 (3x3 filters, 16 positions) or 3 (2x2 filters, 9 positions)
+    // The Winograd epilogues only (a lane holds whole 2x2 blocks of outputs there; output planes with even sides): the
+    // 2x2, stride-2 max-pool of the finished outputs with the coordinates of each maximum (the arithmetic of
+    // maxpool_2x2s2_kernel), written next to the outputs - or instead of them when O is nullptr.
+    float *pool_O, *pool_ix, *pool_iy;
 };
+
+// One 2x2 window of finished outputs (x00 x01 / x10 x11 at rows 2 ty, 2 ty + 1 and columns 2 tx, 2 tx + 1) pooled as
+// eddlhip_maxpool2d does it: running maximum from -3.40282e38 in the order of the window scan, strictly greater wins,
+// and when nothing is greater (a window of NaN) the coordinates are left as they are.
+__device__ __forceinline__ void pool_block(const ConvParams &p, size_t pidx, int ty, int tx, float x00, float x01, float x10, float x11) {
+    float mx = -3.40282e+38f, fx = 0.0f, fy = 0.0f;
+    bool found = false;
+    const float x0 = (float)(2 * tx), y0 = (float)(2 * ty);
+    if (x00 > mx) { mx = x00; fx = x0; fy = y0; found = true; }
+    if (x01 > mx) { mx = x01; fx = x0 + 1.0f; fy = y0; found = true; }
+    if (x10 > mx) { mx = x10; fx = x0; fy = y0 + 1.0f; found = true; }
+    if (x11 > mx) { mx = x11; fx = x0 + 1.0f; fy = y0 + 1.0f; found = true; }
+    p.pool_O[pidx] = mx;
+    if (found) {
+        p.pool_ix[pidx] = fx;
+        p.pool_iy[pidx] = fy;
+    }
+}
 
 // Timeline of a workgroup for eddlhip_conv2d_trace: words 0..3 = the device's constant 100 MHz clock at the marks (entry,
 // operands of the first K-step in LDS, end of the K loop, end of the kernel with its stores drained), word 4 = where the
@@ -518,6 +540,7 @@ __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&
         const int ml = m_local + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
         if (m0 + ml >= p.Kf) continue;
         const float bias = epi[ml], mean = epi[BM + ml], sd = epi[2 * BM + ml], g = epi[3 * BM + ml], b = epi[4 * BM + ml];
+        float fin[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
 #pragma unroll
         for (int a = 0; a < 2; a++) {
             const int oy = 2 * ty + a, ox = 2 * tx;
@@ -542,6 +565,9 @@ __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&
             }
             if (p.residual) x0 = __fadd_rn(x0, r0), x1 = __fadd_rn(x1, r1);
             if (p.relu) x0 = x0 > 0.0f ? x0 : 0.0f, x1 = x1 > 0.0f ? x1 : 0.0f;
+            fin[a][0] = x0;
+            fin[a][1] = x1;
+            if (p.O == nullptr) continue;
             if (pair) {
                 *reinterpret_cast<float2 *>(p.O + oidx) = make_float2(x0, x1);
             } else {
@@ -549,6 +575,8 @@ __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&
                 if (ox + 1 < p.wQ) p.O[oidx + 1] = x1;
             }
         }
+        if (p.pool_O != nullptr)  // (even wP, wQ: both rows and both columns of the block exist)
+            pool_block(p, (((size_t)img * p.Kf + (size_t)(m0 + ml)) * p.wth + ty) * p.wtw + tx, ty, tx, fin[0][0], fin[0][1], fin[1][0], fin[1][1]);
     }
 }
 
@@ -1473,6 +1501,7 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const ConvParams p, co
             }
         }
         const ChannelEpilogue e = load_channel(p, k);
+        float fin[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
 #pragma unroll
         for (int a = 0; a < 2; a++) {
             const int oy = 2 * ty + a, ox = 2 * tx;
@@ -1501,12 +1530,20 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const ConvParams p, co
                 }
                 if (p.residual) x0 = __fadd_rn(x0, r0), x1 = __fadd_rn(x1, r1);
                 if (p.relu) x0 = x0 > 0.0f ? x0 : 0.0f, x1 = x1 > 0.0f ? x1 : 0.0f;
-                *reinterpret_cast<float2 *>(p.O + oidx) = make_float2(x0, x1);
+                fin[a][0] = x0;
+                fin[a][1] = x1;
+                if (p.O != nullptr) *reinterpret_cast<float2 *>(p.O + oidx) = make_float2(x0, x1);
             } else {
-                p.O[oidx] = apply_epilogue(p, e, v0, oidx);
-                if (ox + 1 < p.Q) p.O[oidx + 1] = apply_epilogue(p, e, v1, oidx + 1);
+                fin[a][0] = apply_epilogue(p, e, v0, oidx);
+                if (p.O != nullptr) p.O[oidx] = fin[a][0];
+                if (ox + 1 < p.Q) {
+                    fin[a][1] = apply_epilogue(p, e, v1, oidx + 1);
+                    if (p.O != nullptr) p.O[oidx + 1] = fin[a][1];
+                }
             }
         }
+        if (p.pool_O != nullptr)  // (even P, Q: both rows and both columns of the block exist)
+            pool_block(p, (((size_t)n * p.Kf + k) * th + ty) * tw + tx, ty, tx, fin[0][0], fin[0][1], fin[1][0], fin[1][1]);
     }
 }
 
@@ -1958,6 +1995,15 @@ struct GemmBatch {
     const float *Wp;
     size_t stride;
 };
+// eddlhip_conv2d_fwd_maxpool: the 2x2, stride-2 max-pool the caller wants of this thread's current convolution.  A
+// Winograd form computes it in its epilogue and says so (`done`); after any other form the entry point launches the pool
+// kernel on the convolution's output.
+struct PoolRequest {
+    float *O, *ix, *iy;
+    bool keep;  // the unpooled output is wanted as well
+    bool done;
+};
+thread_local PoolRequest *g_pool_req = nullptr;
 // Workspace a product launch may take for the partial tiles of a K-split plan: fewer than one tile per CU left over,
 // at most 16 slices each, 128 x 128 floats per tile.  The Winograd driver keeps its own buffers behind this much.
 constexpr size_t WINO_INNER_RESERVE = (size_t)16 * 255 * 128 * 128 * sizeof(float);
@@ -2128,6 +2174,8 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
             memcpy(best.key, key, sizeof(key));
             best.tile = -1;
             best.slices = 1;
+            PoolRequest *const pool_req = g_pool_req;  // the candidates are timed as plain convolutions
+            g_pool_req = nullptr;
             hipEvent_t e0, e1;
             EH_TRY_HIP(hipEventCreate(&e0));
             EH_TRY_HIP(hipEventCreate(&e1));
@@ -2190,6 +2238,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
                 }
             }
             g_tuning = false;
+            g_pool_req = pool_req;
             (void)hipEventDestroy(e0);
             (void)hipEventDestroy(e1);
             if (rc != 0) return rc;
@@ -2307,6 +2356,9 @@ int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2,
                     int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
                     const float *bn_var, float bn_eps, const float *residual, int relu) {
     hipStream_t st = state(dev).stream;
+    // a max-pool asked for with this convolution is taken into the epilogue where every 2x2 block of outputs is whole
+    PoolRequest *const pool = (g_pool_req != nullptr && !g_tuning && P % 2 == 0 && Q % 2 == 0) ? g_pool_req : nullptr;
+    if (pool != nullptr) pool->done = true;
     const int ps = fs + 1, np = ps * ps;  // patch side and positions: 4 and 16 for 3x3 filters, 3 and 9 for 2x2
     const int th = (P + 1) / 2, tw = (Q + 1) / 2;
     const int T = N * th * tw, Tp = (T + 127) / 128 * 128;
@@ -2405,6 +2457,10 @@ int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2,
         q.wp_bytes = (unsigned)((size_t)np * rows * Mp * sizeof(float));
         q.main_tiles = q.gm * q.gn; q.nslices = 1; q.slice_steps = q.nsteps;
         q.wspx = C / 16; q.wth = th; q.wtw = tw; q.wT = T; q.wP = P; q.wQ = Q; q.wps = ps;
+        if (pool != nullptr) {
+            q.pool_O = pool->O; q.pool_ix = pool->ix; q.pool_iy = pool->iy;
+            if (!pool->keep) q.O = nullptr;
+        }
         EH_REQUIRE(rows == C && (long long)q.gm * q.gn <= 0x3fffffffLL, "conv2d: internal error, folded Winograd launch");
         q.trace = (g_trace != nullptr && q.main_tiles <= g_trace_wgs) ? g_trace : nullptr;
         // K-steps of 32 channels where the runs divide into them: a workgroup's K loop is long here (16 C channels), few
@@ -2444,6 +2500,10 @@ int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2,
     p.bias = bias; p.bn_g = bn_g; p.bn_b = bn_b; p.bn_mean = bn_mean; p.bn_var = bn_var; p.residual = residual;
     p.bn_eps = bn_eps; p.relu = relu;
     p.N = N; p.Kf = Kf; p.P = P; p.Q = Q; p.PQ = P * Q;
+    if (pool != nullptr) {
+        p.pool_O = pool->O; p.pool_ix = pool->ix; p.pool_iy = pool->iy;
+        if (!pool->keep) p.O = nullptr;
+    }
     {
         const dim3 grid((unsigned)((T + 255) / 256), (unsigned)((Kf + WINO_CH - 1) / WINO_CH));
         if (ps == 4) hipLaunchKernelGGL(wino_output_kernel<4>, grid, dim3(256), 0, st, p, (const float *)M, th, tw, T, Tp);
@@ -2483,6 +2543,23 @@ int eddlhip_conv2d_fwd_upsampled(int dev, const float *I, int up_h, int up_w, co
                                  const float *residual, int relu) {
     return conv2d_fwd_impl(false, dev, I, nullptr, up_h, up_w, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
                            bn_mean, bn_var, bn_eps, residual, relu);
+}
+
+int eddlhip_conv2d_fwd_maxpool(int dev, const float *I, const float *I_second, int up_h, int up_w, const float *K, const float *bias, float *O,
+                               int N, int C, int H, int W, int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q,
+                               const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps,
+                               const float *residual, int relu, float *pool_O, float *pool_indX, float *pool_indY, int keep_O) {
+    EH_REQUIRE(P > 0 && Q > 0 && P % 2 == 0 && Q % 2 == 0, "conv2d_fwd_maxpool: the output planes must have even sides, got %d x %d", P, Q);
+    EH_REQUIRE(N == 0 || (O && pool_O && pool_indX && pool_indY), "conv2d_fwd_maxpool: NULL output tensor");
+    EH_REQUIRE(up_h >= 1 && up_w >= 1 && (I_second == nullptr || (up_h == 1 && up_w == 1)), "conv2d_fwd_maxpool: bad input form");
+    if (N == 0) return 0;
+    PoolRequest req = {pool_O, pool_indX, pool_indY, keep_O != 0, false};
+    g_pool_req = &req;
+    const int rc = conv2d_fwd_impl(false, dev, I, I_second, up_h, up_w, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g,
+                                   bn_b, bn_mean, bn_var, bn_eps, residual, relu);
+    g_pool_req = nullptr;
+    if (rc != 0 || req.done) return rc;
+    return eddlhip_maxpool2d(dev, O, pool_O, pool_indX, pool_indY, N, Kf, P, Q, 2, 2, 2, 2, 0, 0, 0, 0);
 }
 
 int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const float *bias, float *O, int N, int C, int H, int W, int Kf,

@@ -653,6 +653,22 @@ void Net::fuse() {
                 fused_away.push_back(m);
                 absorbed.push_back(m->child[0]);
             }
+            // a 2x2, stride-2, unpadded LMaxPool of the chain's output joins the call (eddlhip_conv2d_fwd_maxpool: a
+            // convolution in a Winograd form pools in its epilogue); the unpooled tensor is written only if read elsewhere
+            if (conv->cd->r % 2 == 0 && conv->cd->c % 2 == 0) {
+                for (Layer *c2 : s.last->child) {
+                    LMaxPool *mp = dynamic_cast<LMaxPool *>(c2);
+                    if (mp == nullptr || mp->parent.size() != 1) continue;
+                    const PoolDescriptor *pd = mp->pd;
+                    if (pd->ksize != vector<int>{2, 2} || pd->stride != vector<int>{2, 2} || pd->pad != vector<int>{0, 0, 0, 0}) continue;
+                    s.pool = mp;
+                    s.keep = s.last->child.size() > 1 || contains(lout, s.last);
+                    absorbed.push_back(mp);
+                    done.push_back(mp);
+                    if (!s.keep) fused_away.push_back(s.last);
+                    break;
+                }
+            }
         } else if (dynamic_cast<LDense *>(l) != nullptr) {
             s.chain = true;
             LActivation *a = dynamic_cast<LActivation *>(sole_child(l));
@@ -693,6 +709,15 @@ void Net::run_step(const FusedStep &s) {
         const float *mean = bn ? bn->mean->ptr : nullptr, *var = bn ? bn->variance->ptr : nullptr;
         const float eps = bn ? bn->epsilon : 0.0f;
         const float *res = s.res ? s.res->output->ptr : nullptr;
+        if (s.pool != nullptr) {
+            const int c_in = s.src2 != nullptr ? 2 * I->shape[1] : I->shape[1];
+            gpu_check(eddlhip_conv2d_fwd_maxpool(device, I->ptr, s.src2 != nullptr ? s.src2->output->ptr : nullptr, s.up_h, s.up_w, D->K->ptr, bias,
+                                                 O->ptr, I->shape[0], c_in, I->shape[2], I->shape[3], D->nk, D->kr, D->kc, D->sr, D->sc,
+                                                 s.pad_top, s.pad_left, D->r, D->c, g, b, mean, var, eps, res, s.relu ? 1 : 0,
+                                                 s.pool->output->ptr, s.pool->pd->indX->ptr, s.pool->pd->indY->ptr, s.keep ? 1 : 0),
+                      "Net::forward (fused convolution and max-pool)");
+            return;
+        }
         if (s.up_h != 1 || s.up_w != 1)
             gpu_check(eddlhip_conv2d_fwd_upsampled(device, I->ptr, s.up_h, s.up_w, D->K->ptr, bias, O->ptr, I->shape[0], I->shape[1],
                                                    I->shape[2], I->shape[3], D->nk, D->kr, D->kc, D->sr, D->sc, s.pad_top, s.pad_left,

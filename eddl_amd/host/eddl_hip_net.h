@@ -225,6 +225,8 @@ struct FusedStep {
     int pad_top = 0, pad_left = 0;
     int up_h = 1, up_w = 1;     // conv chains: whole factors of a folded nearest UpSampling2D (src is then its parent)
     bool chain = false;         // false: first->forward()
+    LPool *pool = nullptr;      // conv chains: a 2x2, stride-2, unpadded LMaxPool of last's output computed by the same call
+    bool keep = true;           // conv chains with a pool: some other layer (or the caller) reads last's output as well
 };
 
 class Net {

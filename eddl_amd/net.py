@@ -467,8 +467,25 @@ class Net:
             chain.append(cur)
         for m in chain:
             absorbed.add(id(m))
+        # a 2x2, stride-2, unpadded MaxPool of the chain's output joins the call (eddlhip_conv2d_fwd_maxpool: a convolution
+        # in a Winograd form pools in its epilogue); the unpooled tensor is kept only if somebody else reads it
+        pool, keep = None, True
+        if fuse and cd.out_shape[2] % 2 == 0 and cd.out_shape[3] % 2 == 0:
+            for c in last.children:
+                pd = c.attrs.get("pd")
+                if c.kind == "maxpool2d" and len(c.parents) == 1 and list(pd.ksize) == [2, 2] and list(pd.stride) == [2, 2] and not any(pd.pad):
+                    pool = c
+                    keep = len(last.children) > 1 or last in self.lout
+                    absorbed.add(id(c))
+                    break
         O = hip.empty(last.out_shape)
-        self.out[id(last)] = O
+        if keep:
+            self.out[id(last)] = O
+        pooled = None
+        if pool is not None:
+            pooled = (hip.empty(pool.out_shape), hip.full(pool.out_shape, 0.0), hip.full(pool.out_shape, 0.0))
+            self.out[id(pool)] = pooled[0]
+            self.aux[id(pool)] = {"indX": pooled[1], "indY": pooled[2]}
         I = self.out[id(src)]
         dp = self.dparams[id(l)]
         bias = dp["bias"] if cd.use_bias else None
@@ -486,10 +503,15 @@ class Net:
         name = "+".join(m.name for m in ([l] if not chain else [l] + chain))
         if src is not l.parents[0]:
             name = l.parents[0].name + "+" + name
+        members = [l] + chain
+        if pool is not None:
+            name += "+" + pool.name
+            members = members + [pool]
+            nbytes += 12 * int(np.prod(pool.out_shape)) - (0 if keep else 4 * N * Kf * P * Q)
         self.ops.append(Op("conv2d", name,
                            lambda: hip.conv2D(I, dp["K"], bias, O, cd.sr, cd.sc, pt, pl, bn=dbn, residual=R, relu=relu, second=second,
-                                              upsample=upsample),
-                           flops, nbytes, [l] + chain))
+                                              upsample=upsample, pool=pooled, keep=keep),
+                           flops, nbytes, members))
 
     def _emit_dense(self, l, fuse, absorbed, sole_child):
         """LDense::forward = mult2D + sum2D_rowwise (src/layers/core/layer_dense.cpp:65-73); a fused plan

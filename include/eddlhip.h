@@ -180,6 +180,22 @@ int eddlhip_conv2d_fwd_upsampled(int dev, const float *I, int up_h, int up_w, co
                                  const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var,
                                  float bn_eps, const float *residual, int relu);
 
+/* A convolution (with its fused epilogue) whose output goes through a 2x2, stride-2, unpadded max-pool - the
+ * Conv -> [BN] -> ReLU -> MaxPool(2, 2) step of the reference's VGG and U-Net encoders (LMaxPool::forward after
+ * LConv::forward, src/layers/pool/layer_maxpool.cpp:62-64 and src/layers/conv/layer_conv2D.cpp:91-93) as one call.
+ * O, pool_O, pool_indX and pool_indY receive exactly what eddlhip_conv2d_fwd (or _concat with I_second != NULL, or
+ * _upsampled with up_h, up_w > 1) followed by eddlhip_maxpool2d(O, 2, 2, 2, 2, no padding) would write, bit for bit
+ * for the convolution form the call takes.  P and Q must be even.  Where the convolution runs in a Winograd form its
+ * epilogue holds whole 2x2 blocks of outputs and pools them itself: no pool launch, and with keep_O == 0 the unpooled
+ * outputs are not written at all (O must still be a buffer of the full size: the other forms compute it and pool it
+ * with the pool kernel; its contents after a call with keep_O == 0 are unspecified). */
+int eddlhip_conv2d_fwd_maxpool(int dev, const float *I, const float *I_second, int up_h, int up_w, const float *K,
+                               const float *bias, float *O, int N, int C, int H, int W, int Kf, int R, int S, int sr, int sc,
+                               int pad_top, int pad_left, int P, int Q,
+                               const float *bn_g, const float *bn_b, const float *bn_mean, const float *bn_var,
+                               float bn_eps, const float *residual, int relu,
+                               float *pool_O, float *pool_indX, float *pool_indY, int keep_O);
+
 /* eddlhip_conv2d_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid it).  No counterpart in the reference.  Same arguments, same kernels,
  * same launch plan and therefore the same result, bit for bit, as eddlhip_conv2d_fwd; the difference is where

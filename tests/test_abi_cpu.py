@@ -29,7 +29,7 @@ def test_version_and_argument_errors_without_a_device():
     from eddl_amd import _lib
     lib = _lib.load()
     assert b"gfx950" in lib.eddlhip_version()
-    assert lib.eddlhip_conv2d_set_algo(9) == -1
+    assert lib.eddlhip_conv2d_set_algo(10) == -1
     assert b"unknown algorithm" in lib.eddlhip_last_error()
     assert lib.eddlhip_conv2d_set_algo(0) == 0
     lp, lq = ctypes.c_int(), ctypes.c_int()

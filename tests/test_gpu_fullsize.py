@@ -149,7 +149,7 @@ def test_winograd_forms_at_full_size(hip, oracle, workload, form):
             assert hip.last_conv_kernel().startswith("winograd["), hip.last_conv_kernel()
     finally:
         hip.force_conv_plan(-1, 1)
-        hip.set_conv_algo("auto")
+        hip.set_conv_algo("winograd_off")
 
 
 def test_conv_scaling_by_powers_of_two_is_exact_at_full_size(hip):

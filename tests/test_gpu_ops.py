@@ -484,6 +484,79 @@ def test_conv2d_winograd_form_only_where_it_applies_and_with_kept_filters(hip, o
         hip.set_conv_algo("auto")
 
 
+@pytest.mark.parametrize("form", [-1, 4, 5])
+@pytest.mark.parametrize("case", ["bias+relu", "bn+residual+relu", "2x2 filter", "two tensors", "upsampled", "nan window"])
+def test_conv2d_fwd_maxpool_is_the_convolution_followed_by_the_pool(hip, form, case):
+    """eddlhip_conv2d_fwd_maxpool against eddlhip_conv2d_fwd* + eddlhip_maxpool2d(2, 2, 2, 2) under the same launch plan
+    (the planner's direct form, the Winograd form in three kernels, the folded Winograd form): pooled values and both
+    index tensors bit for bit, the unpooled output too when it is kept; a window of NaN leaves the indices as they were."""
+    cases = ["bias+relu", "bn+residual+relu", "2x2 filter", "two tensors", "upsampled", "nan window"]
+    rng = np.random.default_rng(500 + 10 * (form + 1) + cases.index(case))
+    N, C, H, W, Kf, fs = 3, 32, 12, 16, 48, 3
+    second = upsample = None
+    if case == "2x2 filter":
+        fs = 2
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    X = hip.array(x)
+    if case == "two tensors":
+        second = hip.array(rng.standard_normal((N, C, H, W), dtype=np.float32))
+    if case == "upsampled":
+        upsample = (2, 2)
+    Cin = 2 * C if second is not None else C
+    Hu, Wu = (H * 2, W * 2) if upsample else (H, W)
+    w = hip.array((rng.standard_normal((Kf, Cin, fs, fs)) * 0.1).astype(np.float32))
+    pad = 1 if fs == 3 else 0
+    P, Q = (Hu, Wu) if fs == 3 else (Hu, Wu)          # 2x2: one more row and column of zeros below and to the right
+    bias = hip.array(rng.standard_normal(Kf).astype(np.float32)) if case in ("bias+relu", "2x2 filter", "nan window") else None
+    bn = res = None
+    if case == "bn+residual+relu":
+        bn = (hip.array(rng.uniform(0.8, 1.2, Kf).astype(np.float32)), hip.array((rng.standard_normal(Kf) * 0.1).astype(np.float32)),
+              hip.array((rng.standard_normal(Kf) * 0.1).astype(np.float32)), hip.array(rng.uniform(0.5, 1.5, Kf).astype(np.float32)), 1e-5)
+    if case in ("bn+residual+relu", "nan window"):
+        r = rng.standard_normal((N, Kf, P, Q), dtype=np.float32)
+        if case == "nan window":
+            r[1, 5, 4:6, 6:8] = np.nan
+        res = hip.array(r)
+    relu = case != "nan window"                        # (the ReLU of this path turns NaN into 0)
+    O1, O2 = hip.full((N, Kf, P, Q), 3.0), hip.full((N, Kf, P, Q), 4.0)
+    pooled = lambda: (hip.full((N, Kf, P // 2, Q // 2), 9.0), hip.full((N, Kf, P // 2, Q // 2), 7.0), hip.full((N, Kf, P // 2, Q // 2), 7.0))
+    A, B, K2 = pooled(), pooled(), pooled()
+    try:
+        hip.force_conv_plan(form, 1)
+        hip.conv2D(X, w, bias, O1, 1, 1, pad, pad, bn=bn, residual=res, relu=relu, second=second, upsample=upsample)
+        name = hip.last_conv_kernel()
+        assert name.startswith("winograd") == (form >= 4), name
+        hip.mpool2D(O1, A[0], A[1], A[2], (2, 2), (2, 2), (0, 0, 0, 0))
+        hip.conv2D(X, w, bias, O2, 1, 1, pad, pad, bn=bn, residual=res, relu=relu, second=second, upsample=upsample, pool=B, keep=True)
+        assert hip.last_conv_kernel() == name
+        ref = O1.numpy()
+        assert np.array_equal(ref, O2.numpy(), equal_nan=True), name
+        for a, b, what in zip(A, B, ("pooled", "indX", "indY")):
+            assert np.array_equal(a.numpy(), b.numpy()), what + " " + name
+        if case == "nan window":
+            assert A[0].numpy()[1, 5, 2, 3] == np.float32(-3.40282e38) and A[1].numpy()[1, 5, 2, 3] == 7.0
+        # without the unpooled output: the same pooled tensors; a Winograd form leaves O alone
+        O3 = hip.full((N, Kf, P, Q), 5.0)
+        hip.conv2D(X, w, bias, O3, 1, 1, pad, pad, bn=bn, residual=res, relu=relu, second=second, upsample=upsample, pool=K2, keep=False)
+        for a, b, what in zip(A, K2, ("pooled", "indX", "indY")):
+            assert np.array_equal(a.numpy(), b.numpy()), what + " without the output, " + name
+        if name.startswith("winograd"):
+            assert np.all(O3.numpy() == 5.0)
+        # the gathered maxima are the kept outputs at the reported coordinates
+        if case != "nan window":
+            n, k = np.indices(A[0].shape)[:2]
+            assert np.array_equal(ref[n, k, A[2].numpy().astype(np.int64), A[1].numpy().astype(np.int64)], A[0].numpy())
+    finally:
+        hip.force_conv_plan(-1, 1)
+
+
+def test_conv2d_fwd_maxpool_refuses_odd_output_planes(hip):
+    X, w, O = hip.array(np.zeros((1, 4, 7, 8), np.float32)), hip.array(np.zeros((8, 4, 3, 3), np.float32)), hip.empty((1, 8, 7, 8))
+    pooled = (hip.empty((1, 8, 3, 4)), hip.empty((1, 8, 3, 4)), hip.empty((1, 8, 3, 4)))
+    with pytest.raises(Exception, match="even sides"):
+        hip.conv2D(X, w, None, O, 1, 1, 1, 1, pool=pooled)
+
+
 def test_conv2d_winograd_never_keeps_infinities_where_the_direct_form_has_them(hip):
     """set_conv_algo("winograd_never"): neither a forced plan nor the plan search takes a Winograd form, so an infinity in
     the input stays an infinity in exactly the outputs whose window holds it (the transforms would subtract it from itself)."""
