@@ -170,9 +170,10 @@ def test_cpp_graphs_match_the_python_runner_bit_for_bit(hip, which, fused, tmp_p
 
 def test_cpp_host_runs_the_plans_a_python_process_saved(hip, tmp_path):
     """Plans travel between processes as a file: the Python host searches a block's convolution once, and the file it saves
-    is rewritten, once to an undivided plan and once to a four-way K-split (so that the plan in force is known).  The C++ host
-    started with either file must give what the Python host gives with that file, bit for bit; the two plans sum in different
-    orders, so the two results differ from each other in their last bits."""
+    is rewritten, to an undivided plan, to a four-way K-split and to the folded Winograd form (so that the plan in force is
+    known; under the last the block's max-pool is computed in the convolution's epilogue).  The C++ host started with any of
+    the files must give what the Python host gives with that file, bit for bit; the plans sum in different orders, so
+    their results differ from each other in their last bits."""
     from eddl_amd import models
     batch, ch, size = 3, 64, 28
     m = models.conv_bn_relu_pool_block(batch=batch, channels=ch, size=size, filters=ch)
@@ -194,19 +195,21 @@ def test_cpp_host_runs_the_plans_a_python_process_saved(hip, tmp_path):
         keys = [l.split("|")[0] for l in lines if l and not l.startswith("#")]
         keys = [k for k in keys if k.split()[:5] == [str(batch), str(ch), str(ch), "3", "3"]]
         assert len(keys) == 1, lines
-        for plan in ("2 1", "2 4"):
-            with open(plans + plan[-1], "w") as f:
+        for plan in ("2 1", "2 4", "5 1"):          # 5: the folded Winograd form, which also pools in its own epilogue
+            with open(plans + plan.replace(" ", "_"), "w") as f:
                 f.write("# rewritten by the test\n" + keys[0] + "| " + plan + "\n")
             hip.conv_autotune(-1)
-            hip.conv_tuned_load(plans + plan[-1])
+            hip.conv_tuned_load(plans + plan.replace(" ", "_"))
             hip.conv_autotune(True)
             want[plan] = m.predict([x])[0]
+            assert hip.last_conv_kernel().startswith("winograd") == (plan == "5 1")
     finally:
         hip.conv_autotune(-1)
     assert not np.array_equal(want["2 1"], want["2 4"]) and np.allclose(want["2 1"], want["2 4"], rtol=1e-4, atol=1e-5)
+    assert not np.array_equal(want["2 1"], want["5 1"]) and np.allclose(want["2 1"], want["5 1"], rtol=1e-4, atol=1e-5)
     for plan in want:
         res = subprocess.run([NET_DRIVER, "fused:block", str(tmp_path / "params.bin"), str(tmp_path / "x.raw"), str(tmp_path / "y.raw"), str(batch), str(size), str(ch), str(ch)],
-                             stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300, env=dict(os.environ, EDDLHIP_PLANS=plans + plan[-1]))
+                             stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300, env=dict(os.environ, EDDLHIP_PLANS=plans + plan.replace(" ", "_")))
         assert res.returncode == 0 and "plans: 1 geometries loaded" in res.stdout and "FAILED" not in res.stdout, (res.stdout[-2000:], res.stderr[-2000:])
         got = np.fromfile(tmp_path / "y.raw", np.float32).reshape(want[plan].shape)
         assert np.array_equal(got, want[plan]), plan
