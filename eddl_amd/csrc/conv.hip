@@ -522,10 +522,57 @@ __device__ __forceinline__ void wino_fold(floatx16 (&y)[2][2], floatx16 &acc, in
     for (int v = 0; v < 16; v++) acc[v] = 0.0f;
 }
 
+// One filter row's four outputs of one 2x2 block (y00 y01 / y10 y11 at rows 2 ty, 2 ty + 1 and columns 2 tx, 2 tx + 1 of
+// image `img`): the convolution's epilogue value by value (the arithmetic of apply_epilogue), two outputs of a row per
+// store where the rows are aligned for it (`pair`), and the block's max-pool where one is asked for.  `epi`: the tile's
+// channel constants (stage_channel_constants), ml: the row within the tile.
+template <int BM>
+__device__ __forceinline__ void wino_store_row(const ConvParams &p, const float *epi, int m0, int ml, int img, int ty, int tx, size_t plane, bool pair,
+                                               float y00, float y01, float y10, float y11) {
+    if (m0 + ml >= p.Kf) return;
+    const float bias = epi[ml], mean = epi[BM + ml], sd = epi[2 * BM + ml], g = epi[3 * BM + ml], b = epi[4 * BM + ml];
+    const float yy[2][2] = {{y00, y01}, {y10, y11}};
+    float fin[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+        const int oy = 2 * ty + a, ox = 2 * tx;
+        if (oy >= p.wP) continue;
+        const size_t oidx = ((size_t)img * p.Kf + (size_t)(m0 + ml)) * plane + (size_t)oy * p.wQ + ox;
+        float x0 = yy[a][0], x1 = yy[a][1];
+        float r0 = 0.0f, r1 = 0.0f;
+        if (p.residual) {
+            if (pair) {
+                const float2 rr = *reinterpret_cast<const float2 *>(p.residual + oidx);
+                r0 = rr.x;
+                r1 = rr.y;
+            } else {
+                r0 = p.residual[oidx];
+                if (ox + 1 < p.wQ) r1 = p.residual[oidx + 1];
+            }
+        }
+        if (p.bias) x0 = __fadd_rn(x0, bias), x1 = __fadd_rn(x1, bias);
+        if (p.bn_mean) {
+            x0 = __fdiv_rn(__fsub_rn(x0, mean), sd), x1 = __fdiv_rn(__fsub_rn(x1, mean), sd);
+            if (p.bn_g) x0 = __fadd_rn(__fmul_rn(x0, g), b), x1 = __fadd_rn(__fmul_rn(x1, g), b);
+        }
+        if (p.residual) x0 = __fadd_rn(x0, r0), x1 = __fadd_rn(x1, r1);
+        if (p.relu) x0 = x0 > 0.0f ? x0 : 0.0f, x1 = x1 > 0.0f ? x1 : 0.0f;
+        fin[a][0] = x0;
+        fin[a][1] = x1;
+        if (p.O == nullptr) continue;
+        if (pair) {
+            *reinterpret_cast<float2 *>(p.O + oidx) = make_float2(x0, x1);
+        } else {
+            p.O[oidx] = x0;
+            if (ox + 1 < p.wQ) p.O[oidx + 1] = x1;
+        }
+    }
+    if (p.pool_O != nullptr)  // (even wP, wQ: both rows and both columns of the block exist)
+        pool_block(p, (((size_t)img * p.Kf + (size_t)(m0 + ml)) * p.wth + ty) * p.wtw + tx, ty, tx, fin[0][0], fin[0][1], fin[1][0], fin[1][1]);
+}
+
 // A wavefront's 32 filters x 32 blocks: lane = block (column) lane % 32, filter rows 8 * (v / 4) + 4 * (lane / 32) + v % 4.
-// The convolution's epilogue value by value (the arithmetic of apply_epilogue), two outputs of a row per store where
-// the rows are aligned for it.  `epi`: the tile's channel constants (stage_channel_constants); m_local: the
-// wavefront's first row in the tile.
+// `epi`: the tile's channel constants (stage_channel_constants); m_local: the wavefront's first row in the tile.
 template <int BM>
 __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&y)[2][2], const float *epi, int m0, int m_local, int n_base,
                                                 int lane) {
@@ -538,45 +585,7 @@ __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&
 #pragma unroll
     for (int v = 0; v < 16; v++) {
         const int ml = m_local + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-        if (m0 + ml >= p.Kf) continue;
-        const float bias = epi[ml], mean = epi[BM + ml], sd = epi[2 * BM + ml], g = epi[3 * BM + ml], b = epi[4 * BM + ml];
-        float fin[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
-#pragma unroll
-        for (int a = 0; a < 2; a++) {
-            const int oy = 2 * ty + a, ox = 2 * tx;
-            if (oy >= p.wP) continue;
-            const size_t oidx = ((size_t)img * p.Kf + (size_t)(m0 + ml)) * plane + (size_t)oy * p.wQ + ox;
-            float x0 = y[a][0][v], x1 = y[a][1][v];
-            float r0 = 0.0f, r1 = 0.0f;
-            if (p.residual) {
-                if (pair) {
-                    const float2 rr = *reinterpret_cast<const float2 *>(p.residual + oidx);
-                    r0 = rr.x;
-                    r1 = rr.y;
-                } else {
-                    r0 = p.residual[oidx];
-                    if (ox + 1 < p.wQ) r1 = p.residual[oidx + 1];
-                }
-            }
-            if (p.bias) x0 = __fadd_rn(x0, bias), x1 = __fadd_rn(x1, bias);
-            if (p.bn_mean) {
-                x0 = __fdiv_rn(__fsub_rn(x0, mean), sd), x1 = __fdiv_rn(__fsub_rn(x1, mean), sd);
-                if (p.bn_g) x0 = __fadd_rn(__fmul_rn(x0, g), b), x1 = __fadd_rn(__fmul_rn(x1, g), b);
-            }
-            if (p.residual) x0 = __fadd_rn(x0, r0), x1 = __fadd_rn(x1, r1);
-            if (p.relu) x0 = x0 > 0.0f ? x0 : 0.0f, x1 = x1 > 0.0f ? x1 : 0.0f;
-            fin[a][0] = x0;
-            fin[a][1] = x1;
-            if (p.O == nullptr) continue;
-            if (pair) {
-                *reinterpret_cast<float2 *>(p.O + oidx) = make_float2(x0, x1);
-            } else {
-                p.O[oidx] = x0;
-                if (ox + 1 < p.wQ) p.O[oidx + 1] = x1;
-            }
-        }
-        if (p.pool_O != nullptr)  // (even wP, wQ: both rows and both columns of the block exist)
-            pool_block(p, (((size_t)img * p.Kf + (size_t)(m0 + ml)) * p.wth + ty) * p.wtw + tx, ty, tx, fin[0][0], fin[0][1], fin[1][0], fin[1][1]);
+        wino_store_row<BM>(p, epi, m0, ml, img, ty, tx, plane, pair, y[0][0][v], y[0][1][v], y[1][0][v], y[1][1][v]);
     }
 }
 
@@ -1271,8 +1280,9 @@ struct WinoParams {
 };
 constexpr int WINO_CH = 4;  // channels (input transform) or filters (output transform) per thread
 
+// (cmajor: the layout of the one-launch form, U[c][position][Mp]; otherwise one packed matrix per position, U[position][rows][Mp])
 template <int PS>
-__global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restrict__ K, float *__restrict__ U, int Kf, int C, int Mp, int rows) {
+__global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restrict__ K, float *__restrict__ U, int Kf, int C, int Mp, int rows, int cmajor) {
     constexpr int R = PS - 1;
     const int idx = blockIdx.x * 256 + threadIdx.x;  // (c, k), k fastest: row c of the packed matrices
     if (idx >= rows * Mp) return;
@@ -1281,6 +1291,7 @@ __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restric
 #pragma unroll
     for (int i = 0; i < R * R; i++) g[i] = (c < C && k < Kf) ? K[((size_t)k * C + c) * (R * R) + i] : 0.0f;
     const size_t plane = (size_t)rows * Mp;
+    auto at = [&](int e) -> float & { return cmajor ? U[((size_t)c * (PS * PS) + e) * Mp + k] : U[(size_t)e * plane + idx]; };
     if constexpr (PS == 4) {
         float t[4][3];
 #pragma unroll
@@ -1292,10 +1303,10 @@ __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restric
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            U[(size_t)(4 * i + 0) * plane + idx] = t[i][0];
-            U[(size_t)(4 * i + 1) * plane + idx] = __fmul_rn(0.5f, __fadd_rn(__fadd_rn(t[i][0], t[i][1]), t[i][2]));
-            U[(size_t)(4 * i + 2) * plane + idx] = __fmul_rn(0.5f, __fadd_rn(__fsub_rn(t[i][0], t[i][1]), t[i][2]));
-            U[(size_t)(4 * i + 3) * plane + idx] = t[i][2];
+            at(4 * i + 0) = t[i][0];
+            at(4 * i + 1) = __fmul_rn(0.5f, __fadd_rn(__fadd_rn(t[i][0], t[i][1]), t[i][2]));
+            at(4 * i + 2) = __fmul_rn(0.5f, __fadd_rn(__fsub_rn(t[i][0], t[i][1]), t[i][2]));
+            at(4 * i + 3) = t[i][2];
         }
     } else {
         float t[3][2];
@@ -1307,9 +1318,9 @@ __global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restric
         }
 #pragma unroll
         for (int i = 0; i < 3; i++) {
-            U[(size_t)(3 * i + 0) * plane + idx] = t[i][0];
-            U[(size_t)(3 * i + 1) * plane + idx] = __fadd_rn(t[i][0], t[i][1]);
-            U[(size_t)(3 * i + 2) * plane + idx] = t[i][1];
+            at(3 * i + 0) = t[i][0];
+            at(3 * i + 1) = __fadd_rn(t[i][0], t[i][1]);
+            at(3 * i + 2) = t[i][1];
         }
     }
 }
@@ -1547,6 +1558,280 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const ConvParams p, co
     }
 }
 
+// Issue order of one channel pair of wino_fused_kernel (see there): H1 matrix instructions, each followed by its share of
+// NDS LDS reads, then H2 matrix instructions, each followed by its share of NVALU vector instructions.
+template <int NDS, int NVALU, int H1, int H2, int K>
+__device__ __forceinline__ void wino_sched_pair() {
+    if constexpr (K < H1) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        constexpr int n = (NDS * (K + 1)) / H1 - (NDS * K) / H1;
+        if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(0x100, n, 0);
+        wino_sched_pair<NDS, NVALU, H1, H2, K + 1>();
+    } else if constexpr (K < H1 + H2) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        constexpr int n = (NVALU * (K - H1 + 1)) / H2 - (NVALU * (K - H1)) / H2;
+        (void)n;  // (the additions are left to the scheduler: address arithmetic counts as vector work, too)
+        wino_sched_pair<NDS, NVALU, H1, H2, K + 1>();
+    }
+}
+
+// ---------------------------------------------------------------- Winograd F(2x2, 3x3) in one launch, no transformed input in memory
+// The whole convolution - input transform, the 16 products, output transform, epilogue - in ONE kernel that reads the
+// NCHW input itself.  The loop order is channels outermost: a workgroup owns a tile of 32 FM filters x 32 FN blocks (2x2
+// output blocks, numbered image by image, row by row) and keeps the accumulators of ALL 16 patch positions of that tile,
+// wavefront i those of position row i (positions 4 i .. 4 i + 3: 4 FM FN blocks of 32x32 per wavefront).  A K-step is CK
+// input channels:
+//   * the load unit writes the step's slice of the transformed filters, U[c][position][filter] (wino_filter_kernel's
+//     channel-major layout: a step's slice of a filter tile is 16 CK rows of 32 FM floats), and the RAW 4x4 patches
+//     of the tile's blocks, R[c][patch element][block], into LDS (buffer_load ... lds; a patch element outside the image,
+//     or of a block past the end, has an out-of-range offset and arrives as 0, as in conv_tap_kernel's gather);
+//   * a lane derives its B operands itself: position row i of V = B^T d B needs two patch rows (i = 0: row 0 - row 2,
+//     1: row 1 + row 2, 2: row 2 - row 1, 3: row 1 - row 3), i.e. eight LDS reads and four additions give the row
+//     combination u[0..3] of the lane's (block, channel), and four more give the wavefront's four operands
+//     u0 - u2, u1 + u2, u2 - u1, u1 - u3 - the very operations, in the very order, of wino_input_store, so V has the bits
+//     it has in the other Winograd forms; it is never stored.
+// After the last channel the wavefronts combine their positions' products along the row (s0 = m0 + m1 + m2,
+// s1 = m1 - m2 - m3), exchange s through LDS, and wavefront q finishes filter rows 8 q + 4 (lane / 32) + 0..3 of every
+// block: y[a][b] = s[0][b] + s[1][b] + s[2][b] (a = 0), s[1][b] - s[2][b] - s[3][b] (a = 1), then the convolution's
+// epilogue (wino_store_row).  Sums: channels in increasing order, two per matrix instruction, one accumulator per
+// position from the first channel to the last; the output transform in the order just given.  Whole tiles only.
+template <int FM, int FN, int CK, int WPE>  // WPE: wavefronts per SIMD the register budget is set for
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void wino_fused_kernel(const ConvParams p) {
+    static_assert(CK % 4 == 0 && FN <= 2 && FM <= 2, "a wavefront stages whole channels; a lane gathers one block");
+    constexpr int MF = 32 * FM, NB = 32 * FN;
+    constexpr int U_FLOATS = CK * 16 * MF;  // a step's filter slice  [c][position][MF]
+    constexpr int R_FLOATS = CK * 16 * NB;  // a step's raw patches   [c][patch element][NB]
+    constexpr int BUF_FLOATS = U_FLOATS + R_FLOATS;
+    constexpr int XCH_FLOATS = 4 * 2 * 16 * 64;  // the exchange of one 32x32 block: [position row][b][v][lane]
+    constexpr int LDS_FLOATS = 2 * BUF_FLOATS > XCH_FLOATS ? 2 * BUF_FLOATS : XCH_FLOATS;
+    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+    __shared__ float epi[5 * MF];
+
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, half = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int m_tile, n_tile, local_tile, slice;
+    bool split;
+    trace_mark(p, 0);
+    tile_of_block(p, m_tile, n_tile, local_tile, slice, split);
+    const int m0 = m_tile * MF, n0 = n_tile * NB;
+    put_channel_constants<MF>(epi, fetch_channel_constants<MF>(p, m0, tid), tid);  // (published by the loop's first barrier)
+
+    // ---- where the tile's pixels go in LDS, and where this lane's patches lie there.  The tile's blocks are a run of
+    // consecutive blocks, i.e. a few SEGMENTS of block rows (a segment: cnt neighbouring blocks of one row of blocks of one
+    // image).  A segment's blocks share pixels with their neighbours, so it is staged as the 4 pixel rows it touches,
+    // 2 cnt + 2 pixels each, every pixel once: slot (segment base) + r (2 cnt + 2) + x is pixel (2 ty - pad_top + r,
+    // 2 tx_first - pad_left + x).  The slots of a channel are consecutive LDS floats, slot k * 64 + lane is written by lane
+    // `lane` of load k: its byte offset in a channel plane (or out of range: padding, a block past the end) is worked out
+    // here once.  16 NB slots always suffice (a segment of one block takes 16).
+    constexpr int SLOTS = 16 * NB, WLC = SLOTS / 64;
+    const int per_img = p.wth * p.wtw;
+    int voff[WLC], my_base[FN], my_stride[FN];
+#pragma unroll
+    for (int k = 0; k < WLC; k++) voff[k] = OOB;
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) my_base[fn] = 0, my_stride[fn] = 0;  // (a block past the end reads slot 0: never stored)
+    int nload;
+    {
+        const int n_end = min(n0 + NB, p.wT);
+        const unsigned Hu = (unsigned)(p.H * p.uh), Wu = (unsigned)(p.W * p.uw);
+        const int img_elems = p.Cimg * p.H * p.W;
+        int base = 0;
+        for (int seg_n = n0; seg_n < n_end;) {  // (uniform)
+            const int row = seg_n / p.wtw, tx0 = seg_n - row * p.wtw;
+            const int cnt = min(p.wtw - tx0, n_end - seg_n), width = 2 * cnt + 2;
+            const int img = row / p.wth, ty = row - img * p.wth;
+            const int y0 = 2 * ty - p.pt, x0 = 2 * tx0 - p.pl, gbase = img * img_elems;
+#pragma unroll
+            for (int k = 0; k < WLC; k++) {
+                const int local = k * 64 + lane - base;
+                if (local >= 0 && local < 4 * width) {
+                    const int r = (local >= width ? 1 : 0) + (local >= 2 * width ? 1 : 0) + (local >= 3 * width ? 1 : 0);
+                    const unsigned y = (unsigned)(y0 + r), x = (unsigned)(x0 + local - r * width);
+                    if (y < Hu && x < Wu) voff[k] = (gbase + (int)(y / (unsigned)p.uh) * p.W + (int)(x / (unsigned)p.uw)) * 4;
+                }
+            }
+#pragma unroll
+            for (int fn = 0; fn < FN; fn++) {
+                const int n = n0 + fn * 32 + l32;
+                if (n >= seg_n && n < seg_n + cnt) my_base[fn] = base + 2 * (n - seg_n), my_stride[fn] = width;
+            }
+            base += 4 * width;
+            seg_n += cnt;
+        }
+        nload = (base + 63) >> 6;  // loads per channel that carry slots in use
+    }
+    const int HW4 = p.H * p.W * 4;
+    const int32x4 dma_w = make_rsrc_words(p.Wp, p.wp_bytes), dma_in = make_rsrc_words(p.I, p.in_bytes);
+    const int32x4 dma_in2 = make_rsrc_words(p.I2, p.in_bytes);
+    // filter slice: a wavefront instruction moves 256 consecutive floats of the slice, i.e. RPI whole rows of MF
+    constexpr int RPI = 256 / MF, U_UNITS = U_FLOATS / 256, UPW = U_UNITS / 4;
+    const int a_voff = ((lane / (MF / 4)) * p.Mp + m0 + 4 * (lane % (MF / 4))) * 4;
+
+    auto load_step = [&](int step, lds_float *us, lds_float *rs, bool checked) {
+#pragma unroll
+        for (int j = 0; j < UPW; j++) {
+            const int u = wave + 4 * j;
+            lds_dma_b128(dma_w, us + u * 256, a_voff, (step * (CK * 16) + u * RPI) * p.Mp * 4);
+        }
+#pragma unroll
+        for (int jc = 0; jc < CK / 4; jc++) {
+            const int cl = wave + 4 * jc, c = step * CK + cl;
+            const bool cok = !checked || c < p.C;
+            const bool second = c >= p.Csplit;  // uniform in the wavefront: the channel comes from the second tensor
+            const int soff = (cok ? (second ? c - p.Csplit : c) : 0) * HW4;
+#pragma unroll
+            for (int k = 0; k < WLC; k++)
+                if (k < nload) lds_dma_b32(second ? dma_in2 : dma_in, rs + cl * SLOTS + k * 64, cok ? voff[k] : OOB, soff);
+        }
+    };
+
+    floatx16 acc[4][FM][FN];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+            for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[j][fm][fn][v] = 0.0f;
+
+    // position row i = wave: patch rows ra and rb, combined as d[ra] + d[rb] (i = 1) or d[ra] - d[rb]
+    const int ra = wave == 0 ? 0 : (wave == 2 ? 2 : 1), rb = wave == 0 ? 2 : (wave == 1 ? 2 : (wave == 2 ? 1 : 3));
+    const unsigned sgn = wave == 1 ? 0u : 0x80000000u;
+    const int a_off = (half * 16 + 4 * wave) * MF + l32;
+    int ra_off[FN], rb_off[FN];  // this lane's two patch rows, as LDS offsets within a step's pixels (channel `half` of a pair)
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) {
+        ra_off[fn] = half * SLOTS + my_base[fn] + ra * my_stride[fn];
+        rb_off[fn] = half * SLOTS + my_base[fn] + rb * my_stride[fn];
+    }
+
+    // The K loop, software-pipelined over channel pairs and across K-steps: the operands of the pair after the current one
+    // are read from LDS, and its B operands derived, while the matrix instructions of the current pair are issued (a
+    // matrix instruction occupies its pipe for 64 cycles; the reads go first - their results are needed soonest).  Per
+    // pair: 2 FM + 4 FN two-address LDS reads, 12 FN vector instructions, 4 FM FN matrix instructions.  The first pair of
+    // a step is read right after the barrier that publishes the step's buffer, in front of the second half of the last
+    // pair's matrix instructions of the step before.
+    static_assert((CK / 2) % 2 == 0, "the first pair of a step always lands in operand set 0");
+    float a[2][4][FM], d[2][4][FN], vv[2][4][FN];
+    auto read_pair = [&](const lds_float *__restrict__ us, const lds_float *__restrict__ rs, int cp, int into) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int fm = 0; fm < FM; fm++) a[into][j][fm] = us[a_off + cp * (32 * MF) + j * MF + fm * 32];
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) {  // (a patch starts at an even slot: 8-byte reads)
+            typedef float floatx2 __attribute__((ext_vector_type(2)));
+            typedef const __attribute__((address_space(3))) floatx2 *lds_f2;
+            const floatx2 a0 = *(lds_f2)(rs + ra_off[fn] + cp * (2 * SLOTS)), a1 = *(lds_f2)(rs + ra_off[fn] + cp * (2 * SLOTS) + 2);
+            const floatx2 b0 = *(lds_f2)(rs + rb_off[fn] + cp * (2 * SLOTS)), b1 = *(lds_f2)(rs + rb_off[fn] + cp * (2 * SLOTS) + 2);
+            d[0][0][fn] = a0.x, d[0][1][fn] = a0.y, d[0][2][fn] = a1.x, d[0][3][fn] = a1.y;
+            d[1][0][fn] = b0.x, d[1][1][fn] = b0.y, d[1][2][fn] = b1.x, d[1][3][fn] = b1.y;
+        }
+    };
+    auto transform = [&](int into) __attribute__((always_inline)) {
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) {
+            float u[4];
+#pragma unroll
+            for (int s = 0; s < 4; s++) u[s] = __fadd_rn(d[0][s][fn], __builtin_bit_cast(float, __builtin_bit_cast(unsigned, d[1][s][fn]) ^ sgn));
+            vv[into][0][fn] = __fsub_rn(u[0], u[2]);
+            vv[into][1][fn] = __fadd_rn(u[1], u[2]);
+            vv[into][2][fn] = __fsub_rn(u[2], u[1]);
+            vv[into][3][fn] = __fsub_rn(u[1], u[3]);
+        }
+    };
+    auto mfmas = [&](int cur, int j_lo, int j_hi) __attribute__((always_inline)) {  // positions j_lo .. j_hi - 1 of the row
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+                for (int fn = 0; fn < FN; fn++)
+                    if (j >= j_lo && j < j_hi)
+                        acc[j][fm][fn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][j][fm], vv[cur][j][fn], acc[j][fm][fn], 0, 0, 0);
+    };
+    constexpr int NDS = 2 * FM + 2 * FN, NVALU = 12 * FN, NMFMA = 4 * FM * FN;
+
+    auto us_of = [&](int buf) { return (lds_float *)&lds[buf * BUF_FLOATS]; };
+    auto rs_of = [&](int buf) { return (lds_float *)&lds[buf * BUF_FLOATS + U_FLOATS]; };
+    const int nsteps = p.nsteps, full_steps = p.C / CK;
+    constexpr int WAIT_ALL = 0x0F70;  // vmcnt(0): this wavefront's LDS-direct loads have landed
+    load_step(0, us_of(0), rs_of(0), full_steps < 1);
+    __builtin_amdgcn_s_waitcnt(WAIT_ALL);
+    __syncthreads();
+    trace_mark(p, 1);
+    read_pair(us_of(0), rs_of(0), 0, 0);
+    transform(0);
+    for (int step = 0; step < nsteps; step++) {
+        const int cur = step & 1, nxt = cur ^ 1;
+        if (step + 1 < nsteps) load_step(step + 1, us_of(nxt), rs_of(nxt), step + 1 >= full_steps);
+        const lds_float *us = us_of(cur), *rs = rs_of(cur);
+#pragma unroll
+        for (int cp = 0; cp + 1 < CK / 2; cp++) {
+            const int set = cp & 1;
+            read_pair(us, rs, cp + 1, set ^ 1);
+            transform(set ^ 1);
+            mfmas(set, 0, 4);
+            wino_sched_pair<NDS, NVALU, NMFMA / 2, NMFMA - NMFMA / 2, 0>();
+        }
+        // the last pair of the step: its matrix instructions straddle the barrier and the reads of the next step's first
+        // pair (after the last step these reads fetch the other buffer's stale contents, which nothing uses)
+        mfmas(1, 0, 2);
+        __builtin_amdgcn_sched_barrier(0);  // (nothing moves across: the wait comes after the first half's matrix instructions)
+        __builtin_amdgcn_s_waitcnt(WAIT_ALL);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        read_pair(us_of(nxt), rs_of(nxt), 0, 0);
+        mfmas(1, 2, 4);
+        transform(0);
+        __builtin_amdgcn_sched_group_barrier(0x100, NDS, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, NMFMA / 2, 0);
+    }
+    trace_mark(p, 2);
+
+    // ---- output transform: along the position row in registers, across the rows through LDS, then the epilogue
+    const size_t plane = (size_t)p.wP * p.wQ;
+    const bool pair = (p.wQ % 2 == 0) && (((size_t)p.O | (size_t)(p.residual ? p.residual : p.O)) % 8 == 0);
+    float *xch = &lds[0];
+#pragma unroll
+    for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+        for (int fn = 0; fn < FN; fn++) {
+            if (fm + fn > 0) __syncthreads();  // the reads of the block before are done
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const float s0 = __fadd_rn(__fadd_rn(acc[0][fm][fn][v], acc[1][fm][fn][v]), acc[2][fm][fn][v]);
+                const float s1 = __fsub_rn(__fsub_rn(acc[1][fm][fn][v], acc[2][fm][fn][v]), acc[3][fm][fn][v]);
+                xch[((wave * 2 + 0) * 16 + v) * 64 + lane] = s0;
+                xch[((wave * 2 + 1) * 16 + v) * 64 + lane] = s1;
+            }
+            __syncthreads();
+            const int n = n0 + fn * 32 + l32;
+            if (n < p.wT) {
+                const int img = n / per_img, r = n - img * per_img, ty = r / p.wtw, tx = r - ty * p.wtw;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    float y[2][2];
+#pragma unroll
+                    for (int b = 0; b < 2; b++) {
+                        float t[4];
+#pragma unroll
+                        for (int i = 0; i < 4; i++) t[i] = xch[((i * 2 + b) * 16 + 4 * wave + k) * 64 + lane];
+                        y[0][b] = __fadd_rn(__fadd_rn(t[0], t[1]), t[2]);
+                        y[1][b] = __fsub_rn(__fsub_rn(t[1], t[2]), t[3]);
+                    }
+                    wino_store_row<MF>(p, epi, m0, fm * 32 + 8 * wave + 4 * half + k, img, ty, tx, plane, pair, y[0][0], y[0][1], y[1][0], y[1][1]);
+                }
+            }
+        }
+    if (p.trace != nullptr) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        trace_mark(p, 3);
+    }
+}
+
 // ---------------------------------------------------------------- host side
 int g_algo = 0;
 // Measurement: while collecting, every launch of a convolution kernel (not the filter repack, not
@@ -1625,6 +1910,17 @@ const Variant k2x2[2][4] = {
     {TAP(2, 2, 2, 2, 2, 2, 4, true), TAP(1, 4, 2, 1, 2, 2, 4, true), TAP(2, 2, 1, 1, 2, 2, 4, true), TAP(1, 4, 1, 1, 2, 2, 4, true)}};
 const Variant kgen[2][4] = {{GEN(2, 2, 2, 2, false), GEN(1, 4, 2, 1, false), GEN(2, 2, 1, 1, false), GEN(1, 4, 1, 1, false)},
                             {GEN(2, 2, 2, 2, true), GEN(1, 4, 2, 1, true), GEN(2, 2, 1, 1, true), GEN(1, 4, 1, 1, true)}};
+
+// The one-launch Winograd form's tile shapes: 32 FM filters x 32 FN blocks, CK channels per K-step.
+struct FusedVariant {
+    const char *name;
+    int fm, fn, ck;
+    void (*kernel)(const ConvParams);
+};
+#define FUSED(FM, FN, CK, WPE) {"wino_fused_kernel<" #FM "," #FN "," #CK "," #WPE ">", FM, FN, CK, wino_fused_kernel<FM, FN, CK, WPE>}
+const FusedVariant kfused[] = {FUSED(1, 1, 4, 4), FUSED(2, 1, 4, 3)};
+constexpr int NUM_FUSED = (int)(sizeof(kfused) / sizeof(kfused[0]));
+constexpr int FUSED_ROW_ALIGN = 8;  // the transformed filters are padded to whole K-steps of every variant
 
 // Launch plan: tile shape and, for the tiles that do not divide evenly over the CUs, the number
 // of K slices.  The MFMA pipe of a CU is shared by its resident workgroups, so a launch takes as
@@ -1736,6 +2032,8 @@ struct CachedFilters {
     float *Wp;
     float *Wwino;  // 3x3 (2x2) filters: the 16 (9) transformed matrices of the Winograd form [16][wino_rows][Mp], made on first use
     int wino_rows;
+    float *Wfused;  // 3x3 filters: the transformed filters of the one-launch Winograd form [fused_rows][16][Mp], made on first use
+    int fused_rows;
     bool stale;  // K was written through this library since the last repack
 };
 std::mutex g_cache_mutex;
@@ -1757,8 +2055,13 @@ int repack(int dev, CachedFilters &e) {
     EH_CHECK_LAUNCH();
     if (e.Wwino != nullptr) {
         const dim3 grid((unsigned)(((size_t)e.wino_rows * e.Mp + 255) / 256));
-        if (e.R == 3) hipLaunchKernelGGL(wino_filter_kernel<4>, grid, dim3(256), 0, state(dev).stream, e.K, e.Wwino, e.Kf, e.C, e.Mp, e.wino_rows);
-        else hipLaunchKernelGGL(wino_filter_kernel<3>, grid, dim3(256), 0, state(dev).stream, e.K, e.Wwino, e.Kf, e.C, e.Mp, e.wino_rows);
+        if (e.R == 3) hipLaunchKernelGGL(wino_filter_kernel<4>, grid, dim3(256), 0, state(dev).stream, e.K, e.Wwino, e.Kf, e.C, e.Mp, e.wino_rows, 0);
+        else hipLaunchKernelGGL(wino_filter_kernel<3>, grid, dim3(256), 0, state(dev).stream, e.K, e.Wwino, e.Kf, e.C, e.Mp, e.wino_rows, 0);
+        EH_CHECK_LAUNCH();
+    }
+    if (e.Wfused != nullptr) {
+        const dim3 grid((unsigned)(((size_t)e.fused_rows * e.Mp + 255) / 256));
+        hipLaunchKernelGGL(wino_filter_kernel<4>, grid, dim3(256), 0, state(dev).stream, e.K, e.Wfused, e.Kf, e.C, e.Mp, e.fused_rows, 1);
         EH_CHECK_LAUNCH();
     }
     e.stale = false;
@@ -1803,6 +2106,7 @@ void conv_filters_released(int dev, const void *base, size_t bytes) {
             (void)hipStreamSynchronize(state(dev).stream);
             (void)hipFree(c[i].Wp);
             if (c[i].Wwino) (void)hipFree(c[i].Wwino);
+            if (c[i].Wfused) (void)hipFree(c[i].Wfused);
             c[i] = c.back();
             c.pop_back();
         } else {
@@ -1835,6 +2139,8 @@ int eddlhip_conv2d_cache_filters(int dev, const float *K, int Kf, int C, int R, 
     e.Wp = nullptr;
     e.Wwino = nullptr;
     e.wino_rows = 0;
+    e.Wfused = nullptr;
+    e.fused_rows = 0;
     e.stale = true;
     EH_REQUIRE((size_t)e.rows * e.Mp * sizeof(float) < ((size_t)1 << 31),
                "conv2d_cache_filters: the repacked filter matrix (%d taps x %d channels) exceeds the 2 GiB a buffer descriptor covers", e.rows, e.Mp);
@@ -1860,6 +2166,7 @@ int eddlhip_conv2d_uncache_filters(int dev, const float *K) {
             synced = true;
             EH_TRY_HIP(hipFree(c[i].Wp));
             if (c[i].Wwino) EH_TRY_HIP(hipFree(c[i].Wwino));
+            if (c[i].Wfused) EH_TRY_HIP(hipFree(c[i].Wfused));
             c[i] = c.back();
             c.pop_back();
         } else {
@@ -1870,7 +2177,7 @@ int eddlhip_conv2d_uncache_filters(int dev, const float *K) {
 }
 
 int eddlhip_conv2d_force_plan(int tile, int slices) {
-    EH_REQUIRE(tile >= -1 && tile <= 5, "conv2d_force_plan: tile is -1 (automatic), 0..3, or 4 / 5 (the Winograd forms where they apply)");
+    EH_REQUIRE(tile >= -1 && tile <= 6, "conv2d_force_plan: tile is -1 (automatic), 0..3, or 4 / 5 / 6 (the Winograd forms where they apply)");
     g_force_tile = tile;
     g_force_slices = slices;
     return 0;
@@ -1917,7 +2224,7 @@ int eddlhip_conv2d_tuned_load(int dev, const char *host_path) {
         int *k = t.key;
         const int got = sscanf(line, "%d %d %d %d %d %d %d %d %d %d | %d %d", k, k + 1, k + 2, k + 3, k + 4, k + 5, k + 6, k + 7, k + 8, k + 9, &t.tile,
                                &t.slices);
-        if (got != 12 || t.tile < -1 || t.tile > 5 || t.slices < 1 || t.slices > 64) {
+        if (got != 12 || t.tile < -1 || t.tile > 6 || t.slices < 1 || t.slices > (t.tile == 6 ? NUM_FUSED : 16)) {
             bad = true;
             break;
         }
@@ -2011,6 +2318,10 @@ constexpr size_t WINO_INNER_RESERVE = (size_t)16 * 255 * 128 * 128 * sizeof(floa
 int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
                     int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
                     const float *bn_var, float bn_eps, const float *residual, int relu);
+
+int conv2d_winograd_fused(int variant, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
+                          int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
+                          const float *bn_var, float bn_eps, const float *residual, int relu);
 
 // Whether the Winograd form can run this convolution: 3x3, stride 1, and the product launch within the limits of
 // conv2d_fwd_impl (one "image" of transformed input or output below 1 GiB, fewer than 2^31 blocks).
@@ -2156,6 +2467,13 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     // fixed scratch array, whose size it exceeds, and not for the scalar-order or register-staged algorithm switches
     const bool wino_ok = !gemm && !no_alloc && g_algo == 0 && !g_wino_never && winograd_applies(N, C, Kf, R, S, sr, sc, P, Q);
     const bool fold_ok = wino_ok && winograd_fold_applies(N, C, Kf, R, S, sr, sc, P, Q);
+    // the one-launch form (3x3 filters only) needs no transformed copy of the input, so none of V's limits apply
+    const bool fused_ok = !gemm && !no_alloc && g_algo == 0 && !g_wino_never && R == 3 && S == 3 && sr == 1 && sc == 1 &&
+                          (long long)C * 16 * p.Mp * 4 < (1LL << 31);
+    if (fused_ok && g_force_tile == 6)
+        return conv2d_winograd_fused(g_force_slices < 1 ? 0 : (g_force_slices > NUM_FUSED ? NUM_FUSED - 1 : g_force_slices - 1), dev, I,
+                                     two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean, bn_var,
+                                     bn_eps, residual, relu);
     if ((wino_ok && (g_force_tile == 4 || (g_wino && g_force_tile < 0 && !g_tuning))) || (fold_ok && g_force_tile == 5))
         return conv2d_winograd(g_force_tile == 5, R, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b,
                                bn_mean, bn_var, bn_eps, residual, relu);
@@ -2237,6 +2555,15 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
                     best.slices = 1;
                 }
             }
+            if (rc == 0 && fused_ok) {
+                float ms = 0.0f;
+                for (int fv = 0; fv < NUM_FUSED; fv++)
+                    if (measure(6, fv + 1, &ms) == 0 && ms < best_ms && ms < 0.98f * planned_ms) {
+                        best_ms = ms;
+                        best.tile = 6;
+                        best.slices = fv + 1;
+                    }
+            }
             g_tuning = false;
             g_pool_req = pool_req;
             (void)hipEventDestroy(e0);
@@ -2251,6 +2578,9 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
         if (found != nullptr && ((found->tile == 4 && wino_ok) || (found->tile == 5 && fold_ok)))
             return conv2d_winograd(found->tile == 5, R, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g,
                                    bn_b, bn_mean, bn_var, bn_eps, residual, relu);
+        if (found != nullptr && found->tile == 6 && fused_ok)
+            return conv2d_winograd_fused(found->slices - 1, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g,
+                                         bn_b, bn_mean, bn_var, bn_eps, residual, relu);
         if (found != nullptr && found->tile >= 0 && found->tile < 4)
             plan = forced_plan(family, found->tile, found->slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
     }
@@ -2399,8 +2729,8 @@ int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2,
     float *Uw = (float *)base, *V = (float *)(base + u_bytes), *M = (float *)(base + u_bytes + v_bytes);
     if (U == nullptr) {
         const dim3 grid((unsigned)(((size_t)rows * Mp + 255) / 256));
-        if (ps == 4) hipLaunchKernelGGL(wino_filter_kernel<4>, grid, dim3(256), 0, st, K, Uw, Kf, C, Mp, rows);
-        else hipLaunchKernelGGL(wino_filter_kernel<3>, grid, dim3(256), 0, st, K, Uw, Kf, C, Mp, rows);
+        if (ps == 4) hipLaunchKernelGGL(wino_filter_kernel<4>, grid, dim3(256), 0, st, K, Uw, Kf, C, Mp, rows, 0);
+        else hipLaunchKernelGGL(wino_filter_kernel<3>, grid, dim3(256), 0, st, K, Uw, Kf, C, Mp, rows, 0);
         EH_CHECK_LAUNCH();
         U = Uw;
     }
@@ -2513,6 +2843,100 @@ int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2,
     char inner[sizeof(g_last_kernel)];
     snprintf(inner, sizeof(inner), "%s", g_last_kernel);
     snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%.100s, %d blocks]", inner, Tp);
+    return 0;
+}
+
+// The one-launch Winograd form of a 3x3 stride-1 convolution (wino_fused_kernel).  Workspace: the transformed filters,
+// unless a registered filter tensor keeps them.
+int conv2d_winograd_fused(int variant, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
+                          int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
+                          const float *bn_var, float bn_eps, const float *residual, int relu) {
+    hipStream_t st = state(dev).stream;
+    const FusedVariant &fv = kfused[variant];
+    // a max-pool asked for with this convolution is taken into the epilogue where every 2x2 block of outputs is whole
+    PoolRequest *const pool = (g_pool_req != nullptr && !g_tuning && P % 2 == 0 && Q % 2 == 0) ? g_pool_req : nullptr;
+    if (pool != nullptr) pool->done = true;
+    const int th = (P + 1) / 2, tw = (Q + 1) / 2;
+    const int rows = (C + FUSED_ROW_ALIGN - 1) / FUSED_ROW_ALIGN * FUSED_ROW_ALIGN, Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
+    const size_t u_floats = (size_t)16 * rows * Mp;
+    EH_REQUIRE(u_floats * sizeof(float) < ((size_t)1 << 31), "conv2d: the transformed filters (16 x %d x %d) exceed 2 GiB", rows, Mp);
+
+    const float *U = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_cache_mutex);
+        for (CachedFilters &e : g_cache[dev]) {
+            if (e.K == K && e.Kf == Kf && e.C == C && e.R == 3 && e.S == 3) {
+                if (e.Wfused == nullptr && !state(dev).capturing) {
+                    if (hipMalloc((void **)&e.Wfused, u_floats * sizeof(float)) != hipSuccess) {
+                        e.Wfused = nullptr;
+                        (void)hipGetLastError();
+                        break;  // no room to keep them: transform per call
+                    }
+                    e.fused_rows = rows;
+                    e.stale = true;
+                }
+                if (e.Wfused != nullptr) {
+                    if (e.stale) EH_TRY(repack(dev, e));
+                    U = e.Wfused;
+                }
+                break;
+            }
+        }
+    }
+    if (U == nullptr) {
+        void *ws = nullptr;
+        EH_TRY(get_workspace(dev, u_floats * sizeof(float), &ws));
+        const dim3 grid((unsigned)(((size_t)rows * Mp + 255) / 256));
+        hipLaunchKernelGGL(wino_filter_kernel<4>, grid, dim3(256), 0, st, K, (float *)ws, Kf, C, Mp, rows, 1);
+        EH_CHECK_LAUNCH();
+        U = (const float *)ws;
+    }
+
+    ConvParams q;
+    memset(&q, 0, sizeof(q));
+    const int Cimg = I2 ? C / 2 : C;
+    q.Csplit = I2 ? C / 2 : C; q.Cimg = Cimg; q.uh = uh; q.uw = uw;
+    q.Wp = U; q.K = K;
+    q.bias = bias; q.bn_g = bn_g; q.bn_b = bn_b; q.bn_mean = bn_mean; q.bn_var = bn_var;
+    q.bn_eps = bn_eps; q.relu = relu;
+    q.C = C; q.H = H; q.W = W; q.Kf = Kf; q.R = 3; q.S = 3; q.sr = 1; q.sc = 1; q.pt = pad_top; q.pl = pad_left; q.P = P; q.Q = Q;
+    q.CRS = C * 9; q.Mp = Mp; q.PQ = P * Q;
+    q.nsteps = (C + fv.ck - 1) / fv.ck;
+    q.slice_steps = q.nsteps; q.nslices = 1;
+    q.wp_bytes = (unsigned)(u_floats * sizeof(float));
+    q.wth = th; q.wtw = tw; q.wP = P; q.wQ = Q; q.wps = 4;
+    q.gm = (Kf + 32 * fv.fm - 1) / (32 * fv.fm);
+    // a launch covers one batch chunk: input within the 2 GiB a buffer descriptor addresses, fewer than 2^31 blocks
+    const long long img_elems = (long long)Cimg * H * W, per_img = (long long)th * tw;
+    long long max_imgs = (1LL << 29) / img_elems;
+    if (max_imgs > 0x3ffffe00LL / per_img) max_imgs = 0x3ffffe00LL / per_img;
+    EH_REQUIRE(max_imgs >= 1, "conv2d: one image of %lld elements is too large for the Winograd form", img_elems);
+    const int chunk_imgs = (int)((N < max_imgs) ? N : max_imgs);
+    for (long long b0 = 0; b0 < N; b0 += chunk_imgs) {
+        const int nb = (int)((N - b0 < chunk_imgs) ? N - b0 : chunk_imgs);
+        q.N = nb;
+        q.I = I + (size_t)b0 * img_elems;
+        q.I2 = (I2 ? I2 : I) + (size_t)b0 * img_elems;
+        q.O = O + (size_t)b0 * Kf * q.PQ;
+        q.residual = residual ? residual + (size_t)b0 * Kf * q.PQ : nullptr;
+        q.in_bytes = (unsigned)((size_t)nb * img_elems * sizeof(float));
+        q.wT = (int)(nb * per_img);
+        q.npix = q.wT;
+        q.gn = (q.wT + 32 * fv.fn - 1) / (32 * fv.fn);
+        EH_REQUIRE((long long)q.gm * q.gn <= 0x3fffffffLL, "conv2d: too many tiles");
+        q.main_tiles = q.gm * q.gn;
+        if (pool != nullptr) {
+            const size_t po = (size_t)b0 * Kf * per_img;
+            q.pool_O = pool->O + po; q.pool_ix = pool->ix + po; q.pool_iy = pool->iy + po;
+            if (!pool->keep) q.O = nullptr;
+        }
+        q.trace = (g_trace != nullptr && q.main_tiles <= g_trace_wgs) ? g_trace : nullptr;
+        EH_TRY(prof_begin(st));
+        hipLaunchKernelGGL(fv.kernel, dim3((unsigned)q.main_tiles), dim3(256), 0, st, q);
+        EH_CHECK_LAUNCH();
+        EH_TRY(prof_end(st));
+    }
+    snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%s, %lld blocks]", fv.name, (long long)N * per_img);
     return 0;
 }
 

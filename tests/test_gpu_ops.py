@@ -361,13 +361,19 @@ WINOGRAD_CASES = [
 ]
 
 
-@pytest.mark.parametrize("form", [4, 5], ids=["three-kernels", "folded"])
+WINOGRAD_FORMS = [(4, 1), (5, 1), (6, 1), (6, 2)]
+WINOGRAD_FORM_IDS = ["three-kernels", "folded", "one-launch-32x32", "one-launch-64x32"]
+
+
+@pytest.mark.parametrize("form", WINOGRAD_FORMS, ids=WINOGRAD_FORM_IDS)
 @pytest.mark.parametrize("case", WINOGRAD_CASES, ids=lambda c: "x".join(str(v) for v in c[:5]))
 def test_conv2d_winograd_form_against_oracle(hip, oracle, case, form):
     """The Winograd forms (force_conv_plan(4, .): transforms and products as separate launches; 5: the output transform
-    folded into the one product launch, for channel counts that are whole K-steps) against the CPU oracle's direct
-    convolution of the same logical input (concatenated / resized / zero-padded on the host), to the convolution
-    tolerance; the epilogue after it is the oracle's, step by step."""
+    folded into the one product launch, for channel counts that are whole K-steps; (6, v): everything in one launch that
+    reads the input itself, tile shape v) against the CPU oracle's direct convolution of the same logical input
+    (concatenated / resized / zero-padded on the host), to the convolution tolerance; the epilogue after it is the
+    oracle's, step by step."""
+    form, variant = form
     N, C, H, W, Kf, (pt, pl), out, use_bias, use_bn, use_res, relu, two, up = case
     rng = np.random.default_rng(77)
     Ci = C // 2 if two else C
@@ -396,15 +402,15 @@ def test_conv2d_winograd_form_against_oracle(hip, oracle, case, form):
         ref = oracle.relu(ref)
     O = hip.full((N, Kf, P, Q), 3.0)
     dbn = (hip.array(bn[0]), hip.array(bn[1]), hip.array(bn[2]), hip.array(bn[3]), bn[4]) if bn else None
-    hip.force_conv_plan(form, 1)
+    hip.force_conv_plan(form, variant)
     try:
         hip.conv2D(hip.array(a), hip.array(w), hip.array(bias) if use_bias else None, O, 1, 1, pt, pl, bn=dbn,
                    residual=hip.array(res) if use_res else None, relu=relu, second=hip.array(b) if two else None, upsample=up)
         name = hip.last_conv_kernel()
     finally:
         hip.force_conv_plan(-1, 1)
-    if form == 4 or C % 16 == 0:
-        assert name.startswith("winograd[") and ("true,true>" in name) == (form == 5), name
+    if form != 5 or C % 16 == 0:
+        assert name.startswith("winograd[") and ("true,true>" in name) == (form == 5) and ("wino_fused_kernel" in name) == (form == 6), name
     else:
         assert not name.startswith("winograd["), name       # the folded form needs whole K-steps of channels: the direct form ran
     assert_conv_close(ref, O.numpy(), "winograd %s" % (case,))
@@ -484,7 +490,7 @@ def test_conv2d_winograd_form_only_where_it_applies_and_with_kept_filters(hip, o
         hip.set_conv_algo("auto")
 
 
-@pytest.mark.parametrize("form", [-1, 4, 5])
+@pytest.mark.parametrize("form", [-1, 4, 5, 6, 8])
 @pytest.mark.parametrize("case", ["bias+relu", "bn+residual+relu", "2x2 filter", "two tensors", "upsampled", "nan window"])
 def test_conv2d_fwd_maxpool_is_the_convolution_followed_by_the_pool(hip, form, case):
     """eddlhip_conv2d_fwd_maxpool against eddlhip_conv2d_fwd* + eddlhip_maxpool2d(2, 2, 2, 2) under the same launch plan
@@ -521,11 +527,14 @@ def test_conv2d_fwd_maxpool_is_the_convolution_followed_by_the_pool(hip, form, c
     O1, O2 = hip.full((N, Kf, P, Q), 3.0), hip.full((N, Kf, P, Q), 4.0)
     pooled = lambda: (hip.full((N, Kf, P // 2, Q // 2), 9.0), hip.full((N, Kf, P // 2, Q // 2), 7.0), hip.full((N, Kf, P // 2, Q // 2), 7.0))
     A, B, K2 = pooled(), pooled(), pooled()
+    variant = 1
+    if form == 8:                                      # the one-launch form on its 64-filter tile
+        form, variant = 6, 2
     try:
-        hip.force_conv_plan(form, 1)
+        hip.force_conv_plan(form, variant)
         hip.conv2D(X, w, bias, O1, 1, 1, pad, pad, bn=bn, residual=res, relu=relu, second=second, upsample=upsample)
         name = hip.last_conv_kernel()
-        assert name.startswith("winograd") == (form >= 4), name
+        assert name.startswith("winograd") == (form >= 4 and not (form == 6 and fs == 2)), name   # (the one-launch form: 3x3 filters only)
         hip.mpool2D(O1, A[0], A[1], A[2], (2, 2), (2, 2), (0, 0, 0, 0))
         hip.conv2D(X, w, bias, O2, 1, 1, pad, pad, bn=bn, residual=res, relu=relu, second=second, upsample=upsample, pool=B, keep=True)
         assert hip.last_conv_kernel() == name
