@@ -198,6 +198,7 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, pl
         hip.conv_autotune(True)
         model.run()
         hip.synchronize()
+        hip.workspace_trim()   # the search's candidates took more workspace than the plans it kept
         if plans:
             hip.conv_tuned_save(plans)
     step = model.run

@@ -30,6 +30,7 @@ PROTOTYPES = {
     "eddlhip_memcpy_d2d": [c_int, P, P, c_size_t],
     "eddlhip_fill": [c_int, P, c_size_t, c_float],
     "eddlhip_workspace_bytes": [c_int, ctypes.POINTER(c_size_t)],
+    "eddlhip_workspace_trim": [c_int],
     "eddlhip_event_create": [c_int, ctypes.POINTER(c_void_p)],
     "eddlhip_event_destroy": [c_int, c_void_p],
     "eddlhip_event_record": [c_int, c_void_p],

@@ -169,6 +169,10 @@ class Backend:
         self._check(self.lib.eddlhip_workspace_bytes(self.dev, ctypes.byref(n)))
         return n.value
 
+    def workspace_trim(self):
+        """Releases the library's workspace; it grows back to what the calls from now on need (after a plan search)."""
+        self._check(self.lib.eddlhip_workspace_trim(self.dev))
+
     def record(self, fn):
         """Records the launches ``fn()`` makes into a Graph instead of running them.  ``fn`` must have
         run once before (workspace at its final size) and may only launch kernels."""

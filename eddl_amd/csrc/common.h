@@ -29,6 +29,8 @@ struct DeviceState {
 
 DeviceState &state(int dev);
 int set_error(int code, const char *fmt, ...);
+// Empties the calling thread's error text (after a failure that was handled inside the library).
+void clear_error();
 // Makes `dev` current and initialises it on first use.
 int use_device(int dev);
 // Returns a workspace of at least `bytes` (contents undefined); waits for the stream before

@@ -524,20 +524,19 @@ __device__ __forceinline__ void wino_fold(floatx16 (&y)[2][2], floatx16 &acc, in
 
 // One filter row's four outputs of one 2x2 block (y00 y01 / y10 y11 at rows 2 ty, 2 ty + 1 and columns 2 tx, 2 tx + 1 of
 // image `img`): the convolution's epilogue value by value (the arithmetic of apply_epilogue), two outputs of a row per
-// store where the rows are aligned for it (`pair`), and the block's max-pool where one is asked for.  `epi`: the tile's
-// channel constants (stage_channel_constants), ml: the row within the tile.
-template <int BM>
-__device__ __forceinline__ void wino_store_row(const ConvParams &p, const float *epi, int m0, int ml, int img, int ty, int tx, size_t plane, bool pair,
+// store where the rows are aligned for it (`pair`), and the block's max-pool where one is asked for.  `e`: the channel
+// constants of filter m.
+__device__ __forceinline__ void wino_store_row(const ConvParams &p, const ChannelEpilogue &e, int m, int img, int ty, int tx, size_t plane, bool pair,
                                                float y00, float y01, float y10, float y11) {
-    if (m0 + ml >= p.Kf) return;
-    const float bias = epi[ml], mean = epi[BM + ml], sd = epi[2 * BM + ml], g = epi[3 * BM + ml], b = epi[4 * BM + ml];
+    if (m >= p.Kf) return;
+    const float bias = e.bias, mean = e.mean, sd = e.sd, g = e.g, b = e.b;
     const float yy[2][2] = {{y00, y01}, {y10, y11}};
     float fin[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
 #pragma unroll
     for (int a = 0; a < 2; a++) {
         const int oy = 2 * ty + a, ox = 2 * tx;
         if (oy >= p.wP) continue;
-        const size_t oidx = ((size_t)img * p.Kf + (size_t)(m0 + ml)) * plane + (size_t)oy * p.wQ + ox;
+        const size_t oidx = ((size_t)img * p.Kf + (size_t)m) * plane + (size_t)oy * p.wQ + ox;
         float x0 = yy[a][0], x1 = yy[a][1];
         float r0 = 0.0f, r1 = 0.0f;
         if (p.residual) {
@@ -568,7 +567,15 @@ __device__ __forceinline__ void wino_store_row(const ConvParams &p, const float 
         }
     }
     if (p.pool_O != nullptr)  // (even wP, wQ: both rows and both columns of the block exist)
-        pool_block(p, (((size_t)img * p.Kf + (size_t)(m0 + ml)) * p.wth + ty) * p.wtw + tx, ty, tx, fin[0][0], fin[0][1], fin[1][0], fin[1][1]);
+        pool_block(p, (((size_t)img * p.Kf + (size_t)m) * p.wth + ty) * p.wtw + tx, ty, tx, fin[0][0], fin[0][1], fin[1][0], fin[1][1]);
+}
+
+// the constants of row ml of a tile as stage_channel_constants laid them out in LDS
+template <int BM>
+__device__ __forceinline__ ChannelEpilogue channel_from_lds(const float *epi, int ml) {
+    ChannelEpilogue e;
+    e.bias = epi[ml], e.mean = epi[BM + ml], e.sd = epi[2 * BM + ml], e.g = epi[3 * BM + ml], e.b = epi[4 * BM + ml];
+    return e;
 }
 
 // A wavefront's 32 filters x 32 blocks: lane = block (column) lane % 32, filter rows 8 * (v / 4) + 4 * (lane / 32) + v % 4.
@@ -585,7 +592,7 @@ __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&
 #pragma unroll
     for (int v = 0; v < 16; v++) {
         const int ml = m_local + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-        wino_store_row<BM>(p, epi, m0, ml, img, ty, tx, plane, pair, y[0][0][v], y[0][1][v], y[1][0][v], y[1][1][v]);
+        wino_store_row(p, channel_from_lds<BM>(epi, ml), m0 + ml, img, ty, tx, plane, pair, y[0][0][v], y[0][1][v], y[1][0][v], y[1][1][v]);
     }
 }
 
@@ -1614,7 +1621,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
     trace_mark(p, 0);
     tile_of_block(p, m_tile, n_tile, local_tile, slice, split);
     const int m0 = m_tile * MF, n0 = n_tile * NB;
-    put_channel_constants<MF>(epi, fetch_channel_constants<MF>(p, m0, tid), tid);  // (published by the loop's first barrier)
+    // a tile the launch plan divides along the channels: this workgroup sums steps step_lo .. step_hi - 1 only
+    const int step_lo = split ? slice * p.slice_steps : 0;
+    const int step_hi = split ? min(step_lo + p.slice_steps, p.nsteps) : p.nsteps;
+    if (!split) put_channel_constants<MF>(epi, fetch_channel_constants<MF>(p, m0, tid), tid);  // (published by the loop's first barrier)
 
     // ---- where the tile's pixels go in LDS, and where this lane's patches lie there.  The tile's blocks are a run of
     // consecutive blocks, i.e. a few SEGMENTS of block rows (a segment: cnt neighbouring blocks of one row of blocks of one
@@ -1755,17 +1765,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 
     auto us_of = [&](int buf) { return (lds_float *)&lds[buf * BUF_FLOATS]; };
     auto rs_of = [&](int buf) { return (lds_float *)&lds[buf * BUF_FLOATS + U_FLOATS]; };
-    const int nsteps = p.nsteps, full_steps = p.C / CK;
+    const int full_steps = p.C / CK;
     constexpr int WAIT_ALL = 0x0F70;  // vmcnt(0): this wavefront's LDS-direct loads have landed
-    load_step(0, us_of(0), rs_of(0), full_steps < 1);
+    load_step(step_lo, us_of(0), rs_of(0), step_lo >= full_steps);
     __builtin_amdgcn_s_waitcnt(WAIT_ALL);
     __syncthreads();
     trace_mark(p, 1);
     read_pair(us_of(0), rs_of(0), 0, 0);
     transform(0);
-    for (int step = 0; step < nsteps; step++) {
-        const int cur = step & 1, nxt = cur ^ 1;
-        if (step + 1 < nsteps) load_step(step + 1, us_of(nxt), rs_of(nxt), step + 1 >= full_steps);
+    for (int step = step_lo; step < step_hi; step++) {
+        const int cur = (step - step_lo) & 1, nxt = cur ^ 1;
+        if (step + 1 < step_hi) load_step(step + 1, us_of(nxt), rs_of(nxt), step + 1 >= full_steps);
         const lds_float *us = us_of(cur), *rs = rs_of(cur);
 #pragma unroll
         for (int cp = 0; cp + 1 < CK / 2; cp++) {
@@ -1808,20 +1818,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
             }
             __syncthreads();
             const int n = n0 + fn * 32 + l32;
-            if (n < p.wT) {
-                const int img = n / per_img, r = n - img * per_img, ty = r / p.wtw, tx = r - ty * p.wtw;
+            const int nc = n < p.wT ? n : 0;
+            const int img = nc / per_img, r = nc - img * per_img, ty = r / p.wtw, tx = r - ty * p.wtw;
 #pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    float y[2][2];
+            for (int k = 0; k < 4; k++) {
+                float y[2][2];
 #pragma unroll
-                    for (int b = 0; b < 2; b++) {
-                        float t[4];
+                for (int b = 0; b < 2; b++) {
+                    float t[4];
 #pragma unroll
-                        for (int i = 0; i < 4; i++) t[i] = xch[((i * 2 + b) * 16 + 4 * wave + k) * 64 + lane];
-                        y[0][b] = __fadd_rn(__fadd_rn(t[0], t[1]), t[2]);
-                        y[1][b] = __fsub_rn(__fsub_rn(t[1], t[2]), t[3]);
-                    }
-                    wino_store_row<MF>(p, epi, m0, fm * 32 + 8 * wave + 4 * half + k, img, ty, tx, plane, pair, y[0][0], y[0][1], y[1][0], y[1][1]);
+                    for (int i = 0; i < 4; i++) t[i] = xch[((i * 2 + b) * 16 + 4 * wave + k) * 64 + lane];
+                    y[0][b] = __fadd_rn(__fadd_rn(t[0], t[1]), t[2]);
+                    y[1][b] = __fsub_rn(__fsub_rn(t[1], t[2]), t[3]);
+                }
+                if (split) {
+                    // this slice's share of the four outputs, raw: wino_fused_reduce_kernel adds the slices and finishes
+                    // (layout [slice][tile][32x32 block][wavefront][k][lane] of four floats: a store writes 1 KB)
+                    const size_t tiles = (gridDim.x - (unsigned)p.main_tiles) / p.nslices;
+                    floatx4 *dst = reinterpret_cast<floatx4 *>(p.partial) +
+                                   (((((size_t)slice * tiles + local_tile) * (FM * FN) + fm * FN + fn) * 4 + wave) * 4 + k) * 64 + lane;
+                    floatx4 yv;
+                    yv.x = y[0][0], yv.y = y[0][1], yv.z = y[1][0], yv.w = y[1][1];
+                    *dst = yv;
+                } else if (n < p.wT) {
+                    const int ml = fm * 32 + 8 * wave + 4 * half + k;
+                    wino_store_row(p, channel_from_lds<MF>(epi, ml), m0 + ml, img, ty, tx, plane, pair, y[0][0], y[0][1], y[1][0], y[1][1]);
                 }
             }
         }
@@ -1830,6 +1851,47 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
         __syncthreads();
         trace_mark(p, 3);
     }
+}
+
+// Finishes the tiles of wino_fused_kernel that the launch plan divided along the channels: one workgroup per 32x32 block of
+// such a tile, the fused kernel's thread -> (filter row, block) mapping; adds the slices' four raw outputs in increasing
+// channel order, starting from slice 0's values (a fixed order: results do not depend on scheduling), then the epilogue.
+template <int FM, int FN>
+__global__ __launch_bounds__(256) void wino_fused_reduce_kernel(const ConvParams p) {
+    constexpr int MF = 32 * FM, NB = 32 * FN;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
+    const int blk = blockIdx.x % (FM * FN), local_tile = blockIdx.x / (FM * FN), fm = blk / FN, fn = blk % FN;
+    const size_t tiles = gridDim.x / (FM * FN);
+    const int tile = p.main_tiles + local_tile;
+    const int m_first = (tile % p.gm) * MF + fm * 32 + 8 * wave + 4 * half;  // this lane's rows: m_first + 0..3
+    const int n = (tile / p.gm) * NB + fn * 32 + l32;
+    ChannelEpilogue chan[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) chan[k] = load_channel(p, m_first + k < p.Kf ? m_first + k : p.Kf - 1);
+    const size_t slice_stride = tiles * (FM * FN) * 4 * 4 * 64;
+    const floatx4 *src = reinterpret_cast<const floatx4 *>(p.partial) + ((((size_t)local_tile * (FM * FN) + blk) * 4 + wave) * 4) * 64 + lane;
+    floatx4 y[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) y[k] = src[k * 64];
+    for (int sl = 1; sl < p.nslices; sl++) {
+        floatx4 x[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) x[k] = src[(size_t)sl * slice_stride + k * 64];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            y[k].x = __fadd_rn(y[k].x, x[k].x);
+            y[k].y = __fadd_rn(y[k].y, x[k].y);
+            y[k].z = __fadd_rn(y[k].z, x[k].z);
+            y[k].w = __fadd_rn(y[k].w, x[k].w);
+        }
+    }
+    if (n >= p.wT) return;
+    const int per_img = p.wth * p.wtw;
+    const int img = n / per_img, r = n - img * per_img, ty = r / p.wtw, tx = r - ty * p.wtw;
+    const size_t plane = (size_t)p.wP * p.wQ;
+    const bool pair = (p.wQ % 2 == 0) && (((size_t)p.O | (size_t)(p.residual ? p.residual : p.O)) % 8 == 0);
+#pragma unroll
+    for (int k = 0; k < 4; k++) wino_store_row(p, chan[k], m_first + k, img, ty, tx, plane, pair, y[k].x, y[k].y, y[k].z, y[k].w);
 }
 
 // ---------------------------------------------------------------- host side
@@ -1864,7 +1926,7 @@ thread_local char g_last_kernel[128] = "";
 int g_split = 1;  // divide the tiles left over after a whole number per CU along K (set_algo 5 turns it off)
 bool g_wino = false;  // set_algo(7): the Winograd form wherever it applies (8: only where a searched plan asks for it)
 bool g_wino_never = false;  // set_algo(9): no Winograd form at all, not in the plan search and not from a kept plan
-int g_force_tile = -1, g_force_slices = -1;  // eddlhip_conv2d_force_plan
+thread_local int g_force_tile = -1, g_force_slices = -1;  // eddlhip_conv2d_force_plan (per calling thread: the plan search steers its own launches with them)
 unsigned long long *g_trace = nullptr;       // eddlhip_conv2d_trace
 long long g_trace_wgs = 0;
 
@@ -1876,7 +1938,8 @@ struct TunedPlan {
     int key[10];       // N C Kf R S sr sc P Q direct
     int tile, slices;  // tile -1: the planner's own choice was the fastest; tile 4: the Winograd form
 };
-bool g_autotune = false, g_tuning = false;
+bool g_autotune = false;
+thread_local bool g_tuning = false;  // this thread is inside a plan search: the convolutions it times start no search of their own
 std::vector<TunedPlan> g_tuned[EDDLHIP_MAX_DEVICES];
 
 struct Variant {
@@ -1916,11 +1979,30 @@ struct FusedVariant {
     const char *name;
     int fm, fn, ck;
     void (*kernel)(const ConvParams);
+    void (*reduce)(const ConvParams);
 };
-#define FUSED(FM, FN, CK, WPE) {"wino_fused_kernel<" #FM "," #FN "," #CK "," #WPE ">", FM, FN, CK, wino_fused_kernel<FM, FN, CK, WPE>}
+#define FUSED(FM, FN, CK, WPE) \
+    {"wino_fused_kernel<" #FM "," #FN "," #CK "," #WPE ">", FM, FN, CK, wino_fused_kernel<FM, FN, CK, WPE>, wino_fused_reduce_kernel<FM, FN>}
 const FusedVariant kfused[] = {FUSED(1, 1, 4, 4), FUSED(2, 1, 4, 3)};
 constexpr int NUM_FUSED = (int)(sizeof(kfused) / sizeof(kfused[0]));
+constexpr int FUSED_TILE0 = 6;      // plan "tile" numbers 6 .. 6 + NUM_FUSED - 1 name these shapes (0..3: direct tiles, 4 / 5: the other Winograd forms)
 constexpr int FUSED_ROW_ALIGN = 8;  // the transformed filters are padded to whole K-steps of every variant
+
+// K slices of the left-over tiles of a one-launch Winograd plan that asks for `slices` of them (T blocks in the launch):
+// the tiles beyond a whole number per CU are divided, as in forced_plan; 1 = nothing is divided
+int fused_slices(const FusedVariant &fv, int slices, long long T, int C, int Kf, int num_cu, long long *leftover_out = nullptr, int *slice_steps_out = nullptr) {
+    const int nsteps = (C + fv.ck - 1) / fv.ck;
+    const long long tiles = (long long)((Kf + 32 * fv.fm - 1) / (32 * fv.fm)) * ((T + 32 * fv.fn - 1) / (32 * fv.fn));
+    const long long leftover = tiles % num_cu;
+    const int want = slices < 1 ? 1 : (slices > nsteps ? nsteps : slices);
+    int slice_steps = (nsteps + want - 1) / want;
+    int nslices = (nsteps + slice_steps - 1) / slice_steps;
+    if (leftover == 0) nslices = 1;
+    if (nslices == 1) slice_steps = nsteps;
+    if (leftover_out) *leftover_out = nslices > 1 ? leftover : 0;
+    if (slice_steps_out) *slice_steps_out = slice_steps;
+    return nslices;
+}
 
 // Launch plan: tile shape and, for the tiles that do not divide evenly over the CUs, the number
 // of K slices.  The MFMA pipe of a CU is shared by its resident workgroups, so a launch takes as
@@ -2177,7 +2259,8 @@ int eddlhip_conv2d_uncache_filters(int dev, const float *K) {
 }
 
 int eddlhip_conv2d_force_plan(int tile, int slices) {
-    EH_REQUIRE(tile >= -1 && tile <= 6, "conv2d_force_plan: tile is -1 (automatic), 0..3, or 4 / 5 / 6 (the Winograd forms where they apply)");
+    EH_REQUIRE(tile >= -1 && tile < FUSED_TILE0 + NUM_FUSED, "conv2d_force_plan: tile is -1 (automatic), 0..3, or 4 .. %d (the Winograd forms where they apply)",
+               FUSED_TILE0 + NUM_FUSED - 1);
     g_force_tile = tile;
     g_force_slices = slices;
     return 0;
@@ -2224,7 +2307,7 @@ int eddlhip_conv2d_tuned_load(int dev, const char *host_path) {
         int *k = t.key;
         const int got = sscanf(line, "%d %d %d %d %d %d %d %d %d %d | %d %d", k, k + 1, k + 2, k + 3, k + 4, k + 5, k + 6, k + 7, k + 8, k + 9, &t.tile,
                                &t.slices);
-        if (got != 12 || t.tile < -1 || t.tile > 6 || t.slices < 1 || t.slices > (t.tile == 6 ? NUM_FUSED : 16)) {
+        if (got != 12 || t.tile < -1 || t.tile >= FUSED_TILE0 + NUM_FUSED || t.slices < 1 || t.slices > 16) {  // (no search tries more than 16 slices)
             bad = true;
             break;
         }
@@ -2301,6 +2384,11 @@ namespace {
 struct GemmBatch {
     const float *Wp;
     size_t stride;
+    // Workspace the launch may take (its partial tiles), which the Winograd driver leaves free in front of its own
+    // buffers; with need_out set the call launches nothing and only reports what it would take: exactly, under the plan
+    // that is fixed for its geometry, or the largest need of any plan while a search could still pick one.
+    size_t reserve;
+    size_t *need_out;
 };
 // eddlhip_conv2d_fwd_maxpool: the 2x2, stride-2 max-pool the caller wants of this thread's current convolution.  A
 // Winograd form computes it in its epilogue and says so (`done`); after any other form the entry point launches the pool
@@ -2313,15 +2401,16 @@ struct PoolRequest {
 thread_local PoolRequest *g_pool_req = nullptr;
 // Workspace a product launch may take for the partial tiles of a K-split plan: fewer than one tile per CU left over,
 // at most 16 slices each, 128 x 128 floats per tile.  The Winograd driver keeps its own buffers behind this much.
-constexpr size_t WINO_INNER_RESERVE = (size_t)16 * 255 * 128 * 128 * sizeof(float);
+// The plan search tries the Winograd forms that keep a transformed input in memory only below this much workspace.
+constexpr size_t WINO_SEARCH_CAP = (size_t)512 << 20;
 
 int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
                     int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
                     const float *bn_var, float bn_eps, const float *residual, int relu);
 
-int conv2d_winograd_fused(int variant, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
-                          int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
-                          const float *bn_var, float bn_eps, const float *residual, int relu);
+int conv2d_winograd_fused(int variant, int slices, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O,
+                          int N, int C, int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b,
+                          const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu);
 
 // Whether the Winograd form can run this convolution: 3x3, stride 1, and the product launch within the limits of
 // conv2d_fwd_impl (one "image" of transformed input or output below 1 GiB, fewer than 2^31 blocks).
@@ -2342,7 +2431,152 @@ bool winograd_fold_applies(int N, int C, int Kf, int R, int S, int sr, int sc, i
 int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
                     int H, int W, int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g,
                     const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu,
-                    const GemmBatch *gemm = nullptr) {
+                    const GemmBatch *gemm = nullptr);
+
+// One convolution call, as the plan search repeats it.
+struct ConvCall {
+    int dev;
+    const float *I, *I2;
+    int uh, uw;
+    const float *K, *bias;
+    float *O;
+    int N, C, H, W, Kf, R, S, sr, sc, pt, pl, P, Q;
+    const float *bn_g, *bn_b, *bn_mean, *bn_var;
+    float bn_eps;
+    const float *residual;
+    int relu;
+};
+int run_call(const ConvCall &c) {
+    return conv2d_fwd_impl(false, c.dev, c.I, c.I2, c.uh, c.uw, c.K, c.bias, c.O, c.N, c.C, c.H, c.W, c.Kf, c.R, c.S, c.sr, c.sc, c.pt, c.pl, c.P, c.Q,
+                           c.bn_g, c.bn_b, c.bn_mean, c.bn_var, c.bn_eps, c.residual, c.relu);
+}
+
+constexpr int kSearchSlices[8] = {1, 2, 3, 4, 6, 8, 12, 16};  // K-slice counts the search tries per tile shape
+
+// What the Winograd forms that keep a transformed input take from the workspace (3x3: patch side 4, 2x2: 3): transformed
+// filters unless kept, V, and for the three-kernel form M and room for the product launch's partial tiles.
+size_t winograd_workspace(bool fold, int N, int C, int Kf, int fs, int P, int Q, int num_cu) {
+    const size_t np = (size_t)(fs + 1) * (fs + 1);
+    const size_t T = (size_t)N * ((P + 1) / 2) * ((Q + 1) / 2), Tp = (T + 127) / 128 * 128;
+    const size_t rows = ((size_t)C + 15) / 16 * 16, Mp = ((size_t)Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
+    size_t bytes = np * rows * Mp * 4 + np * C * Tp * 4;
+    if (!fold) bytes += np * Kf * Tp * 4 + (size_t)16 * (num_cu - 1) * 128 * 128 * 4;
+    return bytes;
+}
+
+// The plan search of eddlhip_conv2d_autotune (the reference finds its algorithm the same way, by measurement on a layer's
+// first forward: src/hardware/gpu/nn/gpu_conv.cu:42-66, 211-213).  Runs the call under every launch plan on the call's own
+// tensors (each plan writes the same output, up to the rounding of its summation order), every launch timed by itself,
+// and takes each plan's FASTEST launch (noise only ever adds time).  Then, so that two searches of one geometry agree:
+// of all plans within 3 % of the fastest one it keeps the first in a fixed order of preference - the planner's own plan,
+// the one-launch Winograd form, the direct tiles, the Winograd forms with a transformed input in memory; within a form
+// fewer K slices first.  Returns 0 with *out filled, 1 when these tensors cannot be searched on (the output overlaps an
+// input: repeating the call would change what it reads), or minus the error code of a runtime failure.
+int search_plan(const ConvCall &c, const Variant *family, long long chunk_pix, bool wino_ok, bool fold_ok, bool fused_ok, TunedPlan *out) {
+    {
+        const size_t out_bytes = (size_t)c.N * c.Kf * c.P * c.Q * 4, in_bytes = (size_t)c.N * (c.I2 ? c.C / 2 : c.C) * c.H * c.W * 4;
+        const char *o_lo = (const char *)c.O, *o_hi = o_lo + out_bytes;
+        auto overlaps = [&](const float *ptr, size_t bytes) { return ptr != nullptr && (const char *)ptr < o_hi && o_lo < (const char *)ptr + bytes; };
+        if (overlaps(c.I, in_bytes) || overlaps(c.I2, in_bytes) || overlaps(c.residual, out_bytes)) return 1;
+    }
+    hipStream_t st = state(c.dev).stream;
+    const int num_cu = state(c.dev).num_cu;
+    struct Cand {
+        int rank, tile, slices;
+        float ms;
+    };
+    std::vector<Cand> cands;
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess) return -set_error(EDDLHIP_EHIP, "conv2d plan search: hipEventCreate failed");
+    if (hipEventCreate(&e1) != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return -set_error(EDDLHIP_EHIP, "conv2d plan search: hipEventCreate failed");
+    }
+    PoolRequest *const pool_req = g_pool_req;  // the candidates are timed as plain convolutions
+    g_pool_req = nullptr;
+    const int ft = g_force_tile, fs = g_force_slices;
+    int fatal = 0;
+    // 0: timed; EDDLHIP_EINVAL / EDDLHIP_ENOMEM: the plan does not apply here (skipped); anything else: give up
+    auto time_plan = [&](int rank, int tile, int slices) {
+        if (fatal != 0) return;
+        g_force_tile = tile;
+        g_force_slices = slices;
+        float best = 0.0f;
+        int reps = 1;
+        int rc = 0;
+        for (int rep = 0; rep <= reps && rc == 0; rep++) {  // launch 0 warms up and sets the number of timed launches
+            if (hipEventRecord(e0, st) != hipSuccess) rc = EDDLHIP_EHIP;
+            if (rc == 0) rc = run_call(c);
+            float ms = 0.0f;
+            if (rc == 0 && (hipEventRecord(e1, st) != hipSuccess || hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess))
+                rc = set_error(EDDLHIP_EHIP, "conv2d plan search: timing a launch failed");
+            if (rc != 0) break;
+            if (rep == 0) reps = ms >= 0.35f ? 3 : (ms >= 0.1f ? 5 : 9);
+            else if (rep == 1 || ms < best) best = ms;
+        }
+        g_force_tile = ft;
+        g_force_slices = fs;
+        if (rc == 0) cands.push_back({rank, tile, slices, best});
+        else if (rc == EDDLHIP_EINVAL || rc == EDDLHIP_ENOMEM) clear_error();
+        else fatal = rc;
+    };
+    g_tuning = true;
+    time_plan(0, -1, -1);
+    if (fatal == 0 && cands.empty()) fatal = set_error(EDDLHIP_EINVAL, "conv2d plan search: the planner's own plan did not run");
+    if (fused_ok)  // the one-launch Winograd form: its tile shapes, each undivided and with the left-over tiles in K slices
+        for (int fv = NUM_FUSED - 1; fv >= 0; fv--) {
+            int last_slices = 0;
+            for (int sl : kSearchSlices) {
+                const int ns = fused_slices(kfused[fv], sl, (long long)c.N * ((c.P + 1) / 2) * ((c.Q + 1) / 2), c.C, c.Kf, num_cu);
+                if (ns == last_slices) continue;  // the same plan as the one before
+                last_slices = ns;
+                time_plan(1 + (NUM_FUSED - 1 - fv), FUSED_TILE0 + fv, sl);
+            }
+        }
+    for (int tile = 0; tile < 4; tile++) {
+        int last_slices = 0;
+        for (int sl : kSearchSlices) {
+            const Plan fp = forced_plan(family, tile, sl, c.Kf, c.C, c.R * c.S, chunk_pix, num_cu);
+            if (fp.nslices == last_slices) continue;
+            last_slices = fp.nslices;
+            time_plan(10 + tile, tile, sl);
+        }
+    }
+    if (fold_ok && winograd_workspace(true, c.N, c.C, c.Kf, c.R, c.P, c.Q, num_cu) <= WINO_SEARCH_CAP) time_plan(20, 5, 1);
+    if (wino_ok && fatal == 0 && winograd_workspace(false, c.N, c.C, c.Kf, c.R, c.P, c.Q, num_cu) <= WINO_SEARCH_CAP) {
+        // the three-kernel form: its product launch is a geometry of its own, searched first (one untimed call with the
+        // search open), then timed under what that search kept
+        g_tuning = false;
+        g_force_tile = 4;
+        const int wrc = run_call(c);
+        g_force_tile = ft;
+        g_tuning = true;
+        if (wrc == 0) time_plan(21, 4, 1);
+        else if (wrc == EDDLHIP_EINVAL || wrc == EDDLHIP_ENOMEM) clear_error();
+        else fatal = wrc;
+    }
+    g_tuning = false;
+    g_pool_req = pool_req;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (fatal != 0) return -fatal;
+    float fastest = cands[0].ms;
+    for (const Cand &k : cands) fastest = k.ms < fastest ? k.ms : fastest;
+    const Cand *pick = nullptr;
+    for (const Cand &k : cands)
+        if (k.ms <= 1.03f * fastest && (pick == nullptr || k.rank < pick->rank || (k.rank == pick->rank && k.slices < pick->slices))) pick = &k;
+    out->tile = pick->tile;
+    out->slices = pick->tile < 0 ? 1 : pick->slices;
+    if (getenv("EDDLHIP_TUNE_VERBOSE"))
+        fprintf(stderr, "tune %d %d %d %d -> %d %dx%d s%d: planned %.1f us, fastest %.1f us, kept %.1f us (tile %d x %d slices) of %zu plans\n", c.N, c.C,
+                c.H, c.W, c.Kf, c.R, c.S, c.sr, cands[0].ms * 1e3f, fastest * 1e3f, pick->ms * 1e3f, out->tile, out->slices, cands.size());
+    return 0;
+}
+
+int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
+                    int H, int W, int Kf, int R, int S, int sr, int sc, int pad_top, int pad_left, int P, int Q, const float *bn_g,
+                    const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu,
+                    const GemmBatch *gemm) {
     EH_REQUIRE(N >= 0 && C > 0 && H > 0 && W > 0, "conv2d: bad input shape %dx%dx%dx%d", N, C, H, W);
     EH_REQUIRE(Kf > 0 && R > 0 && S > 0, "conv2d: bad filter shape %dx%dx%dx%d", Kf, C, R, S);
     EH_REQUIRE(sr > 0 && sc > 0, "conv2d: strides must be positive");
@@ -2470,13 +2704,14 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     // the one-launch form (3x3 filters only) needs no transformed copy of the input, so none of V's limits apply
     const bool fused_ok = !gemm && !no_alloc && g_algo == 0 && !g_wino_never && R == 3 && S == 3 && sr == 1 && sc == 1 &&
                           (long long)C * 16 * p.Mp * 4 < (1LL << 31);
-    if (fused_ok && g_force_tile == 6)
-        return conv2d_winograd_fused(g_force_slices < 1 ? 0 : (g_force_slices > NUM_FUSED ? NUM_FUSED - 1 : g_force_slices - 1), dev, I,
-                                     two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b, bn_mean, bn_var,
-                                     bn_eps, residual, relu);
+    if (fused_ok && g_force_tile >= FUSED_TILE0 && g_force_tile < FUSED_TILE0 + NUM_FUSED)
+        return conv2d_winograd_fused(g_force_tile - FUSED_TILE0, g_force_slices, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top,
+                                     pad_left, P, Q, bn_g, bn_b, bn_mean, bn_var, bn_eps, residual, relu);
     if ((wino_ok && (g_force_tile == 4 || (g_wino && g_force_tile < 0 && !g_tuning))) || (fold_ok && g_force_tile == 5))
         return conv2d_winograd(g_force_tile == 5, R, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g, bn_b,
                                bn_mean, bn_var, bn_eps, residual, relu);
+    const bool query = gemm != nullptr && gemm->need_out != nullptr;  // report the workspace need, launch nothing
+    bool plan_open = false;                                         // a search could still pick any plan for this geometry
     if (g_autotune && g_force_tile < 0 && g_algo == 0 && g_split != 0) {
         const int key[10] = {N, C, Kf, R, S, sr, sc, P, Q, direct};
         const TunedPlan *found = nullptr;
@@ -2484,105 +2719,40 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
             if (memcmp(t.key, key, sizeof(key)) == 0) found = &t;
         // (no search inside a search: a convolution being timed runs its product launch, a geometry of its own, under the
         // plan already kept for it)
-        if (found == nullptr && !g_tuning && !no_alloc && !state(dev).capturing && !g_prof_on) {
-            // First call with this geometry: run every plan on the call's own tensors (each writes the same output, up to
-            // the rounding of its summation order) and keep the fastest.  The planner's choice stays unless another plan
-            // beats it by more than the noise of the measurement.
+        const bool can_search = found == nullptr && !g_tuning && !no_alloc && !state(dev).capturing && !g_prof_on;
+        plan_open = can_search;
+        if (can_search && !query) {
+            const ConvCall call = {dev, I, I2, uh, uw, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q,
+                                   bn_g, bn_b, bn_mean, bn_var, bn_eps, residual, relu};
             TunedPlan best;
             memcpy(best.key, key, sizeof(key));
-            best.tile = -1;
-            best.slices = 1;
-            PoolRequest *const pool_req = g_pool_req;  // the candidates are timed as plain convolutions
-            g_pool_req = nullptr;
-            hipEvent_t e0, e1;
-            EH_TRY_HIP(hipEventCreate(&e0));
-            EH_TRY_HIP(hipEventCreate(&e1));
-            auto measure = [&](int tile, int slices, float *ms) -> int {
-                g_force_tile = tile;
-                g_force_slices = slices;
-                int rc = 0;
-                for (int rep = 0; rep < 4 && rc == 0; rep++) {  // the first launch is not timed
-                    if (rep == 1) rc = hipEventRecord(e0, st) == hipSuccess ? 0 : EDDLHIP_EHIP;
-                    if (rc == 0)
-                        rc = conv2d_fwd_impl(false, dev, I, I2, uh, uw, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
-                                             bn_mean, bn_var, bn_eps, residual, relu);
-                }
-                g_force_tile = -1;
-                g_force_slices = -1;
-                if (rc != 0) return rc;
-                if (hipEventRecord(e1, st) != hipSuccess || hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(ms, e0, e1) != hipSuccess)
-                    return EDDLHIP_EHIP;
-                return 0;
-            };
-            g_tuning = true;
-            float planned_ms = 0.0f, best_ms = 0.0f;
-            int rc = measure(-1, -1, &planned_ms);
-            best_ms = planned_ms;
-            static const int kSlices[8] = {1, 2, 3, 4, 6, 8, 12, 16};
-            for (int tile = 0; tile < 4 && rc == 0; tile++) {
-                int last_slices = 0;
-                for (int si = 0; si < 8 && rc == 0; si++) {
-                    const Plan fp = forced_plan(family, tile, kSlices[si], Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
-                    if (fp.nslices == last_slices) continue;  // the same plan as the one before
-                    last_slices = fp.nslices;
-                    float ms = 0.0f;
-                    if (measure(tile, kSlices[si], &ms) != 0) continue;  // a plan that does not apply here
-                    if (ms < best_ms && ms < 0.98f * planned_ms) {
-                        best_ms = ms;
-                        best.tile = tile;
-                        best.slices = kSlices[si];
-                    }
-                }
-            }
-            if (rc == 0 && wino_ok) {
-                // the Winograd form; its product launch is a geometry of its own, searched first (one untimed call with the
-                // search open), then timed under what that search kept
-                g_tuning = false;
-                g_force_tile = 4;
-                int wrc = conv2d_fwd_impl(false, dev, I, I2, uh, uw, K, bias, O, N, C, H, W, Kf, R, S, sr, sc, pad_top, pad_left, P, Q, bn_g, bn_b,
-                                          bn_mean, bn_var, bn_eps, residual, relu);
-                g_force_tile = -1;
-                g_tuning = true;
-                float ms = 0.0f;
-                if (wrc == 0 && measure(4, 1, &ms) == 0 && ms < best_ms && ms < 0.98f * planned_ms) {
-                    best_ms = ms;
-                    best.tile = 4;
-                    best.slices = 1;
-                }
-                if (fold_ok && measure(5, 1, &ms) == 0 && ms < best_ms && ms < 0.98f * planned_ms) {
-                    best_ms = ms;
-                    best.tile = 5;
-                    best.slices = 1;
-                }
-            }
-            if (rc == 0 && fused_ok) {
-                float ms = 0.0f;
-                for (int fv = 0; fv < NUM_FUSED; fv++)
-                    if (measure(6, fv + 1, &ms) == 0 && ms < best_ms && ms < 0.98f * planned_ms) {
-                        best_ms = ms;
-                        best.tile = 6;
-                        best.slices = fv + 1;
-                    }
-            }
-            g_tuning = false;
-            g_pool_req = pool_req;
-            (void)hipEventDestroy(e0);
-            (void)hipEventDestroy(e1);
-            if (rc != 0) return rc;
-            if (getenv("EDDLHIP_TUNE_VERBOSE"))
-                fprintf(stderr, "tune %d %d %d %d -> %d %dx%d s%d: planned %.1f us, best %.1f us (tile %d x %d slices)\n", N, C, H, W, Kf, R, S, sr,
-                        planned_ms * 1e3f / 3, best_ms * 1e3f / 3, best.tile, best.slices);
-            g_tuned[dev].push_back(best);
-            found = &g_tuned[dev].back();
+            const int src = search_plan(call, family, (long long)chunk_imgs * p.PQ, wino_ok, fold_ok, fused_ok, &best);
+            if (src < 0) return -src;  // a runtime error inside the search
+            if (src == 0) {
+                g_tuned[dev].push_back(best);
+                found = &g_tuned[dev].back();
+            }  // (src > 0: no search on these tensors - the planner's plan, nothing recorded)
         }
         if (found != nullptr && ((found->tile == 4 && wino_ok) || (found->tile == 5 && fold_ok)))
             return conv2d_winograd(found->tile == 5, R, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g,
                                    bn_b, bn_mean, bn_var, bn_eps, residual, relu);
-        if (found != nullptr && found->tile == 6 && fused_ok)
-            return conv2d_winograd_fused(found->slices - 1, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g,
+        if (found != nullptr && found->tile >= FUSED_TILE0 && found->tile < FUSED_TILE0 + NUM_FUSED && fused_ok)
+            return conv2d_winograd_fused(found->tile - FUSED_TILE0, found->slices, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g,
                                          bn_b, bn_mean, bn_var, bn_eps, residual, relu);
         if (found != nullptr && found->tile >= 0 && found->tile < 4)
             plan = forced_plan(family, found->tile, found->slices, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
+    }
+    if (query && plan_open) {
+        // the largest partial-tile need of any plan the search tries
+        size_t worst = 0;
+        for (int tile = 0; tile < 4; tile++)
+            for (int sl : kSearchSlices) {
+                const Plan fp = forced_plan(family, tile, sl, Kf, C, R * S, (long long)chunk_imgs * p.PQ, state(dev).num_cu);
+                const size_t need = fp.nslices > 1 ? (size_t)fp.nslices * fp.leftover * family[tile].bm * family[tile].bn * sizeof(float) : 0;
+                if (need > worst) worst = need;
+            }
+        *gemm->need_out = worst;
+        return 0;
     }
     const Variant *v = &family[plan.tile];
     const int bk = v->cpb ? v->cpb * R * S : 16;
@@ -2613,6 +2783,12 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     const size_t wp_bytes = cached ? 0 : (((size_t)rows * p.Mp * sizeof(float) + 255) & ~(size_t)255);
     const size_t taps_bytes = v->cpb ? 0 : (((size_t)rows * sizeof(int32x4) + 255) & ~(size_t)255);
     const size_t partial_bytes = (size_t)nslices * leftover * tile_floats * sizeof(float);
+    if (query) {
+        *gemm->need_out = wp_bytes + taps_bytes + partial_bytes;
+        return 0;
+    }
+    if (gemm)  // (checked before the workspace is touched: growing it would free the caller's buffers)
+        EH_REQUIRE(wp_bytes + taps_bytes + partial_bytes <= gemm->reserve, "conv2d: internal error, workspace of a product launch");
     void *ws = nullptr;
     if (no_alloc) {
         const size_t need = wp_bytes + taps_bytes + partial_bytes;
@@ -2629,7 +2805,6 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     if (gemm) {
         EH_REQUIRE(v->cpb != 0 && gemm->stride == (size_t)rows * p.Mp && p.PQ % v->bn == 0,
                    "conv2d: internal error, the product launch of a Winograd convolution does not fit its operands");
-        EH_REQUIRE(wp_bytes + taps_bytes + partial_bytes <= WINO_INNER_RESERVE, "conv2d: internal error, workspace of a product launch");
         p.w_img_stride = gemm->stride;
     }
     p.taps = (const int32x4 *)((char *)ws + wp_bytes);
@@ -2723,9 +2898,23 @@ int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2,
     const size_t u_bytes = U ? 0 : ((u_floats * sizeof(float) + 255) & ~(size_t)255);
     const size_t v_bytes = (v_floats * sizeof(float) + 255) & ~(size_t)255;
     const size_t m_bytes = fold ? 0 : ((m_floats * sizeof(float) + 255) & ~(size_t)255);  // folded: M is never written
+    // what the product launch of the three-kernel form will take for its partial tiles lies in front of U, V and M
+    size_t inner = 0;
+    if (!fold) {
+        const GemmBatch gq = {K, (size_t)rows * Mp, 0, &inner};
+        const int ft = g_force_tile, fsl = g_force_slices;
+        g_force_tile = -1;
+        g_force_slices = -1;
+        const int qrc = conv2d_fwd_impl(false, dev, K, nullptr, 1, 1, K, nullptr, O, np, C, 1, Tp, Kf, 1, 1, 1, 1, 0, 0, 1, Tp, nullptr, nullptr, nullptr, nullptr,
+                                        0.0f, nullptr, 0, &gq);
+        g_force_tile = ft;
+        g_force_slices = fsl;
+        if (qrc != 0) return qrc;
+        inner = (inner + 255) & ~(size_t)255;
+    }
     void *ws = nullptr;
-    EH_TRY(get_workspace(dev, WINO_INNER_RESERVE + u_bytes + v_bytes + m_bytes, &ws));
-    char *base = (char *)ws + WINO_INNER_RESERVE;
+    EH_TRY(get_workspace(dev, inner + u_bytes + v_bytes + m_bytes, &ws));
+    char *base = (char *)ws + inner;
     float *Uw = (float *)base, *V = (float *)(base + u_bytes), *M = (float *)(base + u_bytes + v_bytes);
     if (U == nullptr) {
         const dim3 grid((unsigned)(((size_t)rows * Mp + 255) / 256));
@@ -2812,7 +3001,7 @@ int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2,
 
     // ---- the 16 products: M[xi] = U[xi] x V[xi]
     {
-        const GemmBatch gb = {U, (size_t)rows * Mp};
+        const GemmBatch gb = {U, (size_t)rows * Mp, inner, nullptr};
         const int ft = g_force_tile, fs = g_force_slices;
         g_force_tile = -1;
         g_force_slices = -1;
@@ -2840,17 +3029,17 @@ int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2,
         else hipLaunchKernelGGL(wino_output_kernel<3>, grid, dim3(256), 0, st, p, (const float *)M, th, tw, T, Tp);
     }
     EH_CHECK_LAUNCH();
-    char inner[sizeof(g_last_kernel)];
-    snprintf(inner, sizeof(inner), "%s", g_last_kernel);
-    snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%.100s, %d blocks]", inner, Tp);
+    char product[sizeof(g_last_kernel)];
+    snprintf(product, sizeof(product), "%s", g_last_kernel);
+    snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%.100s, %d blocks]", product, Tp);
     return 0;
 }
 
 // The one-launch Winograd form of a 3x3 stride-1 convolution (wino_fused_kernel).  Workspace: the transformed filters,
-// unless a registered filter tensor keeps them.
-int conv2d_winograd_fused(int variant, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O, int N, int C,
-                          int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b, const float *bn_mean,
-                          const float *bn_var, float bn_eps, const float *residual, int relu) {
+// unless a registered filter tensor keeps them, and the partial output tiles of a K-split plan.
+int conv2d_winograd_fused(int variant, int slices, int dev, const float *I, const float *I2, int uh, int uw, const float *K, const float *bias, float *O,
+                          int N, int C, int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b,
+                          const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu) {
     hipStream_t st = state(dev).stream;
     const FusedVariant &fv = kfused[variant];
     // a max-pool asked for with this convolution is taken into the epilogue where every 2x2 block of outputs is whole
@@ -2860,6 +3049,19 @@ int conv2d_winograd_fused(int variant, int dev, const float *I, const float *I2,
     const int rows = (C + FUSED_ROW_ALIGN - 1) / FUSED_ROW_ALIGN * FUSED_ROW_ALIGN, Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
     const size_t u_floats = (size_t)16 * rows * Mp;
     EH_REQUIRE(u_floats * sizeof(float) < ((size_t)1 << 31), "conv2d: the transformed filters (16 x %d x %d) exceed 2 GiB", rows, Mp);
+
+    // a launch covers one batch chunk: input within the 2 GiB a buffer descriptor addresses, fewer than 2^30 blocks
+    const int Cimg = I2 ? C / 2 : C;
+    const long long img_elems = (long long)Cimg * H * W, per_img = (long long)th * tw;
+    long long max_imgs = (1LL << 29) / img_elems;
+    if (max_imgs > 0x3ffffe00LL / per_img) max_imgs = 0x3ffffe00LL / per_img;
+    EH_REQUIRE(max_imgs >= 1, "conv2d: one image of %lld elements is too large for the Winograd form", img_elems);
+    const int chunk_imgs = (int)((N < max_imgs) ? N : max_imgs);
+    long long leftover = 0;
+    int slice_steps = 0;
+    const int nslices = fused_slices(fv, slices, chunk_imgs * per_img, C, Kf, state(dev).num_cu, &leftover, &slice_steps);
+    const size_t tile_floats = (size_t)32 * fv.fm * 32 * fv.fn * 4;  // four outputs per filter and block
+    const size_t partial_bytes = (size_t)nslices * leftover * tile_floats * sizeof(float);
 
     const float *U = nullptr;
     {
@@ -2883,9 +3085,10 @@ int conv2d_winograd_fused(int variant, int dev, const float *I, const float *I2,
             }
         }
     }
+    const size_t u_bytes = U ? 0 : ((u_floats * sizeof(float) + 255) & ~(size_t)255);
+    void *ws = nullptr;
+    if (u_bytes + partial_bytes > 0) EH_TRY(get_workspace(dev, u_bytes + partial_bytes, &ws));
     if (U == nullptr) {
-        void *ws = nullptr;
-        EH_TRY(get_workspace(dev, u_floats * sizeof(float), &ws));
         const dim3 grid((unsigned)(((size_t)rows * Mp + 255) / 256));
         hipLaunchKernelGGL(wino_filter_kernel<4>, grid, dim3(256), 0, st, K, (float *)ws, Kf, C, Mp, rows, 1);
         EH_CHECK_LAUNCH();
@@ -2894,7 +3097,6 @@ int conv2d_winograd_fused(int variant, int dev, const float *I, const float *I2,
 
     ConvParams q;
     memset(&q, 0, sizeof(q));
-    const int Cimg = I2 ? C / 2 : C;
     q.Csplit = I2 ? C / 2 : C; q.Cimg = Cimg; q.uh = uh; q.uw = uw;
     q.Wp = U; q.K = K;
     q.bias = bias; q.bn_g = bn_g; q.bn_b = bn_b; q.bn_mean = bn_mean; q.bn_var = bn_var;
@@ -2902,16 +3104,10 @@ int conv2d_winograd_fused(int variant, int dev, const float *I, const float *I2,
     q.C = C; q.H = H; q.W = W; q.Kf = Kf; q.R = 3; q.S = 3; q.sr = 1; q.sc = 1; q.pt = pad_top; q.pl = pad_left; q.P = P; q.Q = Q;
     q.CRS = C * 9; q.Mp = Mp; q.PQ = P * Q;
     q.nsteps = (C + fv.ck - 1) / fv.ck;
-    q.slice_steps = q.nsteps; q.nslices = 1;
     q.wp_bytes = (unsigned)(u_floats * sizeof(float));
     q.wth = th; q.wtw = tw; q.wP = P; q.wQ = Q; q.wps = 4;
     q.gm = (Kf + 32 * fv.fm - 1) / (32 * fv.fm);
-    // a launch covers one batch chunk: input within the 2 GiB a buffer descriptor addresses, fewer than 2^31 blocks
-    const long long img_elems = (long long)Cimg * H * W, per_img = (long long)th * tw;
-    long long max_imgs = (1LL << 29) / img_elems;
-    if (max_imgs > 0x3ffffe00LL / per_img) max_imgs = 0x3ffffe00LL / per_img;
-    EH_REQUIRE(max_imgs >= 1, "conv2d: one image of %lld elements is too large for the Winograd form", img_elems);
-    const int chunk_imgs = (int)((N < max_imgs) ? N : max_imgs);
+    q.partial = (float *)((char *)ws + u_bytes);
     for (long long b0 = 0; b0 < N; b0 += chunk_imgs) {
         const int nb = (int)((N - b0 < chunk_imgs) ? N - b0 : chunk_imgs);
         q.N = nb;
@@ -2923,20 +3119,30 @@ int conv2d_winograd_fused(int variant, int dev, const float *I, const float *I2,
         q.wT = (int)(nb * per_img);
         q.npix = q.wT;
         q.gn = (q.wT + 32 * fv.fn - 1) / (32 * fv.fn);
-        EH_REQUIRE((long long)q.gm * q.gn <= 0x3fffffffLL, "conv2d: too many tiles");
-        q.main_tiles = q.gm * q.gn;
+        const long long tiles = (long long)q.gm * q.gn;
+        EH_REQUIRE(tiles <= 0x3fffffffLL, "conv2d: too many tiles");
+        const long long split_tiles = (nb == chunk_imgs) ? leftover : 0;  // a short last chunk runs undivided
+        q.main_tiles = (int)(tiles - split_tiles);
+        q.nslices = split_tiles > 0 ? nslices : 1;
+        q.slice_steps = split_tiles > 0 ? slice_steps : q.nsteps;
         if (pool != nullptr) {
             const size_t po = (size_t)b0 * Kf * per_img;
             q.pool_O = pool->O + po; q.pool_ix = pool->ix + po; q.pool_iy = pool->iy + po;
             if (!pool->keep) q.O = nullptr;
         }
-        q.trace = (g_trace != nullptr && q.main_tiles <= g_trace_wgs) ? g_trace : nullptr;
+        const long long wgs = q.main_tiles + split_tiles * q.nslices;
+        q.trace = (g_trace != nullptr && wgs <= g_trace_wgs) ? g_trace : nullptr;
         EH_TRY(prof_begin(st));
-        hipLaunchKernelGGL(fv.kernel, dim3((unsigned)q.main_tiles), dim3(256), 0, st, q);
+        hipLaunchKernelGGL(fv.kernel, dim3((unsigned)wgs), dim3(256), 0, st, q);
         EH_CHECK_LAUNCH();
         EH_TRY(prof_end(st));
+        if (split_tiles > 0) {
+            hipLaunchKernelGGL(fv.reduce, dim3((unsigned)(split_tiles * fv.fm * fv.fn)), dim3(256), 0, st, q);
+            EH_CHECK_LAUNCH();
+        }
     }
-    snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%s, %lld blocks]", fv.name, (long long)N * per_img);
+    if (leftover > 0) snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%s +ksplit(%lld tiles x %d), %lld blocks]", fv.name, leftover, nslices, (long long)N * per_img);
+    else snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%s, %lld blocks]", fv.name, (long long)N * per_img);
     return 0;
 }
 

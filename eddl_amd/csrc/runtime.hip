@@ -22,6 +22,8 @@ int set_error(int code, const char *fmt, ...) {
     return code;
 }
 
+void clear_error() { g_error[0] = 0; }
+
 int use_device(int dev) {
     if (dev < 0 || dev >= EDDLHIP_MAX_DEVICES) return set_error(EDDLHIP_ENODEV, "device index %d out of range", dev);
     DeviceState &s = g_state[dev];
@@ -112,6 +114,19 @@ int eddlhip_workspace_bytes(int dev, size_t *bytes) {
     EH_REQUIRE(bytes != nullptr, "bytes is NULL");
     EH_TRY(use_device(dev));
     *bytes = state(dev).workspace_bytes;
+    return 0;
+}
+
+int eddlhip_workspace_trim(int dev) {
+    EH_TRY(use_device(dev));
+    EH_NOT_CAPTURING(dev, "eddlhip_workspace_trim");
+    DeviceState &s = state(dev);
+    if (s.workspace == nullptr) return 0;
+    EH_TRY_HIP(hipStreamSynchronize(s.stream));
+    EH_TRY_HIP(hipFree(s.workspace));
+    s.workspace = nullptr;
+    s.workspace_bytes = 0;
+    s.workspace_generation++;  // graphs recorded before name memory that is gone
     return 0;
 }
 

@@ -24,8 +24,9 @@
  *  - Calls on one device must not overlap from several threads (the reference drives one
  *    device from one thread: src/net/net_api.cpp:146-171).  Different devices may be driven
  *    from different threads.  The tuning and measurement switches (eddlhip_conv2d_set_algo,
- *    _force_plan, _profile, _profile_read) act on the whole process: change them only while
- *    no other thread is inside the library.
+ *    _autotune, _tuned_load / _tuned_save, _profile, _profile_read, _trace) act on the whole
+ *    process: change them only while no other thread is inside the library.
+ *    eddlhip_conv2d_force_plan acts on the calling thread only.
  */
 #ifndef EDDLHIP_H
 #define EDDLHIP_H
@@ -61,8 +62,12 @@ int eddlhip_memcpy_d2h(int dev, void *host_dst, const void *dev_src, size_t byte
 int eddlhip_memcpy_d2d(int dev, void *dev_dst, const void *dev_src, size_t bytes);
 int eddlhip_fill(int dev, float *A, size_t n, float v);
 /* Size of the library's private workspace on the device right now (it only grows; 0 before the first call that
- * needs one).  No counterpart in the reference. */
+ * needs one).  eddlhip_workspace_trim waits for the device's kernels and releases the workspace, so that it grows back
+ * to what the calls from then on need - e.g. after a plan search, whose candidates take more than the plans it keeps.
+ * Not while a graph is being recorded; graphs recorded before name the released memory and refuse to launch.
+ * No counterpart in the reference. */
 int eddlhip_workspace_bytes(int dev, size_t *bytes);
+int eddlhip_workspace_trim(int dev);
 
 /* Batch staging.  The reference moves a batch to the device through pageable host tensors and
  * blocking copies (Net::distributeTensor / collectTensor, src/net/net_func.cpp:195-249; a D2H +
@@ -233,12 +238,17 @@ int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const fl
  * multiplications, the role of the WINOGRAD algorithms among those the reference lets cuDNN choose from
  * (src/hardware/gpu/nn/gpu_conv.cu:42-66).  Sums run in a fixed order (reproducible) and differ from the direct form's
  * by rounding: the result meets the same tolerance against the reference's CPU convolution, it is not bit-identical to
- * the direct form.  It takes workspace (16/4 of the input and of the output, plus 256 MB for its product launch), so
- * eddlhip_conv2d_fwd_noalloc never uses it.  Chosen per geometry by the plan search (below) where it is faster, or
- * everywhere by 7, or by eddlhip_conv2d_force_plan(4, .).  A second form, for input channel counts that are multiples of
- * 16 (force_plan(5, .), or the search): one product launch walks through all 16 patch positions and folds each product
- * into the outputs as it completes, so the products are never written and there is no output-transform launch; it sums
- * the 16 positions in another order than the first form (same tolerance, not the same bits).  Non-finite inputs: the
+ * the direct form.  It takes workspace (16/4 of the input and of the output, plus what its product launch needs for the
+ * partial tiles of a K-split plan), so eddlhip_conv2d_fwd_noalloc never uses it.  Chosen per geometry by the plan search
+ * (below) where it is faster, or everywhere by 7, or by eddlhip_conv2d_force_plan(4, .).  A second form, for input channel
+ * counts that are multiples of 16 (force_plan(5, .), or the search): one product launch walks through all 16 patch
+ * positions and folds each product into the outputs as it completes, so the products are never written and there is no
+ * output-transform launch; it sums the 16 positions in another order than the first form (same tolerance, not the same
+ * bits).  A third form, for 3x3 filters (force_plan(6, .) / (7, .), or the search): ONE launch that reads the NCHW input
+ * itself - raw pixels and transformed filters are staged through LDS, a lane derives its transformed operands from LDS
+ * reads and additions, a workgroup keeps all 16 positions' products of its tile (32 or 64 filters x 32 blocks) in
+ * registers and transforms them at the end - so no transformed input or product is ever in memory and the only
+ * workspace is the transformed filters (unless registered) and the partial output tiles of a K-split plan.  Non-finite inputs: the
  * transforms take differences of neighbouring pixels, so an infinity in the input can turn into NaN in outputs where the
  * direct form yields an infinity (all finite inputs give finite outputs as in the direct form); a caller that relies on
  * the propagation of infinities keeps the plan search off or calls eddlhip_conv2d_set_algo(9).
@@ -251,8 +261,14 @@ const char *eddlhip_conv2d_last_kernel(void);
 
 /* Plan search on first use.  eddlhip_conv2d_autotune(1): from now on the first eddlhip_conv2d_fwd* call with a geometry the
  * device has not seen (N, C, Kf, R, S, strides, output size P x Q) runs that convolution under every launch plan (tile
- * shape x K slices, three timed launches each, on the call's own tensors) and remembers the fastest; later calls with
- * that geometry take it.  The reference does the same on a layer's first forward, with
+ * shape x K slices and the Winograd forms, every launch timed by itself, the fastest of three to nine launches per plan,
+ * on the call's own tensors) and remembers one; later calls with that geometry take it.  Which one: of all plans within
+ * 3 % of the fastest, the first in a fixed order of preference (the planner's own plan, the one-launch Winograd form, the
+ * direct tiles, the Winograd forms that keep a transformed input in memory - those are tried only below 512 MB of
+ * workspace; within a form fewer K slices first), so that two searches of one geometry agree unless two plans differ by
+ * just that margin.  A caller that needs run-to-run identical bits loads a plans file instead of searching.  The call's
+ * tensors must not alias: when the output overlaps an input or the residual, nothing is searched or recorded and the
+ * planner's plan runs (repeating such a call would change what it reads).  The reference does the same on a layer's first forward, with
  * cudnnFindConvolutionForwardAlgorithm (src/hardware/gpu/nn/gpu_conv.cu:42-66, 211-213).  Neither the epilogue, nor the
  * image size and paddings (a folded Pad layer changes both), nor the form of the input (one tensor, two, upsampled) is
  * part of the geometry, so a layer computes the same sums in a fused plan and layer by layer.  A plan that divides tiles
@@ -275,7 +291,8 @@ int eddlhip_conv2d_tuned_load(int dev, const char *host_path);
  * workgroup), 1 (64x128), 2 (64x64), 3 (32x128) or -1 to give the choice back to the planner;
  * slices = number of K slices the tiles left over after a whole number per CU are divided into
  * (1 = none).  tile = 4: the Winograd form wherever it applies (its product launch is planned or searched as usual),
- * 5: its folded form wherever that applies; the planner's choice elsewhere. */
+ * 5: its folded form wherever that applies, 6 / 7: its one-launch form on tiles of 32 / 64 filters x 32 blocks, `slices`
+ * K slices for the left-over tiles as above; the planner's choice elsewhere.  Acts on the calling thread only. */
 int eddlhip_conv2d_force_plan(int tile, int slices);
 
 /* Filters that stay fixed between calls (inference).  Every eddlhip_conv2d_fwd first repacks its

@@ -361,16 +361,17 @@ WINOGRAD_CASES = [
 ]
 
 
-WINOGRAD_FORMS = [(4, 1), (5, 1), (6, 1), (6, 2)]
-WINOGRAD_FORM_IDS = ["three-kernels", "folded", "one-launch-32x32", "one-launch-64x32"]
+WINOGRAD_FORMS = [(4, 1), (5, 1), (6, 1), (7, 1), (6, 4), (7, 3)]
+WINOGRAD_FORM_IDS = ["three-kernels", "folded", "one-launch-32x32", "one-launch-64x32", "one-launch-32x32-4-slices", "one-launch-64x32-3-slices"]
 
 
 @pytest.mark.parametrize("form", WINOGRAD_FORMS, ids=WINOGRAD_FORM_IDS)
 @pytest.mark.parametrize("case", WINOGRAD_CASES, ids=lambda c: "x".join(str(v) for v in c[:5]))
 def test_conv2d_winograd_form_against_oracle(hip, oracle, case, form):
     """The Winograd forms (force_conv_plan(4, .): transforms and products as separate launches; 5: the output transform
-    folded into the one product launch, for channel counts that are whole K-steps; (6, v): everything in one launch that
-    reads the input itself, tile shape v) against the CPU oracle's direct convolution of the same logical input
+    folded into the one product launch, for channel counts that are whole K-steps; (6, s) and (7, s): everything in one
+    launch that reads the input itself, on 32- and 64-filter tiles, the tiles divided into s slices along the channels and
+    finished by a second kernel when s > 1) against the CPU oracle's direct convolution of the same logical input
     (concatenated / resized / zero-padded on the host), to the convolution tolerance; the epilogue after it is the
     oracle's, step by step."""
     form, variant = form
@@ -410,7 +411,8 @@ def test_conv2d_winograd_form_against_oracle(hip, oracle, case, form):
     finally:
         hip.force_conv_plan(-1, 1)
     if form != 5 or C % 16 == 0:
-        assert name.startswith("winograd[") and ("true,true>" in name) == (form == 5) and ("wino_fused_kernel" in name) == (form == 6), name
+        assert name.startswith("winograd[") and ("true,true>" in name) == (form == 5) and ("wino_fused_kernel" in name) == (form >= 6), name
+        assert ("+ksplit" in name) == (form >= 6 and variant > 1 and C > 4), name
     else:
         assert not name.startswith("winograd["), name       # the folded form needs whole K-steps of channels: the direct form ran
     assert_conv_close(ref, O.numpy(), "winograd %s" % (case,))
@@ -490,7 +492,7 @@ def test_conv2d_winograd_form_only_where_it_applies_and_with_kept_filters(hip, o
         hip.set_conv_algo("auto")
 
 
-@pytest.mark.parametrize("form", [-1, 4, 5, 6, 8])
+@pytest.mark.parametrize("form", [-1, 4, 5, 6, 7, 9])
 @pytest.mark.parametrize("case", ["bias+relu", "bn+residual+relu", "2x2 filter", "two tensors", "upsampled", "nan window"])
 def test_conv2d_fwd_maxpool_is_the_convolution_followed_by_the_pool(hip, form, case):
     """eddlhip_conv2d_fwd_maxpool against eddlhip_conv2d_fwd* + eddlhip_maxpool2d(2, 2, 2, 2) under the same launch plan
@@ -528,13 +530,13 @@ def test_conv2d_fwd_maxpool_is_the_convolution_followed_by_the_pool(hip, form, c
     pooled = lambda: (hip.full((N, Kf, P // 2, Q // 2), 9.0), hip.full((N, Kf, P // 2, Q // 2), 7.0), hip.full((N, Kf, P // 2, Q // 2), 7.0))
     A, B, K2 = pooled(), pooled(), pooled()
     variant = 1
-    if form == 8:                                      # the one-launch form on its 64-filter tile
-        form, variant = 6, 2
+    if form == 9:                                      # the one-launch form on its 64-filter tile, three K slices per tile
+        form, variant = 7, 3
     try:
         hip.force_conv_plan(form, variant)
         hip.conv2D(X, w, bias, O1, 1, 1, pad, pad, bn=bn, residual=res, relu=relu, second=second, upsample=upsample)
         name = hip.last_conv_kernel()
-        assert name.startswith("winograd") == (form >= 4 and not (form == 6 and fs == 2)), name   # (the one-launch form: 3x3 filters only)
+        assert name.startswith("winograd") == (form >= 4 and not (form >= 6 and fs == 2)), name   # (the one-launch form: 3x3 filters only)
         hip.mpool2D(O1, A[0], A[1], A[2], (2, 2), (2, 2), (0, 0, 0, 0))
         hip.conv2D(X, w, bias, O2, 1, 1, pad, pad, bn=bn, residual=res, relu=relu, second=second, upsample=upsample, pool=B, keep=True)
         assert hip.last_conv_kernel() == name
