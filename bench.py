@@ -198,9 +198,23 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, pl
         hip.conv_autotune(True)
         model.run()
         hip.synchronize()
-        hip.workspace_trim()   # the search's candidates took more workspace than the plans it kept
+        hip.workspace_trim()   # (the search has done so itself wherever its candidates grew the workspace)
         if plans:
             hip.conv_tuned_save(plans)
+    plans_info = None
+    if tune:
+        # the table the run ended up with (sorted lines of eddlhip_conv2d_tuned_save): its hash names the plans this line was measured under
+        import hashlib
+        import tempfile
+        with tempfile.NamedTemporaryFile("r", suffix=".txt") as fh:
+            hip.conv_tuned_save(fh.name)
+            lines = sorted(l.strip() for l in open(fh.name) if l.strip() and not l.startswith("#"))
+        forms = {"planner": 0, "direct_tile": 0, "winograd_three_kernels": 0, "winograd_folded": 0, "winograd_one_launch": 0}
+        for l in lines:
+            tile = int(l.split("|")[1].split()[0])
+            forms["planner" if tile < 0 else "direct_tile" if tile < 4 else "winograd_three_kernels" if tile == 4 else "winograd_folded" if tile == 5 else "winograd_one_launch"] += 1
+        plans_info = {"geometries": len(lines), "sha16": hashlib.sha256("\n".join(lines).encode()).hexdigest()[:16], "kept": forms,
+                      "workspace_bytes_after_search": hip.workspace_bytes()}
     step = model.run
     if graph:
         model.capture()
@@ -263,18 +277,22 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, pl
     # HBM bytes per launch of that kernel come from committed counter runs (two rocprofv3 --pmc passes cannot run
     # inside this process); they are reported only when the file names the kernel this run found dominant
     tpath = os.path.join(ROOT, "profiles", "traffic_%s.json" % workload)
-    if os.path.exists(tpath) and fused:  # the committed counter runs are of the fused plan
+    if os.path.exists(tpath) and fused:  # the committed counter runs are of the fused plan; the file lists every kernel of them by name
         with open(tpath) as fh:
             t = json.load(fh)
-        same_kernel = t.get("kernel", "").replace(" ", "") == dom_name.replace(" ", "")
-        if same_kernel and t.get("launches_per_step") in (None, dom_launches):
-            roofline["traffic"] = t.get("hbm_bytes_per_launch")
+        # (a kernel trace spells out a defaulted last template argument, the library's name for the kernel does not)
+        table = {k.replace(",false>", ">"): v for k, v in t.get("kernels", {}).items()}
+        entry = table.get(dom_name.replace(" ", ""))
+        if entry:
+            roofline["traffic"] = entry["hbm_bytes_per_launch"]
+            roofline["traffic_fetch_bytes"], roofline["traffic_write_bytes"] = entry.get("fetch_bytes_per_launch"), entry.get("write_bytes_per_launch")
             roofline["traffic_measured_at_commit"] = t.get("commit")
-        elif same_kernel:  # the plan search gave that kernel other layers in this run than in the counter runs
-            roofline["traffic_note"] = ("profiles/traffic_%s.json averages %s launches per step of this kernel, this run has %d"
-                                        % (workload, t.get("launches_per_step"), dom_launches))
+            per_step = entry["launches_in_counter_run"] / max(t.get("steps_in_counter_run", 1), 1)
+            if abs(per_step - dom_launches) > 1e-9:  # the plan search gave that kernel other layers in this run than in the counter runs
+                roofline["traffic_note"] = ("profiles/traffic_%s.json averages %.4g launches per step of this kernel, this run has %d"
+                                            % (workload, per_step, dom_launches))
         else:
-            roofline["traffic_note"] = "profiles/traffic_%s.json is for %s, not this run's dominant kernel" % (workload, t.get("kernel"))
+            roofline["traffic_note"] = "profiles/traffic_%s.json has no row for this run's dominant kernel" % workload
     # convolutions whose arithmetic intensity is below the ridge (first layers with 1-3 input channels, 1-filter
     # last layers): priced against the HBM roof
     hbm_bound = [{"name": r["name"], "kernel": r.get("kernel"), "ms": r.get("kernel_ms", r["ms"]),
@@ -283,6 +301,7 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, pl
                  for r in conv_rows if r["bytes"] > 0 and r["flops"] / r["bytes"] < RIDGE_FLOP_PER_BYTE and r.get("kernel_ms", r["ms"]) > 0]
     conv_ms = sum(r["ms"] for r in conv_rows)
     conv_flops = sum(r["flops"] for r in conv_rows)
+    executed_flops = sum(r.get("kernel_flops", r["flops"]) for r in conv_rows)  # what the launches multiply (Winograd layers: 2.25x less)
     summary = {"value": batch * steps / wall, "unit": "images/sec", "ms_per_step": wall * 1e3 / steps, "steps": steps, "warmup": warmup,
                "batch": batch, "fused_ops": len(model.ops), "roofline": roofline, "hbm_bound_convs": hbm_bound,
                # the layers' direct-form flop count over their device time: layers that run in the Winograd form multiply 2.25
@@ -291,10 +310,43 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, pl
                "conv_total": {"tflops": conv_flops / conv_ms / 1e9 if conv_ms else 0.0, "ms": conv_ms, "gflop": conv_flops / 1e9,
                               "frac_fp32_mfma_peak": (conv_flops / conv_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS) if conv_ms else 0.0,
                               "flops_counted": "direct form", "layers": len(conv_rows),
+                              # the flops the launches really multiply over the same time: the matrix pipe's useful share
+                              "executed_gflop": executed_flops / 1e9,
+                              "mfma_util": (executed_flops / conv_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS) if conv_ms else 0.0,
                               "winograd_layers": sum(1 for r in conv_rows if r.get("form") == "winograd")},
-               "device_ms_sum_of_ops": sum(op_ms)}
+               "device_ms_sum_of_ops": sum(op_ms), "plans": plans_info, "workspace_bytes": hip.workspace_bytes()}
     del model
     return summary, rows, out_host, desc
+
+
+def dropin_path():
+    """VGG-16, batch 32, through the drop-in route: the C++ host layer (the reference's Tensor / Layer / Net classes and
+    eddl:: functions over the binding's gpu_* functions), each mode in a child process of its own that builds the net from
+    the benchmark's seeds, lets the binding's gpu_init switch the plan search on (nothing in the environment) and times 20
+    forwards with the input resident: `layer_walk` is what an unchanged EDDL program gets (one gpu_* call per layer, a wait
+    after each, as the reference's wrappers wait), `fused_plan` the same net after eddl_hip::fuse(net)."""
+    import subprocess
+    import tempfile
+    driver = os.path.join(ROOT, "eddl_amd", "host", "net_driver")
+    if not os.path.exists(driver):
+        return {"note": "eddl_amd/host/net_driver is not built"}
+    result = {"workload": WORKLOADS["vgg16"][3], "unit": "images/sec", "plan_search": "on (gpu_init)", "host": "C++ (eddl_amd/host, tests/host/net_driver.cpp)"}
+    env = {k: v for k, v in os.environ.items() if k not in ("EDDLHIP_NO_TUNE", "EDDLHIP_PLANS", "EDDLHIP_PLANS_SAVE")}
+    with tempfile.TemporaryDirectory() as tmp:
+        for key, flags in (("layer_walk", "time"), ("fused_plan", "fused+time")):
+            cmd = [driver, flags + ":vgg16", "synth:3", "synth:1003:uniform", os.path.join(tmp, "y.raw"), "32", "224", "1000", "64", "128", "256", "512", "512", "4096"]
+            try:
+                res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300, env=env)
+            except subprocess.TimeoutExpired:
+                result[key] = {"note": "timed out"}
+                continue
+            line = [l for l in res.stdout.splitlines() if l.startswith("ms_per_forward")]
+            if res.returncode != 0 or not line:
+                result[key] = {"note": "net_driver failed: " + (res.stderr or res.stdout)[-300:]}
+                continue
+            f = line[0].split()
+            result[key] = {"value": float(f[3]), "ms_per_forward": float(f[1]), "workspace_bytes": int(f[5]), "tuned_geometries": int(f[7])}
+    return result
 
 
 # the other configurations, run after the headline workload: (steps, warmup, images of the oracle's parity sample)
@@ -320,6 +372,8 @@ def main():
     ap.add_argument("--no-workloads", action="store_true",
                     help="report the headline workload only (without it a default VGG-16 run also measures the other four "
                          "configurations, briefly, into the 'workloads' object of the JSON line)")
+    ap.add_argument("--no-dropin", action="store_true",
+                    help="skip the two child processes that time VGG-16 through the C++ host layer (the 'dropin' object of the JSON line)")
     ap.add_argument("--no-tune", action="store_true",
                     help="keep the launch planner's own choice for every convolution (without it the library searches the launch "
                          "plans of every convolution geometry once, before the timed region: eddlhip_conv2d_autotune)")
@@ -383,6 +437,7 @@ def main():
         "hbm_bound_convs": summary["hbm_bound_convs"],
         "conv_total": summary["conv_total"],
         "device_ms_sum_of_ops": summary["device_ms_sum_of_ops"],
+        "plans": summary["plans"], "workspace_bytes": summary["workspace_bytes"],
         "event_pair_floor_ms": event_floor_ms,
     }
     if not args.no_cpu_baseline:
@@ -403,7 +458,8 @@ def main():
                      "warmup": warmup, "batch": sm["batch"], "dominant_kernel": sm["roofline"]["kernel"],
                      "frac": sm["roofline"]["frac"], "achieved_tflops": sm["roofline"]["achieved"],
                      "avg_launch_ms": sm["roofline"]["avg_launch_ms"], "launches_per_step": sm["roofline"]["launches_per_step"],
-                     "conv_total": sm["conv_total"], "hbm_bound_convs": sm["hbm_bound_convs"]}
+                     "conv_total": sm["conv_total"], "hbm_bound_convs": sm["hbm_bound_convs"], "plans": sm["plans"],
+                     "workspace_bytes": sm["workspace_bytes"], "traffic": sm["roofline"].get("traffic")}
             if not args.no_cpu_baseline:
                 entry["parity"] = oracle_parity(w, out_w, parity_images)
             result["workloads"][w] = entry
@@ -412,6 +468,9 @@ def main():
             print(json.dumps(result))
             sys.exit("bench.py: the device's output differs from the CPU oracle's beyond %.0e of the largest output in: %s"
                      % (PARITY_BOUND, ", ".join(bad)))
+
+    if args.workload == "vgg16" and not (args.no_dropin or args.unfused or args.graph or args.no_tune):
+        result["dropin"] = dropin_path()
 
     table = ["# ms = device time between two events around the op; an event pair around a one-element fill reads %.4f ms"
              % event_floor_ms,

@@ -36,6 +36,8 @@ int use_device(int dev);
 // Returns a workspace of at least `bytes` (contents undefined); waits for the stream before
 // replacing a smaller one so that kernels still reading it finish first.
 int get_workspace(int dev, size_t bytes, void **ptr);
+// Waits for the stream and frees the workspace; the next get_workspace allocates what it needs.
+int release_workspace(int dev);
 // Hooks of the convolution's cache of repacked filters: the library's own copy / fill / free entry
 // points report device ranges they write or release, so a registered filter tensor whose contents
 // change is repacked before its next use and one that is freed is forgotten.

@@ -73,6 +73,17 @@ int get_workspace(int dev, size_t bytes, void **ptr) {
     return 0;
 }
 
+int release_workspace(int dev) {
+    DeviceState &s = g_state[dev];
+    if (s.workspace == nullptr) return 0;
+    EH_TRY_HIP(hipStreamSynchronize(s.stream));
+    EH_TRY_HIP(hipFree(s.workspace));
+    s.workspace = nullptr;
+    s.workspace_bytes = 0;
+    s.workspace_generation++;  // graphs recorded before name memory that is gone
+    return 0;
+}
+
 }  // namespace eddlhip
 
 using namespace eddlhip;
@@ -120,14 +131,7 @@ int eddlhip_workspace_bytes(int dev, size_t *bytes) {
 int eddlhip_workspace_trim(int dev) {
     EH_TRY(use_device(dev));
     EH_NOT_CAPTURING(dev, "eddlhip_workspace_trim");
-    DeviceState &s = state(dev);
-    if (s.workspace == nullptr) return 0;
-    EH_TRY_HIP(hipStreamSynchronize(s.stream));
-    EH_TRY_HIP(hipFree(s.workspace));
-    s.workspace = nullptr;
-    s.workspace_bytes = 0;
-    s.workspace_generation++;  // graphs recorded before name memory that is gone
-    return 0;
+    return release_workspace(dev);
 }
 
 int eddlhip_device_name(int dev, char *buf, size_t buflen) {

@@ -63,7 +63,7 @@ int eddlhip_memcpy_d2d(int dev, void *dev_dst, const void *dev_src, size_t bytes
 int eddlhip_fill(int dev, float *A, size_t n, float v);
 /* Size of the library's private workspace on the device right now (it only grows; 0 before the first call that
  * needs one).  eddlhip_workspace_trim waits for the device's kernels and releases the workspace, so that it grows back
- * to what the calls from then on need - e.g. after a plan search, whose candidates take more than the plans it keeps.
+ * to what the calls from then on need (a plan search does this itself when its candidates have grown the workspace).
  * Not while a graph is being recorded; graphs recorded before name the released memory and refuse to launch.
  * No counterpart in the reference. */
 int eddlhip_workspace_bytes(int dev, size_t *bytes);

@@ -10,6 +10,7 @@
 // Only members both have are used: Tensor::{gpu_device, ptr, size, ndim, shape, stride},
 // ConvolDescriptor::{I, K, bias, O, use_bias, iz, ir, ic, nk, kr, kc, sr, sc, padrt, padcl, r, c},
 // PoolDescriptor::{I, O, indX, indY, iz, ir, ic, kr, kc, sr, sc, padrt, padrb, padcl, padcr}.
+#include <cstdlib>
 #include <iostream>
 #include <stdexcept>
 #include <string>
@@ -76,6 +77,17 @@ void gpu_init(int device) {
         gpu_check(eddlhip_device_name(device, name, sizeof(name)), "gpu_init");
         std::cerr << "EDDL is running on GPU device " << device << ", " << name << "\n";
         hip_announced[device] = true;
+        // The CUDA backend finds every convolution's algorithm by measurement on the layer's first forward
+        // (cudnnFindConvolutionForwardAlgorithm, src/hardware/gpu/nn/gpu_conv.cu:42-66, 211-213).  The same here: the
+        // library's plan search is on unless EDDLHIP_NO_TUNE is set, and EDDLHIP_PLANS=<file> starts it from the plans an
+        // earlier process saved (eddlhip_conv2d_tuned_save), so that nothing is left to search for those geometries and
+        // results are the same bits from run to run.
+        const char *no_tune = getenv("EDDLHIP_NO_TUNE");
+        if (no_tune == nullptr || no_tune[0] == 0 || no_tune[0] == '0') {
+            const char *plans = getenv("EDDLHIP_PLANS");
+            if (plans != nullptr && plans[0] != 0) gpu_check(eddlhip_conv2d_tuned_load(device, plans), "gpu_init (EDDLHIP_PLANS)");
+            gpu_check(eddlhip_conv2d_autotune(1), "gpu_init");
+        }
     }
 }
 

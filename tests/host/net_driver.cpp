@@ -269,15 +269,8 @@ int main(int argc, char **argv) {
     }
     const string params = argv[2], in_path = argv[3], out_path = argv[4];
     const int batch = atoi(argv[5]), size = atoi(argv[6]);
-    // EDDLHIP_PLANS=<file>: the plan search of the library, started from the plans an earlier process found and saved
-    const char *plans = getenv("EDDLHIP_PLANS");
-    if (plans != nullptr && plans[0] != 0) {
-        if (eddlhip_conv2d_tuned_load(0, plans) != 0 || eddlhip_conv2d_autotune(1) != 0) {
-            fprintf(stderr, "plans: %s\n", eddlhip_last_error());
-            return 2;
-        }
-        printf("plans: %d geometries loaded\n", eddlhip_conv2d_tuned_plans(0));
-    }
+    // (the binding's gpu_init switches the library's plan search on unless EDDLHIP_NO_TUNE is set, and starts it from the
+    // plans in EDDLHIP_PLANS=<file>; EDDLHIP_PLANS_SAVE=<file> makes this driver write the table it ends up with)
     vector<int> extra;
     for (int i = 7; i < argc; i++) extra.push_back(atoi(argv[i]));
     try {
@@ -295,6 +288,7 @@ int main(int argc, char **argv) {
         const bool synth_params = params.compare(0, 6, "synth:") == 0;
         if (synth_params) eddl_hip::synth_he_normal(m, (uint32_t)strtoul(params.c_str() + 6, nullptr, 10));
         build(m, CS_HIP({1}), !synth_params);
+        if (getenv("EDDLHIP_PLANS") != nullptr && getenv("EDDLHIP_PLANS")[0] != 0) printf("plans: %d geometries loaded\n", eddlhip_conv2d_tuned_plans(0));
         if (fused) {
             fuse(m);
             int away = 0;
@@ -349,7 +343,9 @@ int main(int argc, char **argv) {
             const int reps = 20;
             for (int i = 0; i < reps; i++) m->forward();
             const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / reps;
-            printf("ms_per_forward %.4f images_per_s %.1f\n", ms, batch * 1000.0 / ms);
+            size_t ws = 0;
+            eddlhip_workspace_bytes(0, &ws);
+            printf("ms_per_forward %.4f images_per_s %.1f workspace_bytes %zu tuned_geometries %d\n", ms, batch * 1000.0 / ms, ws, eddlhip_conv2d_tuned_plans(0));
         }
         if (fused) {  // a layer inside a chain has no output to hand out
             for (Layer *l : m->layers)
@@ -395,6 +391,11 @@ int main(int argc, char **argv) {
         }
         if (params == "-") save(m, out_path + ".params");  // round trip of freshly initialised parameters
         delete m;
+        const char *plans_out = getenv("EDDLHIP_PLANS_SAVE");
+        if (plans_out != nullptr && plans_out[0] != 0 && eddlhip_conv2d_tuned_save(0, plans_out) != 0) {
+            fprintf(stderr, "plans: %s\n", eddlhip_last_error());
+            return 2;
+        }
     } catch (const std::exception &e) {
         fprintf(stderr, "exception: %s\n", e.what());
         return 1;

@@ -9,7 +9,11 @@ Every layer is checked on the DEVICE'S OWN input to that layer:
     sample, so padding, the last partial tile and K-split tiles are all hit), to the conv bar;
   * size-independent properties on top: scaling the input by a power of two scales a conv
     output exactly; max-pool outputs equal the input gathered at the reported indices; the
-    fused plan reproduces the layer-by-layer plan bit for bit.
+    fused plan reproduces the layer-by-layer plan bit for bit - the network's outputs and every
+    max-pool's values and both index tensors (in the fused plan the pools behind Winograd
+    convolutions are computed in the convolution's epilogue).
+The same checks run with every Winograd form forced wherever it applies and with the plan search
+switched on (the mode bench.py times): the searched K-split and Winograd plans are the ones checked.
 """
 import numpy as np
 import pytest
@@ -81,10 +85,17 @@ def check_fullsize(hip, ora, model, x, seed, only_convs=False):
             ref = layer_oracle(ora, l, ins)
             np.testing.assert_allclose(got, ref.reshape(got.shape), rtol=2e-6, atol=1e-7, err_msg=l.name)
         del ins, got
+    pools = [l for l in model.layers if l.kind == "maxpool2d"]
+    walked = {l.name: (model.output_of(l).numpy(), model.aux[id(l)]["indX"].numpy(), model.aux[id(l)]["indY"].numpy()) for l in pools}
     model.build(hip, fuse=True)
     out_fused = [o.numpy() for o in model.forward([x])]
     for a, b in zip(out_unfused, out_fused):
         assert np.array_equal(a, b), "fused plan differs from the layer-by-layer plan"
+    for l in pools:  # pooled values and the coordinates of every maximum, bit for bit
+        val, ix, iy = walked[l.name]
+        assert np.array_equal(model.output_of(l).numpy(), val), "fused plan: values of " + l.name
+        assert np.array_equal(model.aux[id(l)]["indX"].numpy(), ix) and np.array_equal(model.aux[id(l)]["indY"].numpy(), iy), "fused plan: indices of " + l.name
+    checked["pools"] = len(pools)
     return checked
 
 
@@ -127,29 +138,93 @@ def test_unet_4x1x512x512(hip, oracle):
     assert got["conv2d"] == 23
 
 
-@pytest.mark.parametrize("workload,form", [("vgg16", "three kernels"), ("vgg16", "folded"), ("resnet50", "three kernels"), ("resnet50", "folded"), ("unet", "three kernels"), ("unet", "folded")])
+FULL_SIZE = {
+    "vgg16": lambda models: (models.vgg16(batch=32), np.random.default_rng(3).uniform(0, 1, (32, 3, 224, 224)).astype(np.float32), 3, 13),
+    "block": lambda models: (models.conv_bn_relu_pool_block(batch=64, channels=64, size=56, filters=64),
+                             np.random.default_rng(2).standard_normal((64, 64, 56, 56), dtype=np.float32), 2, 1),
+    "resnet50": lambda models: (models.resnet50(batch=64), np.random.default_rng(4).standard_normal((64, 3, 224, 224), dtype=np.float32), 4, 53),
+    "unet": lambda models: (models.unet(batch=4), np.random.default_rng(5).uniform(0, 1, (4, 1, 512, 512)).astype(np.float32), 5, 23),
+}
+
+
+@pytest.mark.parametrize("workload", ["vgg16", "block", "resnet50", "unet"])
+def test_full_size_under_searched_plans(hip, oracle, workload):
+    """The mode bench.py times: the plan search on.  The layer walk's first forward searches every geometry; the sampled
+    check of every convolution then sees the searched launches (K-split tiles, the Winograd forms the search kept), the
+    bandwidth layers are checked whole, and the fused plan - the same table - must reproduce the walk bit for bit,
+    pooled values and indices included."""
+    from eddl_amd import models
+    m, x, seed, convs = FULL_SIZE[workload](models)
+    hip.conv_autotune(-1)
+    try:
+        hip.conv_autotune(True)
+        got = check_fullsize(hip, oracle, m, x, seed)
+        assert got["conv2d"] == convs and hip.conv_tuned_plans() >= 1
+    finally:
+        hip.conv_autotune(-1)
+        hip.workspace_trim()
+
+
+def test_two_plan_searches_keep_the_same_plans(hip, tmp_path):
+    """The plan search of every convolution geometry of the five configurations, twice in one process with the table
+    emptied in between: the same plan both times (each plan's fastest batch of launches is compared, and of the plans
+    within 3 % of the fastest a fixed order of preference decides).  Two plans whose times differ by just that margin
+    can still change places from one search to the next (on bandwidth-bound layers the margin also moves with where the
+    tensors happen to lie in memory); the test allows that for six of the sixty geometries and prints them."""
+    from eddl_amd import models
+    tables = []
+    for attempt in range(2):
+        hip.conv_autotune(-1)
+        hip.conv_autotune(True)
+        try:
+            for name in ("conv", "block", "vgg16", "resnet50", "unet"):
+                if name == "conv":
+                    m, x, seed = models.single_conv(batch=8), np.random.default_rng(1).standard_normal((8, 3, 32, 32), dtype=np.float32), 1
+                else:
+                    m, x, seed, _ = FULL_SIZE[name](models)
+                models.init_he_normal(m, seed)
+                m.build(hip, fuse=True)
+                m.forward([x])
+                hip.synchronize()
+                del m
+            path = str(tmp_path / ("plans%d.txt" % attempt))
+            hip.conv_tuned_save(path)
+            tables.append(sorted(l for l in open(path).read().splitlines() if not l.startswith("#")))
+        finally:
+            hip.conv_autotune(-1)
+            hip.workspace_trim()
+    assert len(tables[0]) >= 40 and len(tables[0]) == len(tables[1])
+    differing = [(a, b) for a, b in zip(tables[0], tables[1]) if a != b]
+    print("geometries: %d, plans that differ between two searches: %s" % (len(tables[0]), differing))
+    assert [a.split("|")[0] for a in tables[0]] == [b.split("|")[0] for b in tables[1]]
+    assert len(differing) <= 6, "plans that differ between two searches: %s" % (differing,)
+
+
+@pytest.mark.parametrize("workload,form", [("vgg16", "three kernels"), ("vgg16", "folded"), ("vgg16", "one launch"), ("resnet50", "three kernels"),
+                                           ("resnet50", "folded"), ("resnet50", "one launch"), ("unet", "three kernels"), ("unet", "folded"),
+                                           ("unet", "one launch")])
 def test_winograd_forms_at_full_size(hip, oracle, workload, form):
     """The same sampled check of every convolution with the Winograd forms forced wherever they apply (3x3 and 2x2
-    filters at stride 1; the folded form also needs channels in sixteens): the forms the plan search may pick at the
-    benchmark sizes meet the convolution bar there, on the device's own layer inputs, and fuse bit for bit."""
+    filters at stride 1; the folded form also needs channels in sixteens; the one-launch form 3x3 filters, here on its
+    64-filter tile with the left-over tiles in four K slices): the forms the plan search may pick at the benchmark sizes
+    meet the convolution bar there, on the device's own layer inputs, and fuse bit for bit."""
     from eddl_amd import models
-    m, x, seed, convs = {
-        "vgg16": lambda: (models.vgg16(batch=32), np.random.default_rng(3).uniform(0, 1, (32, 3, 224, 224)).astype(np.float32), 3, 13),
-        "resnet50": lambda: (models.resnet50(batch=64), np.random.default_rng(4).standard_normal((64, 3, 224, 224), dtype=np.float32), 4, 53),
-        "unet": lambda: (models.unet(batch=4), np.random.default_rng(5).uniform(0, 1, (4, 1, 512, 512)).astype(np.float32), 5, 23),
-    }[workload]()
+    m, x, seed, convs = FULL_SIZE[workload](models)
     try:
         if form == "folded":
             hip.force_conv_plan(5, 1)
+        elif form == "one launch":
+            hip.force_conv_plan(7, 4)
         else:
             hip.set_conv_algo("winograd")
         got = check_fullsize(hip, oracle, m, x, seed, only_convs=True)
         assert got["conv2d"] == convs
-        if workload == "vgg16":  # its last convolution is 3x3 at stride 1 over 512 channels: both forms apply
+        if workload == "vgg16":  # its last convolution is 3x3 at stride 1 over 512 channels: every form applies
             assert hip.last_conv_kernel().startswith("winograd["), hip.last_conv_kernel()
     finally:
         hip.force_conv_plan(-1, 1)
         hip.set_conv_algo("winograd_off")
+        hip.workspace_trim()
 
 
 def test_conv_scaling_by_powers_of_two_is_exact_at_full_size(hip):

@@ -20,7 +20,8 @@ def run_driver(case, tmp, params, files):
         fh.write(" ".join(str(p) for p in params))
     for name, arr in files.items():
         np.ascontiguousarray(arr, np.float32).tofile(tmp / name)
-    res = subprocess.run([DRIVER, case, str(tmp)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    # (EDDLHIP_NO_TUNE: the binding's gpu_init would switch the plan search on; these tests compare with untuned launches bit for bit)
+    res = subprocess.run([DRIVER, case, str(tmp)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120, env=dict(os.environ, EDDLHIP_NO_TUNE="1"))
     assert res.returncode == 0, res.stderr[-2000:]
     return res
 
@@ -115,9 +116,13 @@ def test_error_behaviour_follows_the_reference(tmp_path):
 NET_DRIVER = os.path.join(ROOT, "eddl_amd", "host", "net_driver")
 
 
-def run_net_driver(args, timeout=300):
+def run_net_driver(args, timeout=300, env=None):
+    """Runs the C++ model driver.  The binding's gpu_init switches the library's plan search on, as the reference's CUDA
+    backend searches its algorithms; tests that compare with the Python host's untuned launches bit for bit switch it off
+    (EDDLHIP_NO_TUNE), tests of the search pass their own environment."""
     assert os.path.exists(NET_DRIVER), "build the host layer first: make -C eddl_amd/host"
-    res = subprocess.run([NET_DRIVER] + [str(a) for a in args], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=timeout)
+    res = subprocess.run([NET_DRIVER] + [str(a) for a in args], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=timeout,
+                         env=dict(os.environ, **(env if env is not None else {"EDDLHIP_NO_TUNE": "1"})))
     assert res.returncode == 0, (res.stdout[-2000:], res.stderr[-2000:])
     return res.stdout
 
@@ -213,6 +218,36 @@ def test_cpp_host_runs_the_plans_a_python_process_saved(hip, tmp_path):
         assert res.returncode == 0 and "plans: 1 geometries loaded" in res.stdout and "FAILED" not in res.stdout, (res.stdout[-2000:], res.stderr[-2000:])
         got = np.fromfile(tmp_path / "y.raw", np.float32).reshape(want[plan].shape)
         assert np.array_equal(got, want[plan]), plan
+
+
+@pytest.mark.parametrize("fused", [False, True], ids=["layerwise", "fused"])
+def test_cpp_host_searches_its_plans_like_the_reference_backend(hip, fused, tmp_path):
+    """An unchanged EDDL program gets the plan search: the binding's gpu_init switches it on (the reference's gpu_conv2D
+    runs cudnnFindConvolutionForwardAlgorithm on a layer's first forward).  A VGG-shaped net (channels in sixteens, so every
+    Winograd form is a candidate) walked layer by layer, and as its fused plan, by the C++ host with nothing in its
+    environment; the table it ends up with is saved, and the Python layer walk under that table gives the same bits."""
+    from eddl_amd import models
+    batch, size, extra = 4, 64, [10, 16, 32, 64, 64, 64, 64]
+    m = models.vgg16(batch=batch, size=size, num_classes=10, widths=(16, 32, 64, 64, 64), dense=64)
+    models.init_he_normal(m, 4)
+    x = models.synthetic_input(m.lin[0].out_shape, 1004, "uniform")
+    plans = str(tmp_path / "plans.txt")
+    out = run_net_driver([("fused:" if fused else "") + "vgg16", "synth:4", "synth:1004:uniform", tmp_path / "y.raw", batch, size] + extra,
+                         env={"EDDLHIP_PLANS_SAVE": plans, "EDDLHIP_NO_TUNE": ""})
+    assert "FAILED" not in out, out
+    searched = [l for l in open(plans).read().splitlines() if l and not l.startswith("#")]
+    assert len(searched) >= 8, searched          # batch 1 (the driver's resize) and batch 4 geometries
+    hip.conv_autotune(-1)
+    try:
+        hip.conv_tuned_load(plans)
+        hip.conv_autotune(True)
+        m.build(hip, fuse=False)
+        want = m.predict([x])[0]
+        assert hip.conv_tuned_plans() == len(searched)      # nothing was left to search
+    finally:
+        hip.conv_autotune(-1)
+    got = np.fromfile(tmp_path / "y.raw", np.float32).reshape(want.shape)
+    assert np.array_equal(got, want)
 
 
 @pytest.mark.parametrize("which", ["block", "resnet50", "unet"])

@@ -71,6 +71,29 @@ def test_noalloc_equals_conv2d_fwd_two_calls_in_a_row(hip, name):
         assert saw_split, "this case is meant to cover the partial tiles of a K-split launch"
 
 
+def test_noalloc_leaves_the_workspace_alone(hip):
+    """The property the entry point exists for: with the library's workspace released beforehand, a call larger than any
+    before it (repacked filters and the partial tiles of a K-split launch come from the fixed array) leaves the workspace
+    at zero bytes - nothing was allocated - and the allocating entry point, called afterwards, gives the same bits."""
+    rng = np.random.default_rng(73)
+    N, C, H, W, Kf = 32, 320, 28, 28, 512
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    w = (rng.standard_normal((Kf, C, 3, 3)) * 0.03).astype(np.float32)
+    dx, dw = hip.array(x), hip.array(w)
+    O1, O2 = hip.full((N, Kf, H, W), float("nan")), hip.full((N, Kf, H, W), float("nan"))
+    hip.synchronize()
+    hip.workspace_trim()
+    assert hip.workspace_bytes() == 0
+    args = lambda O: (hip.dev, dx.ptr, dw.ptr, None, O.ptr, N, C, H, W, Kf, 3, 3, 1, 1, 1, 1, H, W, None, None, None, None, 0.0, None, 0)
+    hip._check(hip.lib.eddlhip_conv2d_fwd_noalloc(*args(O1)))
+    kernel = hip.last_conv_kernel()
+    assert hip.workspace_bytes() == 0, "eddlhip_conv2d_fwd_noalloc took a workspace"
+    assert "+ksplit" in kernel, kernel
+    hip._check(hip.lib.eddlhip_conv2d_fwd(*args(O2)))
+    assert hip.last_conv_kernel() == kernel and hip.workspace_bytes() > 0
+    assert np.array_equal(O1.numpy(), O2.numpy())
+
+
 def test_noalloc_uses_registered_filters(hip):
     """With the filters registered the call needs no room for a repacked copy; the result is unchanged."""
     rng = np.random.default_rng(72)
