@@ -47,8 +47,6 @@ PROTOTYPES = {
     "eddlhip_graph_end": [c_int, ctypes.POINTER(c_void_p)],
     "eddlhip_graph_launch": [c_int, c_void_p],
     "eddlhip_graph_destroy": [c_int, c_void_p],
-    "eddlhip_probe_mfma_f32": [c_int, c_int, c_int, ctypes.POINTER(c_float), ctypes.POINTER(c_float), ctypes.POINTER(c_float)],
-    "eddlhip_probe_hbm": [c_int, c_size_t, ctypes.POINTER(c_float), ctypes.POINTER(c_float), ctypes.POINTER(c_float)],
     "eddlhip_conv2d_fwd": [c_int, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_fwd_noalloc": [c_int, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
     "eddlhip_conv2d_fwd_concat": [c_int, P, P, P, P, P] + [c_int] * 13 + [P, P, P, P, c_float, P, c_int],
@@ -91,6 +89,27 @@ PROTOTYPES = {
 }
 _RESTYPE = {"eddlhip_version": ctypes.c_char_p, "eddlhip_last_error": ctypes.c_char_p,
             "eddlhip_conv2d_last_kernel": ctypes.c_char_p}
+
+
+# include/eddlhip_probe.h: the benchmark's device probes, in libeddlhip_probe.so
+PROBE_PROTOTYPES = {
+    "eddlhip_probe_mfma_f32": [c_int, c_int, c_int, ctypes.POINTER(c_float), ctypes.POINTER(c_float), ctypes.POINTER(c_float)],
+    "eddlhip_probe_hbm": [c_int, c_size_t, ctypes.POINTER(c_float), ctypes.POINTER(c_float), ctypes.POINTER(c_float)],
+}
+PROBE_LIB_PATH = os.path.join(os.path.dirname(LIB_PATH), "libeddlhip_probe.so")
+
+
+def load_probe():
+    """The probe library (loads libeddlhip.so, which it is linked against, through its run path)."""
+    if not os.path.exists(PROBE_LIB_PATH):
+        raise ImportError("%s is missing: build it with `python -m eddl_amd.build` (hipcc, gfx950)." % PROBE_LIB_PATH)
+    ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    lib = ctypes.CDLL(PROBE_LIB_PATH)
+    for name, args in PROBE_PROTOTYPES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = c_int
+    return lib
 
 
 def load():

@@ -222,10 +222,17 @@ class Backend:
     def download_wait(self, event):
         self._check(self.lib.eddlhip_download_wait_event(self.dev, event.handle))
 
+    def _probe_lib(self):
+        """The device probes live in a library of their own (libeddlhip_probe.so), loaded on first use."""
+        if getattr(self, "_probe", None) is None:
+            from . import _lib
+            self._probe = _lib.load_probe()
+        return self._probe
+
     def probe_mfma_f32(self, vary_operands=True, launches=40):
         """Sustained fp32 MFMA rate of the device with nothing else running: (mean, best launch, worst launch) TFLOP/s."""
         mean, best, worst = ctypes.c_float(), ctypes.c_float(), ctypes.c_float()
-        self._check(self.lib.eddlhip_probe_mfma_f32(self.dev, int(vary_operands), launches, ctypes.byref(mean), ctypes.byref(best),
+        self._check(self._probe_lib().eddlhip_probe_mfma_f32(self.dev, int(vary_operands), launches, ctypes.byref(mean), ctypes.byref(best),
                                                     ctypes.byref(worst)))
         return mean.value, best.value, worst.value
 
@@ -233,7 +240,7 @@ class Backend:
         """What plain streams over device memory sustain with nothing else running: (read, write, copy) GB/s over
         two buffers of ``nbytes`` each; copy counts bytes read plus bytes written."""
         r, w, c = ctypes.c_float(), ctypes.c_float(), ctypes.c_float()
-        self._check(self.lib.eddlhip_probe_hbm(self.dev, int(nbytes), ctypes.byref(r), ctypes.byref(w), ctypes.byref(c)))
+        self._check(self._probe_lib().eddlhip_probe_hbm(self.dev, int(nbytes), ctypes.byref(r), ctypes.byref(w), ctypes.byref(c)))
         return r.value, w.value, c.value
 
     def empty(self, shape):

@@ -5,8 +5,11 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["runtime.hip", "elementwise.hip", "pool.hip", "conv.hip", "dense.hip", "generator.hip", "probe.hip"]
+SOURCES = ["runtime.hip", "elementwise.hip", "pool.hip", "conv.hip", "dense.hip", "generator.hip"]
 LIB = os.path.join(HERE, "libeddlhip.so")
+# the benchmark's device probes: a library of their own beside the C ABI (include/eddlhip_probe.h)
+PROBE_SOURCES = ["probe.hip"]
+PROBE_LIB = os.path.join(HERE, "libeddlhip_probe.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -17,9 +20,7 @@ HIPCC_FLAGS = [
 ]
 
 
-def build(verbose=False):
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB]
+def _compile(cmd, verbose):
     if verbose:
         print(" ".join(cmd))
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -29,6 +30,12 @@ def build(verbose=False):
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
+
+
+def build(verbose=False):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    _compile([hipcc] + HIPCC_FLAGS + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB], verbose)
+    _compile([hipcc] + HIPCC_FLAGS + [os.path.join(CSRC, s) for s in PROBE_SOURCES] + ["-L" + HERE, "-leddlhip", "-Wl,-rpath,$ORIGIN", "-o", PROBE_LIB], verbose)
     return LIB
 
 

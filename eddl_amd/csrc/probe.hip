@@ -5,6 +5,7 @@
 // clock, and the sustained rate is what a kernel can be measured against.  Not part of the
 // reference's interface; the benchmark reports it beside the published peak.
 #include "common.h"
+#include "../../include/eddlhip_probe.h"
 
 using namespace eddlhip;
 

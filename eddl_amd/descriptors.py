@@ -92,6 +92,11 @@ class ConvolDescriptor:
         self.in_, self.iz, self.ir, self.ic = in_shape  # `in` is a Python keyword
         self.z = self.nk
         d0, d1 = self.dilation_rate
+        # (the reference reads these without a check; a graph from a file can hold anything)
+        if min(self.kr, self.kc, self.sr, self.sc, d0, d1) < 1:
+            msg("Kernel sizes, strides and dilations must be positive", "ConvolDescriptor::build")
+        if self.padding == "custom" and len(self.pads) != 4:
+            msg("Custom padding takes four values (top, bottom, left, right), got %d" % len(self.pads), "ConvolDescriptor::build")
         if self.padding == "custom":
             self.r = _out_custom(self.pads[0:2], self.ir, self.kr, self.sr, d0)
             self.c = _out_custom(self.pads[2:4], self.ic, self.kc, self.sc, d1)
@@ -144,6 +149,10 @@ class PoolDescriptor:
         self.sr, self.sc = self.stride
         self.in_, self.iz, self.ir, self.ic = in_shape
         self.z = self.iz
+        if min(self.kr, self.kc, self.sr, self.sc) < 1:
+            msg("Kernel sizes, strides and dilations must be positive", "PoolDescriptor::build")
+        if self.padding == "custom" and len(self.pad) != 4:
+            msg("Custom padding takes four values (top, bottom, left, right), got %d" % len(self.pad), "PoolDescriptor::build")
         if self.padding == "custom":
             # the reference passes the whole 4-vector and reads entries [0] and [1] for BOTH axes
             self.r = _out_custom(self.pad, self.ir, self.kr, self.sr)

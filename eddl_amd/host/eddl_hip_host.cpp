@@ -364,6 +364,9 @@ static WindowGeometry window_geometry(const char *who, const Tensor *A, const st
                                       int sr, int sc, int dil_r, int dil_c, bool custom_cols_read_row_pads) {
     const string where = string(who) + "::build";
     if (A->ndim != 4) msg("Tensors are not 4D", where);
+    // (the reference reads these without a check; a graph from a file can hold anything)
+    if (kr < 1 || kc < 1 || sr < 1 || sc < 1 || dil_r < 1 || dil_c < 1) msg("Kernel sizes, strides and dilations must be positive", where);
+    if (padding == "custom" && pads.size() != 4) msg("Custom padding takes four values (top, bottom, left, right), got " + std::to_string(pads.size()), where);
     const int ir = A->shape[2], ic = A->shape[3];
     WindowGeometry g;
     if (padding == "custom") {

@@ -793,6 +793,11 @@ void Net::load(const string &filename, const string &format) {
             if (!ifs.good() || nd < 0 || nd > 8) msg("the file ends early or is not in the bin format (layer " + l->name + ")", "Net::load");
             vector<int> shape(nd);
             ifs.read(reinterpret_cast<char *>(shape.data()), nd * sizeof(int));
+            // (a record is trusted only as far as it fits the parameter it is for: nothing is allocated from a size the file names)
+            unsigned long long count = ifs.good() ? 1 : 0;
+            for (int d : shape) count = (d > 0 && count <= p->size) ? count * (unsigned long long)d : 0;
+            if (count != p->size)
+                msg("a record of the file does not hold the " + std::to_string(p->size) + " values of a parameter of layer " + l->name, "Net::load");
             Tensor host(shape, DEV_CPU);
             ifs.read(reinterpret_cast<char *>(host.ptr), host.size * sizeof(float));
             if (!ifs.good()) msg("the file ends inside a parameter of layer " + l->name, "Net::load");

@@ -118,21 +118,6 @@ int eddlhip_event_destroy(int dev, void *event);
 int eddlhip_event_record(int dev, void *event);
 int eddlhip_event_elapsed_ms(int dev, void *start, void *stop, float *ms);
 
-/* Device probe: TFLOP/s that v_mfma_f32_32x32x2_f32 sustains with nothing else running, over
- * `launches` back-to-back launches of about 7 ms each (mean, best launch, worst launch).
- * vary_operands == 0: every MFMA reads the same two registers; != 0: operands change from one
- * instruction to the next, as in a real product (the device then lowers its clock at times).
- * No counterpart in the reference; the benchmark reports the result beside the published peak. */
-int eddlhip_probe_mfma_f32(int dev, int vary_operands, int launches, float *tflops_mean, float *tflops_best,
-                           float *tflops_worst);
-/* Device probe: GB/s that plain streams over device memory sustain with nothing else running - read only,
- * write only, and copy (bytes read + bytes written) - over two buffers of `bytes` each that the call
- * allocates and frees (choose them larger than the device's caches: 1 GiB).  16-byte accesses, four in
- * flight per thread or one, with and without the streaming (non-temporal) hint, several grid sizes; the best rate
- * of each kind is returned.  It is what the bandwidth-bound kernels can be measured against beside the
- * published 8 TB/s.  No counterpart in the reference. */
-int eddlhip_probe_hbm(int dev, size_t bytes, float *read_gbs, float *write_gbs, float *copy_gbs);
-
 /* ------------------------------------------------------------------ convolution
  * Replaces gpu_conv2D(ConvolDescriptor*) (src/hardware/gpu/nn/gpu_conv.cu:159-233; CPU
  * semantics src/hardware/cpu/nn/cpu_conv.cpp:55-112,114-226,316-346).

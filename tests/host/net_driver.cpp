@@ -249,8 +249,45 @@ static int onnxinfo(int argc, char **argv) {
     return 0;
 }
 
+// net_driver loadbin <model> <params.bin> <size> [model arguments]: the graph is made but not built (its parameters are
+// host tensors), the file is read into it, and every parameter's size and sum are printed - the bin reader alone, no device.
+static int loadbin(int argc, char **argv) {
+    if (argc < 5) {
+        fprintf(stderr, "usage: net_driver loadbin <model> <params.bin> <size> [model arguments]\n");
+        return 2;
+    }
+    const string which = argv[2];
+    const int size = atoi(argv[4]);
+    vector<int> extra;
+    for (int i = 5; i < argc; i++) extra.push_back(atoi(argv[i]));
+    try {
+        model m = nullptr;
+        if (which == "block") m = block(extra.at(0), size, extra.at(1));
+        else if (which == "vgg16") m = vgg16(size, extra.at(0), {extra.at(1), extra.at(2), extra.at(3), extra.at(4), extra.at(5)}, extra.at(6));
+        else if (which == "resnet50") m = resnet50(size, extra.at(0), extra.at(1));
+        else if (which == "unet") m = unet(size, vector<int>(extra.begin(), extra.end() - 1), extra.back());
+        else {
+            fprintf(stderr, "unknown model %s\n", which.c_str());
+            return 2;
+        }
+        load(m, argv[3]);
+        for (Layer *l : m->layers)
+            for (Tensor *t : l->params) {
+                double sum = 0.0;
+                for (unsigned long i = 0; i < t->size; i++) sum += t->ptr[i];
+                printf("param %s %lu %.9g\n", l->name.c_str(), t->size, sum);
+            }
+        delete m;
+    } catch (const std::exception &e) {
+        fprintf(stderr, "exception: %s\n", e.what());
+        return 1;
+    }
+    return 0;
+}
+
 int main(int argc, char **argv) {
     if (argc >= 2 && !strcmp(argv[1], "errors")) return errors();
+    if (argc >= 2 && !strcmp(argv[1], "loadbin")) return loadbin(argc, argv);
     if (argc >= 2 && !strcmp(argv[1], "onnxinfo")) return onnxinfo(argc, argv);
     if (argc >= 2 && !strcmp(argv[1], "onnx")) return onnx(argc, argv);
     if (argc < 7) {

@@ -9,8 +9,8 @@ import pytest
 from conftest import ROOT
 
 
-def _declared_functions():
-    src = open(os.path.join(ROOT, "include", "eddlhip.h")).read()
+def _declared_functions(header="eddlhip.h"):
+    src = open(os.path.join(ROOT, "include", header)).read()
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
     return sorted(set(re.findall(r"\b(eddlhip_\w+)\s*\(", src)))
 
@@ -23,6 +23,11 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), "libeddlhip.so lacks %s" % n
     assert set(names) == set(_lib.PROTOTYPES), "ctypes prototypes out of step with include/eddlhip.h"
+    # the benchmark's device probes: a library and a header of their own, outside the drop-in boundary
+    probe = _lib.load_probe()
+    probes = _declared_functions("eddlhip_probe.h")
+    assert probes == sorted(_lib.PROBE_PROTOTYPES) and all(hasattr(probe, n) for n in probes)
+    assert not any(hasattr(lib, n) for n in probes), "the probes are meant to stay out of libeddlhip.so"
 
 
 def test_version_and_argument_errors_without_a_device():
