@@ -1683,6 +1683,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
             const int u = wave + 4 * j;
             lds_dma_b128(dma_w, us + u * 256, a_voff, (step * (CK * 16) + u * RPI) * p.Mp * 4);
         }
+        // one input tensor and every channel of the step exists (nearly every step of every layer): nothing is selected
+        if (!checked && p.Csplit == p.C) {
+#pragma unroll
+            for (int jc = 0; jc < CK / 4; jc++) {
+                const int cl = wave + 4 * jc;
+                const int soff = (step * CK + cl) * HW4;
+#pragma unroll
+                for (int k = 0; k < WLC; k++)
+                    if (k < nload) lds_dma_b32(dma_in, rs + cl * SLOTS + k * 64, voff[k], soff);
+            }
+            return;
+        }
 #pragma unroll
         for (int jc = 0; jc < CK / 4; jc++) {
             const int cl = wave + 4 * jc, c = step * CK + cl;
@@ -1707,7 +1719,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 
     // position row i = wave: patch rows ra and rb, combined as d[ra] + d[rb] (i = 1) or d[ra] - d[rb]
     const int ra = wave == 0 ? 0 : (wave == 2 ? 2 : 1), rb = wave == 0 ? 2 : (wave == 1 ? 2 : (wave == 2 ? 1 : 3));
-    const unsigned sgn = wave == 1 ? 0u : 0x80000000u;
+    const float sgn = wave == 1 ? 1.0f : -1.0f;
     const int a_off = (half * 16 + 4 * wave) * MF + l32;
     int ra_off[FN], rb_off[FN];  // this lane's two patch rows, as LDS offsets within a step's pixels (channel `half` of a pair)
 #pragma unroll
@@ -1744,7 +1756,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
         for (int fn = 0; fn < FN; fn++) {
             float u[4];
 #pragma unroll
-            for (int s = 0; s < 4; s++) u[s] = __fadd_rn(d[0][s][fn], __builtin_bit_cast(float, __builtin_bit_cast(unsigned, d[1][s][fn]) ^ sgn));
+            for (int s = 0; s < 4; s++) u[s] = __builtin_fmaf(d[1][s][fn], sgn, d[0][s][fn]);  // d[ra] + d[rb] or d[ra] - d[rb]: one rounding either way
             vv[into][0][fn] = __fsub_rn(u[0], u[2]);
             vv[into][1][fn] = __fadd_rn(u[1], u[2]);
             vv[into][2][fn] = __fsub_rn(u[2], u[1]);
