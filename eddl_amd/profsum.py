@@ -93,14 +93,14 @@ def trace(workload, trace_dir, log, out, extra=""):
     bench = bench_line(log)
     o = ["rocprofv3 kernel trace of the %s benchmark (MI355X, gfx950)%s" % (workload, ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root):",
-         "  rocprofv3 --kernel-trace --stats --output-format csv -d %s -o %s -- python3 bench.py --workload %s --steps 10 --warmup 3 --no-cpu-baseline --no-device-probe --no-workloads --plans gpurun_out/plans_WLTOKEN.txt%s > %s"
+         "  rocprofv3 --kernel-trace --stats --output-format csv -d %s -o %s -- python3 bench.py --workload %s --steps 10 --warmup 3 --no-cpu-baseline --no-device-probe --no-workloads --no-dropin --plans gpurun_out/plans_WLTOKEN.txt%s > %s"
          % (trace_dir, workload, workload, extra, log),
          "  python3 -m eddl_amd.profsum trace %s %s %s %s" % (workload, trace_dir, log, out),
          "",
          "columns: rocprofv3's own *_kernel_stats.csv, unchanged: Name, Calls, TotalDurationNs, AverageNs (= TotalDurationNs / Calls),",
          "Percentage (= TotalDurationNs / sum of TotalDurationNs over all kernels x 100).  The run holds 3 warm-up + 10 timed steps and",
          "the repetitions bench.py uses to time the dominant kernel with HIP events.  The plans file comes from an earlier, unprofiled run",
-         "of the same workload (python3 bench.py --workload W --steps 3 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads",
+         "of the same workload (python3 bench.py --workload W --steps 3 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --no-dropin",
          "--plans gpurun_out/plans_W.txt), which searched the launch plans and saved what it found: the profiled run loads them and",
          "launches no search, so the trace holds the workload only, under the plans a default bench.py run uses.",
          "",
@@ -129,7 +129,7 @@ def traffic(workload, trace_dir, fetch_dir, write_dir, log, out, out_json=None, 
         raise SystemExit("the counter runs hold no copy probe: run bench.py with --copy-probe")
     sf, sw = COPY_PROBE_KIB / max(f[probe[0]]), COPY_PROBE_KIB / max(w[probe[0]])
     bench = bench_line(log)
-    args = "--workload %s%s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --plans gpurun_out/plans_WLTOKEN.txt --copy-probe" % (workload, extra)
+    args = "--workload %s%s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --no-dropin --plans gpurun_out/plans_WLTOKEN.txt --copy-probe" % (workload, extra)
     o = ["HBM traffic per launch of the %s benchmark kernels%s (MI355X, gfx950)%s"
          % (workload, " run layer by layer" if "--unfused" in extra else "", ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root; one counter per run):",
@@ -174,8 +174,16 @@ def traffic(workload, trace_dir, fetch_dir, write_dir, log, out, out_json=None, 
         for k, (b, calls, fb, wb) in per_kernel.items():
             name = short(k, 10 ** 6).split("(")[0].replace(" ", "")
             table[name] = {"hbm_bytes_per_launch": b, "fetch_bytes_per_launch": fb, "write_bytes_per_launch": wb, "launches_in_counter_run": calls}
+        # forwards in the counter run (warm-up, timed steps, bench.py's per-op timing passes): the dominant kernel's dispatches
+        # over its launches per forward
+        steps = None
+        if bench and bench["roofline"].get("launches_per_step"):
+            dom = bench["roofline"]["kernel"].replace(" ", "")
+            hit = [v for k, v in table.items() if k.replace(",false>", ">") == dom]
+            if hit:
+                steps = hit[0]["launches_in_counter_run"] / bench["roofline"]["launches_per_step"]
         with open(out_json, "w") as fh:
-            json.dump({"kernels": table, "fetch_scale": sf, "write_scale": sw, "steps_in_counter_run": 3,
+            json.dump({"kernels": table, "fetch_scale": sf, "write_scale": sw, "steps_in_counter_run": steps,
                        "dominant_kernel_of_that_run": bench["roofline"]["kernel"] if bench else None,
                        "launches_per_step_of_it": bench["roofline"].get("launches_per_step") if bench else None, "source": out, "commit": commit()}, fh, indent=1)
             fh.write("\n")
@@ -189,7 +197,7 @@ def mfma(workload, directory, out):
     dur = durations(directory)
     o = ["Matrix-core counters of the %s benchmark kernels (MI355X, gfx950)%s" % (workload, ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root):",
-         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-workloads --plans gpurun_out/plans_WLTOKEN.txt"
+         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-workloads --no-dropin --plans gpurun_out/plans_WLTOKEN.txt"
          % (MFMA_COUNTERS, directory, workload),
          "  python3 -m eddl_amd.profsum mfma %s %s %s" % (workload, directory, out),
          ""]
@@ -227,8 +235,8 @@ def stalls(workload, sq_dir, tcp_dir, out):
     dur = durations(sq_dir)
     o = ["Wavefront stall counters of the %s benchmark's convolution kernels (MI355X, gfx950)%s" % (workload, ("; library at commit %s" % commit()) if commit() else ""),
          "commands (from the repository root; two passes, the hardware holds 8 SQ counters at a time):",
-         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --plans gpurun_out/plans_WLTOKEN.txt" % (STALL_SQ, sq_dir, workload),
-         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --plans gpurun_out/plans_WLTOKEN.txt" % (STALL_TCP, tcp_dir, workload),
+         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --no-dropin --plans gpurun_out/plans_WLTOKEN.txt" % (STALL_SQ, sq_dir, workload),
+         "  rocprofv3 --pmc %s --kernel-trace --output-format csv -d %s -o m -- python3 bench.py --workload %s --steps 2 --warmup 1 --no-cpu-baseline --no-device-probe --no-workloads --no-dropin --plans gpurun_out/plans_WLTOKEN.txt" % (STALL_TCP, tcp_dir, workload),
          "  python3 -m eddl_amd.profsum stalls %s %s %s %s" % (workload, sq_dir, tcp_dir, out),
          "",
          "columns (each counter: Counter_Value of a dispatch, averaged over the kernel's dispatches; SQ counters are sampled on one of the",
