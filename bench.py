@@ -209,10 +209,11 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, pl
         with tempfile.NamedTemporaryFile("r", suffix=".txt") as fh:
             hip.conv_tuned_save(fh.name)
             lines = sorted(l.strip() for l in open(fh.name) if l.strip() and not l.startswith("#"))
-        forms = {"planner": 0, "direct_tile": 0, "winograd_three_kernels": 0, "winograd_folded": 0, "winograd_one_launch": 0}
+        forms = {"planner": 0, "direct_tile": 0, "winograd_three_kernels": 0, "winograd_folded": 0, "winograd_one_launch": 0, "upsampled_2x2": 0}
         for l in lines:
             tile = int(l.split("|")[1].split()[0])
-            forms["planner" if tile < 0 else "direct_tile" if tile < 4 else "winograd_three_kernels" if tile == 4 else "winograd_folded" if tile == 5 else "winograd_one_launch"] += 1
+            forms["planner" if tile < 0 else "direct_tile" if tile < 4 else "winograd_three_kernels" if tile == 4 else "winograd_folded" if tile == 5
+                  else "winograd_one_launch" if tile < 8 else "upsampled_2x2"] += 1
         plans_info = {"geometries": len(lines), "sha16": hashlib.sha256("\n".join(lines).encode()).hexdigest()[:16], "kept": forms,
                       "workspace_bytes_after_search": hip.workspace_bytes()}
     step = model.run
@@ -250,6 +251,15 @@ def measure(hip, workload, steps, warmup, fused=True, graph=False, tune=True, pl
                 c_in = op.flops // (2 * conv.kr * conv.kc * n_out * kf)
                 positions = (conv.kr + 1) * (conv.kc + 1)          # 16 products for a 3x3 filter, 9 for a 2x2 one
                 kernel_flops, form = 2 * positions * kf * c_in * blocks, "winograd"
+            elif kern.startswith("upsampled2x2["):
+                # a 2x2 filter on an input upsampled twice, as four convolutions of the stored image: 9 products per channel
+                # and stored pixel ("block") where the direct form has 16
+                blocks = int(kern[kern.rindex(",") + 1:].split()[0])
+                kern = kern[len("upsampled2x2["):kern.rindex(",")]
+                conv = [l for l in op.layers if "cd" in l.attrs][0].attrs["cd"]
+                n_out, kf = conv.out_shape[0] * conv.out_shape[2] * conv.out_shape[3], conv.out_shape[1]
+                c_in = op.flops // (2 * conv.kr * conv.kc * n_out * kf)
+                kernel_flops, form = 2 * 9 * kf * c_in * blocks, "upsampled2x2"
             row.update(kernel=kern.split(" +ksplit")[0], kernel_ms=kms, kernel_launches=kl, kernel_flops=kernel_flops, form=form)
         if op.kind in ("conv2d", "dense") and ms > 0:
             row["tflops"] = op.flops / ms / 1e9
@@ -481,7 +491,7 @@ def main():
         table.append("%-44s %9.4f %9s %8s %9.1f %7.2f  %s" % (
             r["name"][:44], r["ms"], "%.2f" % r["tflops"] if "tflops" in r else "-",
             "%.1f" % (100 * r["frac_fp32_mfma_peak"]) if "tflops" in r else "-", r.get("gbs", 0.0), 100 * r.get("frac_hbm_peak", 0.0),
-            ("winograd: " if r.get("form") == "winograd" else "") + r.get("kernel", "")))
+            ("winograd: " if r.get("form") == "winograd" else "upsampled 2x2: " if r.get("form") == "upsampled2x2" else "") + r.get("kernel", "")))
     if args.layers:
         print("\n".join(table), file=sys.stderr)
     out_dir = args.out

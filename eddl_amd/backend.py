@@ -259,8 +259,8 @@ class Backend:
         self._check(self.lib.eddlhip_conv2d_set_algo({"auto": 0, "mfma": 1, "direct": 2, "mfma_staged": 3, "mfma_lds": 4, "ksplit_off": 5, "ksplit_on": 6, "winograd": 7, "winograd_off": 8, "winograd_never": 9}.get(algo, algo)))
 
     def force_conv_plan(self, tile=-1, slices=1):
-        """Override the convolution launch planner (tile 0..3, K slices; tile 4 / 5: the Winograd forms where they apply);
-        tile -1 restores it."""
+        """Override the convolution launch planner (tile 0..3, K slices; tile 4 .. 7: the Winograd forms where they apply;
+        8 / 9: the upsampled-input form of a 2x2 filter); tile -1 restores it."""
         self._check(self.lib.eddlhip_conv2d_force_plan(tile, slices))
 
     def last_conv_kernel(self):

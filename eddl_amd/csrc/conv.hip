@@ -522,6 +522,29 @@ __device__ __forceinline__ void wino_fold(floatx16 (&y)[2][2], floatx16 &acc, in
     for (int v = 0; v < 16; v++) acc[v] = 0.0f;
 }
 
+// The 2x2 convolution of an image upsampled twice: output (2a + i, 2b + j) sees the stored pixels (a .. a + i, b .. b + j)
+// only, each through the sum of the filter taps that land on it, so the four parities are four convolutions of the
+// stored image with 1x1, 1x2, 2x1 and 2x2 filters - 9 multiplications per channel and block where the direct form has 16.
+// The nine filter rows of channel c, U[9 c + r][column of filter m] (Mp columns, zero past Kf), from OIHW 2x2 filters:
+// r = 0: (w00 + w01) + (w10 + w11) [output (0,0), tap 0]; 1, 2: w00 + w10, w01 + w11 [output (0,1), taps 0, 1];
+// 3, 4: w00 + w01, w10 + w11 [output (1,0), taps 0, 2]; 5..8: w00, w01, w10, w11 [output (1,1), taps 0..3].
+__global__ __launch_bounds__(256) void up2x2_filter_kernel(const float *__restrict__ K, float *__restrict__ U, int Kf, int C, int Mp) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)C * Mp) return;
+    const int c = (int)(idx / Mp), m = (int)(idx - (size_t)c * Mp);
+    float w00 = 0.0f, w01 = 0.0f, w10 = 0.0f, w11 = 0.0f;
+    if (m < Kf) {
+        const float *k = K + ((size_t)m * C + c) * 4;
+        w00 = k[0], w01 = k[1], w10 = k[2], w11 = k[3];
+    }
+    const float r[9] = {__fadd_rn(__fadd_rn(w00, w01), __fadd_rn(w10, w11)), __fadd_rn(w00, w10), __fadd_rn(w01, w11), __fadd_rn(w00, w01), __fadd_rn(w10, w11),
+                        w00, w01, w10, w11};
+    // within each group of 64 filters (the tile of conv_up2x2_kernel) filter j of the first 32 and filter 32 + j sit side by side
+    const int col = (m & ~63) + 2 * (m & 31) + ((m >> 5) & 1);
+#pragma unroll
+    for (int run = 0; run < 9; run++) U[((size_t)c * 9 + run) * Mp + col] = r[run];
+}
+
 // One filter row's four outputs of one 2x2 block (y00 y01 / y10 y11 at rows 2 ty, 2 ty + 1 and columns 2 tx, 2 tx + 1 of
 // image `img`): the convolution's epilogue value by value (the arithmetic of apply_epilogue), two outputs of a row per
 // store where the rows are aligned for it (`pair`), and the block's max-pool where one is asked for.  `e`: the channel
@@ -600,11 +623,18 @@ __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&
 // K-step = CPB input channels x (R*S) taps.  Gather work is split by wavefront: a wavefront
 // serves one 64-pixel segment of the tile (its lanes = 64 consecutive output pixels) and CPW of
 // the step's channels; each of its loads is one (channel, tap) row segment of 64 floats.
-template <int WM, int WN, int TM, int TN, int R, int S, int CPB, bool DIRECT, bool WINO = false>
-__global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(const ConvParams p) {  // registers for 3 (4) workgroups per CU
+// MODE: 0 = a convolution; 1 = the 16 (9) products of a Winograd convolution with the output transform folded in
+// (wino_fold); 2 = a 2x2 convolution of an image upsampled twice, as four convolutions of the stored image, one per
+// parity of the output row and column, on four accumulators (see up2x2_filter_kernel).
+template <int WM, int WN, int TM, int TN, int R, int S, int CPB, bool DIRECT, int MODE>
+__device__ __forceinline__ void conv_tap_body(const ConvParams &p) {
+    constexpr bool WINO = MODE == 1;  // the K range is a sequence of runs whose products end in the four outputs of a 2x2 block
+    constexpr bool UP2 = MODE == 2;
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     static_assert(!WINO || (TM == 1 && TN == 1 && R == 1 && S == 1), "the Winograd products run on one 32x32 block per wavefront");
+    static_assert(!UP2 || (DIRECT && R == 2 && S == 2 && TN == 1 && CPB % 2 == 0), "the upsampled form: 2x2 taps of the stored image, LDS-direct loads");
     constexpr int RS = R * S, BK = CPB * RS;
+    constexpr int AK = UP2 ? CPB * 9 : BK;  // filter rows of a K-step (UP2: nine weight sums per channel where the pixel slice has four taps)
     constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
     constexpr int NS = BN / 64;     // 64-pixel segments in a tile row
     constexpr int WPS = 4 / NS;     // wavefronts that share a segment
@@ -616,11 +646,11 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     // halves are served in separate passes, so they do not conflict (SQ_LDS_BANK_CONFLICT reads 0),
     // and without padding four workgroups fit in a CU's LDS instead of three.
     constexpr int LDA = BM, LDB = BN;
-    constexpr int A_VECS = BK * BM / 4;          // float4 in one filter slice
+    constexpr int A_VECS = AK * BM / 4;          // float4 in one filter slice
     constexpr int AV = (A_VECS + 255) / 256;     // float4 filter loads per thread per step (last one partial)
 
     // (+256 floats after each filter slice: where the lanes past the end of a partial last load round park their float4)
-    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA + 256];
+    __shared__ __attribute__((aligned(16))) float As[2][AK * LDA + 256];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -635,7 +665,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     const int m0 = m_tile * BM;
     const long long n0 = (long long)n_tile * BN;
     ChannelEpilogue chan = {0.0f, 0.0f, 1.0f, 1.0f, 0.0f};
-    if (!split) chan = fetch_channel_constants<BM>(p, m0, tid);
+    if (!split && !UP2) chan = fetch_channel_constants<BM>(p, m0, tid);  // (UP2 has no register to spare in its K loop: fetched after it)
 
     const __amdgpu_buffer_rsrc_t rsrc_in = __builtin_amdgcn_make_buffer_rsrc((void *)p.I, 0, p.in_bytes, RSRC_WORD3);
     const __amdgpu_buffer_rsrc_t rsrc_in2 = __builtin_amdgcn_make_buffer_rsrc((void *)p.I2, 0, p.in_bytes, RSRC_WORD3);
@@ -643,7 +673,25 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     // ---- this thread's gathered pixel and its R*S tap offsets (bytes; OOB where the tap leaves the image)
     const int seg = wave % NS, cg = wave / NS;
     int voff[RS];
-    {
+    // UP2: a "pixel" of the launch is pixel (a, b) of the stored image, i.e. the 2x2 block of outputs at (2a, 2b); tap
+    // t = 2 ky + kx of it is the stored pixel (a + ky, b + kx), nothing where that leaves the image (the upsampled image
+    // ends there: what follows is the zero padding below and to the right)
+    if constexpr (UP2) {
+        const int ng = (int)n0 + seg * 64 + lane;
+        const bool pvalid = ng < p.wT;
+        const unsigned ngc = pvalid ? (unsigned)ng : 0u;
+        const unsigned per_img = (unsigned)(p.wth * p.wtw);
+        const int img = (int)(ngc / per_img);
+        const int r = (int)(ngc - (unsigned)img * per_img);
+        const int a = (int)((unsigned)r / (unsigned)p.wtw), b = r - a * p.wtw;
+        const int pix = img * (p.Cimg * p.H * p.W) + a * p.W + b;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int ky = t >> 1, kx = t & 1;
+            const bool ok = pvalid && a + ky < p.H && b + kx < p.W;
+            voff[t] = ok ? (pix + ky * p.W + kx) * 4 : OOB;
+        }
+    } else {
         const int ng = (int)n0 + seg * 64 + lane;  // a launch covers fewer than 2^31 pixels
         const bool pvalid = ng < (int)p.npix;
         const unsigned ngc = pvalid ? (unsigned)ng : 0u;
@@ -688,9 +736,9 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         const int fc = in_slice ? f : tid % A_VECS;
         const int kk = fc / (BM / 4), m4 = (fc % (BM / 4)) * 4;
         a_ptr[j] = wp + (size_t)kk * p.Mp + m0 + m4;
-        a_lds[j] = in_slice ? kk * LDA + m4 : BK * LDA + lane * 4;
+        a_lds[j] = in_slice ? kk * LDA + m4 : AK * LDA + lane * 4;
     }
-    const int a_step = BK * p.Mp;
+    const int a_step = AK * p.Mp;
 
     floatx4 areg[DIRECT ? 1 : AV];
     float breg[DIRECT ? 1 : CPW * RS];
@@ -701,7 +749,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
     // past the end of the packed matrix, which the buffer descriptor bounds) into the parking area
     // behind the slice.
     constexpr int RPI = 256 / BM;
-    constexpr int A_UNITS = (BK + RPI - 1) / RPI;
+    constexpr int A_UNITS = (AK + RPI - 1) / RPI;
     constexpr int A_UPW = (A_UNITS + 3) / 4;
     static_assert((RPI - 1) * BM <= 256, "the parking area holds the surplus rows of the last unit");
     const int32x4 dma_w = make_rsrc_words(wp, p.wp_bytes), dma_in = make_rsrc_words(p.I, p.in_bytes);
@@ -715,7 +763,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
                 const int u = wave + 4 * j;
                 if (A_UNITS % 4 == 0 || j < A_UPW - 1 || u < A_UNITS) {  // uniform in the wavefront
                     const int kk = u * RPI;
-                    lds_dma_b128(dma_w, as + kk * LDA, a_voff_direct, (step * BK + kk) * p.Mp * 4);
+                    lds_dma_b128(dma_w, as + kk * LDA, a_voff_direct, (step * AK + kk) * p.Mp * 4);
                 }
             }
         } else {
@@ -777,13 +825,26 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         }
     };
 
-    floatx16 acc[TM][TN];
+    floatx16 acc[UP2 ? 1 : TM][UP2 ? 1 : TN];
+    if constexpr (!UP2) {
 #pragma unroll
-    for (int tm = 0; tm < TM; tm++)
+        for (int tm = 0; tm < TM; tm++)
 #pragma unroll
-        for (int tn = 0; tn < TN; tn++)
+            for (int tn = 0; tn < TN; tn++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.0f;
+                for (int v = 0; v < 16; v++) acc[tm][tn][v] = 0.0f;
+    }
+    floatx16 uy[UP2 ? TM : 1][2][2];  // UP2: per 32-filter block the outputs (2a + i, 2b + j) of the wavefront's stored pixels (a, b)
+    if constexpr (UP2) {
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) uy[tm][i][j][v] = 0.0f;
+    }
 
     const int full_steps = p.C / CPB;  // steps whose channels all exist
     const int a_off = (lane >> 5) * LDA + wm * TM * 32 + (lane & 31);
@@ -798,6 +859,67 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
             load_a(step + 1, a_nxt);
             if (step + 1 < full_steps) load_b(step + 1, b_nxt, false);
             else load_b(step + 1, b_nxt, true);
+        }
+        if constexpr (UP2) {
+            // Filter rows of channel c: 9 c + {0: all four taps; 1, 2: the two rows of column 0, of column 1; 3, 4: the two
+            // columns of row 0, of row 1; 5..8: taps 0..3}; pixel rows: 4 c + tap.  An MFMA consumes two rows, one per half
+            // wavefront (h).  Per channel: output (1,1) takes taps (0,1) and (2,3), output (0,1) the column sums on taps
+            // (0,1), output (1,0) the row sums on taps (0,2); per channel pair: output (0,0) the full sums on tap 0 of both.
+            const int h = lane >> 5;
+            static_assert(TM == 2, "the filter rows hold the two 32-filter blocks of a wavefront interleaved");
+            typedef float floatx2 __attribute__((ext_vector_type(2)));
+            typedef const __attribute__((address_space(3))) floatx2 *lds_f2;
+            // (up2x2_filter_kernel lays a row's 64 filters out as 32 pairs {j, 32 + j}: both blocks' operands in one 8-byte read)
+            const lds_float *ab = a_cur + 2 * (lane & 31), *bb = b_cur + wn * 32 + (lane & 31);
+            // the operands of channel c + 1 are read from LDS while the MFMAs of channel c run (six read instructions: the
+            // pixel rows (0,1) and (2,3) in one, rows (0,2), and the two filter blocks of each of the four row pairs in one)
+            float bq[2][3], aq[2][4][TM], b00 = 0.0f, a_ee[TM];
+            auto read_channel = [&](int c, int set) {
+                bq[set][0] = bb[(4 * c + h) * LDB];
+                bq[set][1] = bb[(4 * c + 2 + h) * LDB];
+                bq[set][2] = bb[(4 * c + 2 * h) * LDB];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const floatx2 a2 = *(lds_f2)(ab + (9 * c + 1 + 2 * r + h) * LDA);
+                    aq[set][r][0] = a2.x;
+                    aq[set][r][1] = a2.y;
+                }
+            };
+            read_channel(0, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+            for (int c = 0; c < CPB; c++) {
+                const int cur = c & 1, nxt = cur ^ 1;
+                if (c + 1 < CPB) read_channel(c + 1, nxt);
+                if (c % 2 == 1) {  // tap 0 of this channel and the one before, under the sums of all four taps
+                    b00 = bb[(4 * (c - 1 + h)) * LDB];
+                    const floatx2 a2 = *(lds_f2)(ab + (9 * (c - 1 + h)) * LDA);
+                    a_ee[0] = a2.x;
+                    a_ee[1] = a2.y;
+                }
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++) {
+                    uy[tm][1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[cur][2][tm], bq[cur][0], uy[tm][1][1], 0, 0, 0);
+                    uy[tm][0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[cur][0][tm], bq[cur][0], uy[tm][0][1], 0, 0, 0);
+                    uy[tm][1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[cur][1][tm], bq[cur][2], uy[tm][1][0], 0, 0, 0);
+                }
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++) uy[tm][1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[cur][3][tm], bq[cur][1], uy[tm][1][1], 0, 0, 0);
+                if (c % 2 == 1) {
+#pragma unroll
+                    for (int tm = 0; tm < TM; tm++) uy[tm][0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_ee[tm], b00, uy[tm][0][0], 0, 0, 0);
+                }
+                // issue order: one read instruction of channel c + 1 behind each of the first MFMAs of channel c
+                constexpr int kReadsNext = 6, kReadsSum = 2;
+                const int reads = (c + 1 < CPB ? kReadsNext : 0) + (c % 2 == 1 ? kReadsSum : 0);
+                const int mfmas = 4 * TM + (c % 2 == 1 ? TM : 0);
+#pragma unroll
+                for (int i = 0; i < mfmas; i++) {
+                    if (i < reads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
+            }
+            return;
         }
         // operands of tap pair ks+1 are read from LDS while the MFMAs of pair ks run
         float a[2][TM], b[2][TN];
@@ -879,6 +1001,13 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         put_channel_constants<BM>(epi, chan, tid);
         __syncthreads();
         wino_store_tile<BM>(p, wy, epi, m0, wm * 32, (int)n0 + wn * 32, lane);
+    } else if constexpr (UP2) {
+        // (launched with whole tiles only; a lane holds the four outputs of a block like the Winograd forms)
+        float *epi = &As[0][0];
+        stage_channel_constants<BM>(p, epi, m0, tid);
+        __syncthreads();
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++) wino_store_tile<BM>(p, uy[tm], epi, m0, wm * TM * 32 + tm * 32, (int)n0 + wn * 32, lane);
     } else if (split) {
         store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
     } else {
@@ -892,6 +1021,20 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
         __syncthreads();
         trace_mark(p, 3);
     }
+}
+
+template <int WM, int WN, int TM, int TN, int R, int S, int CPB, bool DIRECT, bool WINO = false>
+__global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(const ConvParams p) {  // registers for 3 (4) workgroups per CU
+    conv_tap_body<WM, WN, TM, TN, R, S, CPB, DIRECT, WINO ? 1 : 0>(p);
+}
+
+// A 2x2 stride-1 convolution of an image upsampled twice (nearest neighbour), zero padding below and to the right only:
+// 64 filters x 128 stored pixels per workgroup, four channels per K-step (conv_tap_body, MODE 2).  WGS: workgroups per CU
+// the register budget is set for - three hide more of a short K loop's loads and stores; two run alike from the first
+// to the last when the tile count is a whole number of generations that way and not the other.
+template <int WGS>
+__global__ __launch_bounds__(256, WGS) void conv_up2x2_kernel(const ConvParams p) {
+    conv_tap_body<1, 4, 2, 1, 2, 2, 4, true, 2>(p);
 }
 
 // ---------------------------------------------------------------- MFMA kernel, any filter shape
@@ -1999,6 +2142,8 @@ const FusedVariant kfused[] = {FUSED(1, 1, 4, 4), FUSED(2, 1, 4, 3)};
 constexpr int NUM_FUSED = (int)(sizeof(kfused) / sizeof(kfused[0]));
 constexpr int FUSED_TILE0 = 6;      // plan "tile" numbers 6 .. 6 + NUM_FUSED - 1 name these shapes (0..3: direct tiles, 4 / 5: the other Winograd forms)
 constexpr int FUSED_ROW_ALIGN = 8;  // the transformed filters are padded to whole K-steps of every variant
+constexpr int UP2X2_TILE = FUSED_TILE0 + NUM_FUSED;  // plan "tiles" of the upsampled-input form of a 2x2 convolution: conv_up2x2_kernel<3>, <2>
+constexpr int NUM_PLAN_TILES = UP2X2_TILE + 2;
 
 // K slices of the left-over tiles of a one-launch Winograd plan that asks for `slices` of them (T blocks in the launch):
 // the tiles beyond a whole number per CU are divided, as in forced_plan; 1 = nothing is divided
@@ -2128,6 +2273,7 @@ struct CachedFilters {
     int wino_rows;
     float *Wfused;  // 3x3 filters: the transformed filters of the one-launch Winograd form [fused_rows][16][Mp], made on first use
     int fused_rows;
+    float *Wup;  // 2x2 filters: the nine matrices of the upsampled-input form [9][C][Mp] (up2x2_filter_kernel), made on first use
     bool stale;  // K was written through this library since the last repack
 };
 std::mutex g_cache_mutex;
@@ -2156,6 +2302,10 @@ int repack(int dev, CachedFilters &e) {
     if (e.Wfused != nullptr) {
         const dim3 grid((unsigned)(((size_t)e.fused_rows * e.Mp + 255) / 256));
         hipLaunchKernelGGL(wino_filter_kernel<4>, grid, dim3(256), 0, state(dev).stream, e.K, e.Wfused, e.Kf, e.C, e.Mp, e.fused_rows, 1);
+        EH_CHECK_LAUNCH();
+    }
+    if (e.Wup != nullptr) {
+        hipLaunchKernelGGL(up2x2_filter_kernel, dim3((unsigned)(((size_t)e.C * e.Mp + 255) / 256)), dim3(256), 0, state(dev).stream, e.K, e.Wup, e.Kf, e.C, e.Mp);
         EH_CHECK_LAUNCH();
     }
     e.stale = false;
@@ -2201,6 +2351,7 @@ void conv_filters_released(int dev, const void *base, size_t bytes) {
             (void)hipFree(c[i].Wp);
             if (c[i].Wwino) (void)hipFree(c[i].Wwino);
             if (c[i].Wfused) (void)hipFree(c[i].Wfused);
+            if (c[i].Wup) (void)hipFree(c[i].Wup);
             c[i] = c.back();
             c.pop_back();
         } else {
@@ -2235,6 +2386,7 @@ int eddlhip_conv2d_cache_filters(int dev, const float *K, int Kf, int C, int R, 
     e.wino_rows = 0;
     e.Wfused = nullptr;
     e.fused_rows = 0;
+    e.Wup = nullptr;
     e.stale = true;
     EH_REQUIRE((size_t)e.rows * e.Mp * sizeof(float) < ((size_t)1 << 31),
                "conv2d_cache_filters: the repacked filter matrix (%d taps x %d channels) exceeds the 2 GiB a buffer descriptor covers", e.rows, e.Mp);
@@ -2261,6 +2413,7 @@ int eddlhip_conv2d_uncache_filters(int dev, const float *K) {
             EH_TRY_HIP(hipFree(c[i].Wp));
             if (c[i].Wwino) EH_TRY_HIP(hipFree(c[i].Wwino));
             if (c[i].Wfused) EH_TRY_HIP(hipFree(c[i].Wfused));
+            if (c[i].Wup) EH_TRY_HIP(hipFree(c[i].Wup));
             c[i] = c.back();
             c.pop_back();
         } else {
@@ -2271,8 +2424,9 @@ int eddlhip_conv2d_uncache_filters(int dev, const float *K) {
 }
 
 int eddlhip_conv2d_force_plan(int tile, int slices) {
-    EH_REQUIRE(tile >= -1 && tile < FUSED_TILE0 + NUM_FUSED, "conv2d_force_plan: tile is -1 (automatic), 0..3, or 4 .. %d (the Winograd forms where they apply)",
-               FUSED_TILE0 + NUM_FUSED - 1);
+    EH_REQUIRE(tile >= -1 && tile < NUM_PLAN_TILES,
+               "conv2d_force_plan: tile is -1 (automatic), 0..3, 4 .. %d (the Winograd forms where they apply) or %d, %d (a 2x2 filter on an input upsampled twice)",
+               UP2X2_TILE - 1, UP2X2_TILE, UP2X2_TILE + 1);
     g_force_tile = tile;
     g_force_slices = slices;
     return 0;
@@ -2296,7 +2450,7 @@ int eddlhip_conv2d_tuned_save(int dev, const char *host_path) {
     EH_REQUIRE(dev >= 0 && dev < EDDLHIP_MAX_DEVICES && host_path != nullptr, "conv2d_tuned_save: bad arguments");
     FILE *f = fopen(host_path, "w");
     EH_REQUIRE(f != nullptr, "conv2d_tuned_save: cannot write %s", host_path);
-    fprintf(f, "# eddlhip tuned convolution plans: N C Kf R S sr sc P Q direct | tile slices\n");
+    fprintf(f, "# eddlhip tuned convolution plans: N C Kf R S sr sc P Q kind | tile slices\n");
     for (const TunedPlan &t : g_tuned[dev]) {
         for (int v : t.key) fprintf(f, "%d ", v);
         fprintf(f, "| %d %d\n", t.tile, t.slices);
@@ -2319,7 +2473,7 @@ int eddlhip_conv2d_tuned_load(int dev, const char *host_path) {
         int *k = t.key;
         const int got = sscanf(line, "%d %d %d %d %d %d %d %d %d %d | %d %d", k, k + 1, k + 2, k + 3, k + 4, k + 5, k + 6, k + 7, k + 8, k + 9, &t.tile,
                                &t.slices);
-        if (got != 12 || t.tile < -1 || t.tile >= FUSED_TILE0 + NUM_FUSED || t.slices < 1 || t.slices > 16) {  // (no search tries more than 16 slices)
+        if (got != 12 || t.tile < -1 || t.tile >= NUM_PLAN_TILES || t.slices < 1 || t.slices > 16) {  // (no search tries more than 16 slices)
             bad = true;
             break;
         }
@@ -2424,6 +2578,19 @@ int conv2d_winograd_fused(int variant, int slices, int dev, const float *I, cons
                           int N, int C, int H, int W, int Kf, int pad_top, int pad_left, int P, int Q, const float *bn_g, const float *bn_b,
                           const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu);
 
+int conv2d_up2x2(int variant, int dev, const float *I, const float *K, const float *bias, float *O, int N, int C, int H, int W, int Kf, int P, int Q, const float *bn_g,
+                 const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu);
+
+// Whether a convolution is the one conv_up2x2_kernel computes: a 2x2 stride-1 filter on ONE tensor upsampled twice in both
+// directions, no padding above or to the left (below and to the right the image is followed by zeros, as many as the
+// output size asks for), whole K-steps of 4 channels, and everything within 32-bit offsets.
+bool up2x2_applies(int N, int C, int H, int W, int Kf, int R, int S, int sr, int sc, int uh, int uw, bool two, int pad_top, int pad_left, int P, int Q) {
+    if (R != 2 || S != 2 || sr != 1 || sc != 1 || uh != 2 || uw != 2 || two || pad_top != 0 || pad_left != 0 || C % 4 != 0) return false;
+    const long long T = (long long)N * ((P + 1) / 2) * ((Q + 1) / 2);
+    const long long Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
+    return T <= 0x3fffff80LL && (long long)N * C * H * W * 4 < (1LL << 31) && 9LL * C * Mp * 4 < (1LL << 31);
+}
+
 // Whether the Winograd form can run this convolution: 3x3, stride 1, and the product launch within the limits of
 // conv2d_fwd_impl (one "image" of transformed input or output below 1 GiB, fewer than 2^31 blocks).
 bool winograd_applies(int N, int C, int Kf, int R, int S, int sr, int sc, int P, int Q) {
@@ -2485,7 +2652,8 @@ size_t winograd_workspace(bool fold, int N, int C, int Kf, int fs, int P, int Q,
 // the one-launch Winograd form, the direct tiles, the Winograd forms with a transformed input in memory; within a form
 // fewer K slices first.  Returns 0 with *out filled, 1 when these tensors cannot be searched on (the output overlaps an
 // input: repeating the call would change what it reads), or minus the error code of a runtime failure.
-int search_plan(const ConvCall &c, const Variant *family, const Plan &planned, long long chunk_pix, bool wino_ok, bool fold_ok, bool fused_ok, TunedPlan *out) {
+int search_plan(const ConvCall &c, const Variant *family, const Plan &planned, long long chunk_pix, bool wino_ok, bool fold_ok, bool fused_ok, bool up_ok,
+                TunedPlan *out) {
     {
         const size_t out_bytes = (size_t)c.N * c.Kf * c.P * c.Q * 4, in_bytes = (size_t)c.N * (c.I2 ? c.C / 2 : c.C) * c.H * c.W * 4;
         const char *o_lo = (const char *)c.O, *o_hi = o_lo + out_bytes;
@@ -2550,6 +2718,10 @@ int search_plan(const ConvCall &c, const Variant *family, const Plan &planned, l
     }
     time_plan(0, -1, -1);
     if (fatal == 0 && cands.empty()) fatal = set_error(EDDLHIP_EINVAL, "conv2d plan search: the planner's own plan did not run");
+    if (up_ok) {  // (2x2 filters only: no rank shared with the one-launch Winograd form of 3x3 filters)
+        time_plan(1, UP2X2_TILE, 1);
+        time_plan(2, UP2X2_TILE + 1, 1);
+    }
     if (fused_ok)  // the one-launch Winograd form: its tile shapes, each undivided and with the left-over tiles in K slices
         for (int fv = NUM_FUSED - 1; fv >= 0; fv--) {
             int last_slices = 0;
@@ -2756,6 +2928,11 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     // the one-launch form (3x3 filters only) needs no transformed copy of the input, so none of V's limits apply
     const bool fused_ok = !gemm && !no_alloc && g_algo == 0 && !g_wino_never && R == 3 && S == 3 && sr == 1 && sc == 1 &&
                           (long long)C * 16 * p.Mp * 4 < (1LL << 31);
+    // the upsampled-input form of a 2x2 filter: a geometry of its own in the plans table (kind 2 / 3), since the same
+    // shapes on a stored tensor cannot take it
+    const bool up_ok = !gemm && !no_alloc && g_algo == 0 && up2x2_applies(N, C, H, W, Kf, R, S, sr, sc, uh, uw, two, pad_top, pad_left, P, Q);
+    if (up_ok && (g_force_tile == UP2X2_TILE || g_force_tile == UP2X2_TILE + 1))
+        return conv2d_up2x2(g_force_tile - UP2X2_TILE, dev, I, K, bias, O, N, C, H, W, Kf, P, Q, bn_g, bn_b, bn_mean, bn_var, bn_eps, residual, relu);
     if (fused_ok && g_force_tile >= FUSED_TILE0 && g_force_tile < FUSED_TILE0 + NUM_FUSED)
         return conv2d_winograd_fused(g_force_tile - FUSED_TILE0, g_force_slices, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top,
                                      pad_left, P, Q, bn_g, bn_b, bn_mean, bn_var, bn_eps, residual, relu);
@@ -2765,7 +2942,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
     const bool query = gemm != nullptr && gemm->need_out != nullptr;  // report the workspace need, launch nothing
     bool plan_open = false;                                         // a search could still pick any plan for this geometry
     if (g_autotune && g_force_tile < 0 && g_algo == 0 && g_split != 0) {
-        const int key[10] = {N, C, Kf, R, S, sr, sc, P, Q, direct};
+        const int key[10] = {N, C, Kf, R, S, sr, sc, P, Q, direct + (up_ok ? 2 : 0)};
         const TunedPlan *found = nullptr;
         for (const TunedPlan &t : g_tuned[dev])
             if (memcmp(t.key, key, sizeof(key)) == 0) found = &t;
@@ -2779,7 +2956,7 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
             TunedPlan best;
             memcpy(best.key, key, sizeof(key));
             const size_t ws_before = state(dev).workspace_bytes;
-            const int src = search_plan(call, family, plan, (long long)chunk_imgs * p.PQ, wino_ok, fold_ok, fused_ok, &best);
+            const int src = search_plan(call, family, plan, (long long)chunk_imgs * p.PQ, wino_ok, fold_ok, fused_ok, up_ok, &best);
             if (src < 0) return -src;  // a runtime error inside the search
             // the candidates may have taken far more workspace than the plan that stays: let it grow back to what is needed
             // (not inside another convolution's call, whose buffers live there)
@@ -2792,6 +2969,8 @@ int conv2d_fwd_impl(bool no_alloc, int dev, const float *I, const float *I2, int
         if (found != nullptr && ((found->tile == 4 && wino_ok) || (found->tile == 5 && fold_ok)))
             return conv2d_winograd(found->tile == 5, R, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g,
                                    bn_b, bn_mean, bn_var, bn_eps, residual, relu);
+        if (found != nullptr && (found->tile == UP2X2_TILE || found->tile == UP2X2_TILE + 1) && up_ok)
+            return conv2d_up2x2(found->tile - UP2X2_TILE, dev, I, K, bias, O, N, C, H, W, Kf, P, Q, bn_g, bn_b, bn_mean, bn_var, bn_eps, residual, relu);
         if (found != nullptr && found->tile >= FUSED_TILE0 && found->tile < FUSED_TILE0 + NUM_FUSED && fused_ok)
             return conv2d_winograd_fused(found->tile - FUSED_TILE0, found->slices, dev, I, two ? I2 : nullptr, uh, uw, K, bias, O, N, C, H, W, Kf, pad_top, pad_left, P, Q, bn_g,
                                          bn_b, bn_mean, bn_var, bn_eps, residual, relu);
@@ -3088,6 +3267,74 @@ int conv2d_winograd(bool fold, int fs, int dev, const float *I, const float *I2,
     char product[sizeof(g_last_kernel)];
     snprintf(product, sizeof(product), "%s", g_last_kernel);
     snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%.100s, %d blocks]", product, Tp);
+    return 0;
+}
+
+// A 2x2 convolution of an input upsampled twice, as four convolutions of the stored image (conv_up2x2_kernel; see
+// up2x2_filter_kernel).  Workspace: the nine filter rows per channel, unless a registered filter tensor keeps them.
+int conv2d_up2x2(int variant, int dev, const float *I, const float *K, const float *bias, float *O, int N, int C, int H, int W, int Kf, int P, int Q, const float *bn_g,
+                 const float *bn_b, const float *bn_mean, const float *bn_var, float bn_eps, const float *residual, int relu) {
+    hipStream_t st = state(dev).stream;
+    PoolRequest *const pool = (g_pool_req != nullptr && !g_tuning && P % 2 == 0 && Q % 2 == 0) ? g_pool_req : nullptr;
+    if (pool != nullptr) pool->done = true;
+    const int th = (P + 1) / 2, tw = (Q + 1) / 2;
+    const int T = N * th * tw, Tp = (T + 127) / 128 * 128;
+    const int Mp = (Kf + M_ALIGN - 1) / M_ALIGN * M_ALIGN;
+    const size_t u_floats = (size_t)9 * C * Mp;
+    const float *U = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_cache_mutex);
+        for (CachedFilters &e : g_cache[dev]) {
+            if (e.K == K && e.Kf == Kf && e.C == C && e.R == 2 && e.S == 2) {
+                if (e.Wup == nullptr && !state(dev).capturing) {
+                    if (hipMalloc((void **)&e.Wup, u_floats * sizeof(float)) != hipSuccess) {
+                        e.Wup = nullptr;
+                        (void)hipGetLastError();
+                        break;  // no room to keep them: made per call
+                    }
+                    e.stale = true;
+                }
+                if (e.Wup != nullptr) {
+                    if (e.stale) EH_TRY(repack(dev, e));
+                    U = e.Wup;
+                }
+                break;
+            }
+        }
+    }
+    if (U == nullptr) {
+        void *ws = nullptr;
+        EH_TRY(get_workspace(dev, u_floats * sizeof(float), &ws));
+        hipLaunchKernelGGL(up2x2_filter_kernel, dim3((unsigned)(((size_t)C * Mp + 255) / 256)), dim3(256), 0, st, K, (float *)ws, Kf, C, Mp);
+        EH_CHECK_LAUNCH();
+        U = (const float *)ws;
+    }
+    ConvParams q;
+    memset(&q, 0, sizeof(q));
+    q.I = I; q.I2 = I; q.Csplit = C; q.Cimg = C; q.uh = 1; q.uw = 1;
+    q.Wp = U; q.w_img_stride = 0; q.K = K; q.O = O;
+    q.bias = bias; q.bn_g = bn_g; q.bn_b = bn_b; q.bn_mean = bn_mean; q.bn_var = bn_var; q.residual = residual;
+    q.bn_eps = bn_eps; q.relu = relu;
+    q.N = N; q.C = C; q.H = H; q.W = W; q.Kf = Kf; q.R = 2; q.S = 2; q.sr = 1; q.sc = 1; q.P = 1; q.Q = Tp;
+    q.CRS = 4 * C; q.Mp = Mp; q.PQ = Tp; q.npix = Tp;
+    q.gm = (Kf + 63) / 64; q.gn = Tp / 128;
+    q.in_bytes = (unsigned)((size_t)N * C * H * W * sizeof(float));
+    q.wp_bytes = (unsigned)(u_floats * sizeof(float));
+    q.main_tiles = q.gm * q.gn; q.nslices = 1;
+    q.wth = th; q.wtw = tw; q.wT = T; q.wP = P; q.wQ = Q; q.wps = 3;
+    if (pool != nullptr) {
+        q.pool_O = pool->O; q.pool_ix = pool->ix; q.pool_iy = pool->iy;
+        if (!pool->keep) q.O = nullptr;
+    }
+    EH_REQUIRE((long long)q.gm * q.gn <= 0x3fffffffLL, "conv2d: internal error, launch of the upsampled 2x2 form");
+    q.nsteps = C / 4;
+    q.slice_steps = q.nsteps;
+    EH_TRY(prof_begin(st));
+    if (variant == 0) hipLaunchKernelGGL(conv_up2x2_kernel<3>, dim3((unsigned)q.main_tiles), dim3(256), 0, st, q);
+    else hipLaunchKernelGGL(conv_up2x2_kernel<2>, dim3((unsigned)q.main_tiles), dim3(256), 0, st, q);
+    EH_CHECK_LAUNCH();
+    EH_TRY(prof_end(st));
+    snprintf(g_last_kernel, sizeof(g_last_kernel), "upsampled2x2[conv_up2x2_kernel<%d>, %d blocks]", variant == 0 ? 3 : 2, Tp);
     return 0;
 }
 

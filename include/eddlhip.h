@@ -238,9 +238,23 @@ int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const fl
  * direct form yields an infinity (all finite inputs give finite outputs as in the direct form); a caller that relies on
  * the propagation of infinities keeps the plan search off or calls eddlhip_conv2d_set_algo(9).
  *
+ * The upsampled-input form of a 2x2 filter (force_plan(8, .) / (9, .), or the search): a 2x2 stride-1 convolution of ONE
+ * tensor that eddlhip_conv2d_fwd_upsampled enlarges twice in both directions, without padding above or to the left (the
+ * convolution behind each UpSampling2D of a U-Net decoder, with its Pad of one row below and one column to the right), is
+ * computed on the stored image: output (2a + i, 2b + j) only sees the stored pixels (a .. a + i, b .. b + j), each under
+ * the sum of the filter taps that land on it, so the four parities of the output position are four convolutions with
+ * 1x1, 1x2, 2x1 and 2x2 filters - 9 multiplications per channel where the direct form has 16, no transform and no
+ * workspace beyond the nine weight sums per filter and channel (kept with a registered filter tensor).  One launch, four
+ * accumulators per lane, the epilogue of the Winograd forms (a lane holds whole 2x2 blocks of outputs; the 2x2 max-pool
+ * can ride along).  The weight sums are rounded once in fp32, so the result differs from the direct form's by rounding
+ * (same tolerance).  Because a convolution of the stored, enlarged tensor cannot take this form, such a call is a
+ * geometry of its own in the plans table (kind 2 / 3 instead of 0 / 1): the same layer run after a stand-alone
+ * UpSampling2D keeps its own plan, and the two agree to the convolution's tolerance, not bit for bit.
+ *
  * eddlhip_conv2d_last_kernel() names the kernel the calling thread's last eddlhip_conv2d_fwd
  * launched, followed by " +ksplit(T tiles x S)" when T tiles were divided into S slices; for the Winograd form
- * "winograd[<kernel and plan of the product launch>, <blocks per product> blocks]". */
+ * "winograd[<kernel and plan of the product launch>, <blocks per product> blocks]", for the upsampled-input form
+ * "upsampled2x2[<kernel>, <blocks> blocks]". */
 int eddlhip_conv2d_set_algo(int algo);
 const char *eddlhip_conv2d_last_kernel(void);
 
@@ -256,7 +270,8 @@ const char *eddlhip_conv2d_last_kernel(void);
  * planner's plan runs (repeating such a call would change what it reads).  The reference does the same on a layer's first forward, with
  * cudnnFindConvolutionForwardAlgorithm (src/hardware/gpu/nn/gpu_conv.cu:42-66, 211-213).  Neither the epilogue, nor the
  * image size and paddings (a folded Pad layer changes both), nor the form of the input (one tensor, two, upsampled) is
- * part of the geometry, so a layer computes the same sums in a fused plan and layer by layer.  A plan that divides tiles
+ * part of the geometry, so a layer computes the same sums in a fused plan and layer by layer - with the one exception of
+ * a 2x2 filter on an input upsampled twice (above), whose own form exists only for the folded call.  A plan that divides tiles
  * along K adds its slices in another order than an undivided one, so results with and without the search agree to the
  * convolution's tolerance, not bit for bit.  Calls that must not allocate or wait (graph recording,
  * eddlhip_conv2d_fwd_noalloc, eddlhip_conv2d_profile collecting) do not search; they use what was found.
@@ -277,7 +292,8 @@ int eddlhip_conv2d_tuned_load(int dev, const char *host_path);
  * slices = number of K slices the tiles left over after a whole number per CU are divided into
  * (1 = none).  tile = 4: the Winograd form wherever it applies (its product launch is planned or searched as usual),
  * 5: its folded form wherever that applies, 6 / 7: its one-launch form on tiles of 32 / 64 filters x 32 blocks, `slices`
- * K slices for the left-over tiles as above; the planner's choice elsewhere.  Acts on the calling thread only. */
+ * K slices for the left-over tiles as above; 8 / 9: the upsampled-input form of a 2x2 filter, built for three / two
+ * workgroups per CU; the planner's choice wherever a form does not apply.  Acts on the calling thread only. */
 int eddlhip_conv2d_force_plan(int tile, int slices);
 
 /* Filters that stay fixed between calls (inference).  Every eddlhip_conv2d_fwd first repacks its

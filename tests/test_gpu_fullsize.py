@@ -11,14 +11,16 @@ Every layer is checked on the DEVICE'S OWN input to that layer:
     output exactly; max-pool outputs equal the input gathered at the reported indices; the
     fused plan reproduces the layer-by-layer plan bit for bit - the network's outputs and every
     max-pool's values and both index tensors (in the fused plan the pools behind Winograd
-    convolutions are computed in the convolution's epilogue).
+    convolutions are computed in the convolution's epilogue); the one exception: a searched plan
+    that holds the upsampled-input form of a 2x2 filter, which only the fused call can take, makes
+    the network's outputs agree to the tolerance instead (the pools, in front of it, stay exact).
 The same checks run with every Winograd form forced wherever it applies and with the plan search
 switched on (the mode bench.py times): the searched K-split and Winograd plans are the ones checked.
 """
 import numpy as np
 import pytest
 
-from test_gpu_models import layer_oracle, EXACT
+from test_gpu_models import layer_oracle, EXACT, assert_fused_equals_walk
 
 pytestmark = pytest.mark.gpu
 
@@ -89,8 +91,7 @@ def check_fullsize(hip, ora, model, x, seed, only_convs=False):
     walked = {l.name: (model.output_of(l).numpy(), model.aux[id(l)]["indX"].numpy(), model.aux[id(l)]["indY"].numpy()) for l in pools}
     model.build(hip, fuse=True)
     out_fused = [o.numpy() for o in model.forward([x])]
-    for a, b in zip(out_unfused, out_fused):
-        assert np.array_equal(a, b), "fused plan differs from the layer-by-layer plan"
+    assert_fused_equals_walk(hip, out_unfused, out_fused)  # (bit for bit, unless the search kept the upsampled-input form of a 2x2 filter)
     for l in pools:  # pooled values and the coordinates of every maximum, bit for bit
         val, ix, iy = walked[l.name]
         assert np.array_equal(model.output_of(l).numpy(), val), "fused plan: values of " + l.name
@@ -225,6 +226,35 @@ def test_winograd_forms_at_full_size(hip, oracle, workload, form):
         hip.force_conv_plan(-1, 1)
         hip.set_conv_algo("winograd_off")
         hip.workspace_trim()
+
+
+@pytest.mark.parametrize("shape", [(4, 1024, 32, 32, 512), (4, 512, 64, 64, 256), (4, 256, 128, 128, 128), (4, 128, 256, 256, 64)],
+                         ids=lambda s: "%dx%dx%dx%d->%d" % s)
+@pytest.mark.parametrize("form", [8, 9], ids=["three per CU", "two per CU"])
+def test_upsampled_2x2_form_at_full_size(hip, oracle, shape, form):
+    """U-Net's four decoder steps at the benchmark's size (UpSampling2D x2, Pad of one row below and one column right, Conv
+    2x2 without bias) in the upsampled-input form, which only the fused call can take and the layer walk of the tests above
+    therefore never runs: sampled outputs (corners, edges, the last tile) against the oracle's direct convolution of the
+    enlarged, padded tensor, to the convolution bar; and twice the same bits."""
+    N, C, H, W, Kf = shape
+    rng = np.random.default_rng(C)
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    w = (rng.standard_normal((Kf, C, 2, 2)) * np.sqrt(2.0 / (4 * C))).astype(np.float32)
+    X, Wd, O, O2 = hip.array(x), hip.array(w), hip.full((N, Kf, 2 * H, 2 * W), 3.0), hip.full((N, Kf, 2 * H, 2 * W), 4.0)
+    hip.force_conv_plan(form, 1)
+    try:
+        hip.conv2D(X, Wd, None, O, 1, 1, 0, 0, upsample=(2, 2))
+        assert hip.last_conv_kernel().startswith("upsampled2x2["), hip.last_conv_kernel()
+        hip.conv2D(X, Wd, None, O2, 1, 1, 0, 0, upsample=(2, 2))
+    finally:
+        hip.force_conv_plan(-1, 1)
+    got = O.numpy()
+    assert np.array_equal(got, O2.numpy())
+    padded = np.zeros((N, C, 2 * H + 1, 2 * W + 1), np.float32)
+    padded[:, :, :2 * H, :2 * W] = np.repeat(np.repeat(x, 2, axis=2), 2, axis=3)
+    idx = sample_coords(rng, got.shape, NPTS)
+    ref = oracle.conv2d_at(padded, w, None, (1, 1), 0, 0, idx)
+    assert_conv_bar(ref, got[idx[:, 0], idx[:, 1], idx[:, 2], idx[:, 3]], float(np.abs(got).max()), "upsampled 2x2 %s" % (shape,))
 
 
 def test_conv_scaling_by_powers_of_two_is_exact_at_full_size(hip):

@@ -47,6 +47,32 @@ def layer_oracle(ora, l, ins):
     raise AssertionError(k)
 
 
+def table_has_upsampled_form(hip):
+    """Whether the plan search kept the upsampled-input form of a 2x2 filter (plan tiles 8 / 9) for some geometry: that form
+    exists only for the fused call (UpSampling2D and Pad folded into the convolution), so a fused plan that takes it agrees
+    with the layer walk to the convolution's tolerance, not bit for bit."""
+    import os
+    import tempfile
+    if hip.conv_tuned_plans() == 0:
+        return False
+    fd, path = tempfile.mkstemp(suffix=".txt")
+    os.close(fd)
+    try:
+        hip.conv_tuned_save(path)
+        return any(l.split("|")[1].split()[0] in ("8", "9") for l in open(path).read().splitlines() if l and not l.startswith("#"))
+    finally:
+        os.unlink(path)
+
+
+def assert_fused_equals_walk(hip, walked, fused):
+    exact = not table_has_upsampled_form(hip)
+    for a, b in zip(walked, fused):
+        if exact:
+            assert np.array_equal(a, b), "fused plan differs from the layer-by-layer plan"
+        else:
+            assert np.abs(a - b).max() <= 1e-4 * np.abs(a).max(), "fused plan (upsampled 2x2 form) differs from the layer-by-layer plan by %g" % np.abs(a - b).max()
+
+
 def check_model(hip, ora, model, x, seed):
     from eddl_amd import models
     models.init_he_normal(model, seed)
@@ -73,8 +99,7 @@ def check_model(hip, ora, model, x, seed):
     model.build(hip, fuse=True)
     outs_fused = model.predict([x])
     assert len(model.ops) < n_unfused
-    for a, b in zip(outs_unfused, outs_fused):
-        assert np.array_equal(a, b), "fused plan differs from the layer-by-layer plan"
+    assert_fused_equals_walk(hip, outs_unfused, outs_fused)
     return outs_fused
 
 
@@ -115,7 +140,9 @@ def test_unet_small(hip, oracle):
 
 def test_fused_plan_equals_layer_walk_with_the_plan_search_on(hip, oracle):
     """The plan search keys on what a plan fixes (channels, filter, output pixels), not on paddings or the form of the input,
-    so a folded Pad / Concat / UpSampling and a fused epilogue still give the layer-by-layer result bit for bit."""
+    so a folded Pad / Concat / UpSampling and a fused epilogue still give the layer-by-layer result bit for bit - unless the
+    search keeps the upsampled-input form for a 2x2 filter behind an UpSampling2D, which only the folded call can take: then
+    the two agree to the tolerance (assert_fused_equals_walk)."""
     from eddl_amd import models
     hip.conv_autotune(-1)
     try:

@@ -451,6 +451,89 @@ def test_conv2d_winograd_form_of_2x2_filters_against_oracle(hip, oracle, form):
         assert_conv_close(ref, O.numpy(), "winograd 2x2 %s" % ((N, C, H, W, Kf, pt, pl, out, up),))
 
 
+UP2X2_FORM = 8      # force_conv_plan tiles 8 and 9: the upsampled-input form of a 2x2 filter
+
+
+def test_conv2d_upsampled_2x2_form_against_oracle(hip, oracle):
+    """A 2x2 filter on an input upsampled twice, run as four convolutions of the stored image (one per parity of the output
+    row and column, weight sums as filters: force_conv_plan(8, .)): U-Net's decoder step (UpSampling2D, Pad of one row below
+    and one column right, Conv 2x2) in small, 'valid' and over-padded output sizes, odd stored sizes, ragged filter counts,
+    channel counts that are whole K-steps of four, the fused epilogue with and without a residual - against the oracle's direct convolution of
+    the upsampled, padded tensor; with registered filters (the nine matrices kept, following a write); with the 2x2 max-pool
+    in its epilogue bit for bit the pool kernel's; and where the form does not apply the planner's plan runs."""
+    rng = np.random.default_rng(88)
+    # N, C, H, W (stored), Kf, output size or None (2H x 2W: one row / column of zeros), residual
+    cases = [(2, 32, 6, 6, 16, None, False), (1, 44, 7, 5, 33, None, True), (3, 12, 5, 9, 70, (9, 17), False), (2, 64, 4, 4, 64, (9, 10), True),
+             (1, 96, 11, 3, 24, (21, 5), False), (5, 32, 8, 8, 128, None, False)]
+    for (N, C, H, W, Kf, out, use_res) in cases:
+        a = rng.standard_normal((N, C, H, W), dtype=np.float32)
+        w = (rng.standard_normal((Kf, C, 2, 2)) * np.sqrt(2.0 / (C * 4))).astype(np.float32)
+        logical = np.repeat(np.repeat(a, 2, axis=2), 2, axis=3)
+        P, Q = out or (2 * H, 2 * W)
+        padded = np.zeros((N, C, P + 1, Q + 1), np.float32)
+        ys, xs = min(2 * H, P + 1), min(2 * W, Q + 1)
+        padded[:, :, :ys, :xs] = logical[:, :, :ys, :xs]
+        bias = rng.standard_normal(Kf, dtype=np.float32)
+        bn = _bn_params(rng, Kf)
+        res = rng.standard_normal((N, Kf, P, Q), dtype=np.float32) if use_res else None
+        ref = oracle.conv2d(padded, w, bias, (1, 1), 0, 0, P, Q)
+        ref, _, _ = oracle.batchnorm_inference(ref, bn[2], bn[3], bn[0], bn[1], bn[4])
+        if use_res:
+            ref = ref + res
+        ref = oracle.relu(ref)
+        O = hip.full((N, Kf, P, Q), 3.0)
+        dbn = (hip.array(bn[0]), hip.array(bn[1]), hip.array(bn[2]), hip.array(bn[3]), bn[4])
+        form = UP2X2_FORM + (N % 2)                 # (the kernel built for three workgroups per CU, or for two)
+        hip.force_conv_plan(form, 1)
+        try:
+            hip.conv2D(hip.array(a), hip.array(w), hip.array(bias), O, 1, 1, 0, 0, bn=dbn, residual=hip.array(res) if use_res else None, relu=True,
+                       upsample=(2, 2))
+            name = hip.last_conv_kernel()
+        finally:
+            hip.force_conv_plan(-1, 1)
+        assert name.startswith("upsampled2x2[conv_up2x2_kernel<%d>," % (3 if form == UP2X2_FORM else 2)), name
+        assert_conv_close(ref, O.numpy(), "upsampled 2x2 %s" % ((N, C, H, W, Kf, out, use_res),))
+
+    # registered filters: the nine matrices are kept and follow a write; the pool in the epilogue
+    N, C, H, W, Kf = 2, 32, 6, 8, 40
+    x = rng.standard_normal((N, C, H, W), dtype=np.float32)
+    w = (rng.standard_normal((Kf, C, 2, 2)) * 0.1).astype(np.float32)
+    X, Wd = hip.array(x), hip.array(w)
+    O1, O2, O3 = (hip.full((N, Kf, 2 * H, 2 * W), v) for v in (1.0, 2.0, 3.0))
+    pooled = lambda: tuple(hip.full((N, Kf, H, W), 7.0) for _ in range(3))
+    A, B = pooled(), pooled()
+    hip.cache_conv_filters(Wd)
+    hip.force_conv_plan(UP2X2_FORM, 1)
+    try:
+        hip.conv2D(X, Wd, None, O1, 1, 1, 0, 0, upsample=(2, 2))
+        assert hip.last_conv_kernel().startswith("upsampled2x2[")
+        first = O1.numpy()
+        up = np.repeat(np.repeat(x, 2, axis=2), 2, axis=3)
+        padded = np.zeros((N, C, 2 * H + 1, 2 * W + 1), np.float32)
+        padded[:, :, :2 * H, :2 * W] = up
+        assert_conv_close(oracle.conv2d(padded, w, None, (1, 1), 0, 0, 2 * H, 2 * W), first, "kept filters")
+        Wd.copy_from(2.0 * w)
+        hip.conv2D(X, Wd, None, O2, 1, 1, 0, 0, upsample=(2, 2))
+        assert np.array_equal(O2.numpy(), 2.0 * first)          # doubling is exact in the weight sums and in every product
+        hip.mpool2D(O2, A[0], A[1], A[2], (2, 2), (2, 2), (0, 0, 0, 0))
+        hip.conv2D(X, Wd, None, O3, 1, 1, 0, 0, upsample=(2, 2), pool=B, keep=True)
+        assert hip.last_conv_kernel().startswith("upsampled2x2[") and np.array_equal(O3.numpy(), O2.numpy())
+        for u, v, what in zip(A, B, ("pooled", "indX", "indY")):
+            assert np.array_equal(u.numpy(), v.numpy()), what
+        # where it does not apply (a stored tensor, a padding above / left, a channel count that is no whole K-step): the planner's plan
+        hip.conv2D(hip.array(up), Wd, None, O1, 1, 1, 0, 0)
+        assert not hip.last_conv_kernel().startswith("upsampled2x2[")
+        O4 = hip.empty((N, Kf, 2 * H + 1, 2 * W + 1))
+        hip.conv2D(X, Wd, None, O4, 1, 1, 1, 1, upsample=(2, 2))
+        assert not hip.last_conv_kernel().startswith("upsampled2x2[")
+        w22 = hip.array((rng.standard_normal((Kf, 22, 2, 2)) * 0.1).astype(np.float32))
+        hip.conv2D(hip.array(x[:, :22].copy()), w22, None, O1, 1, 1, 0, 0, upsample=(2, 2))
+        assert not hip.last_conv_kernel().startswith("upsampled2x2[")
+    finally:
+        hip.force_conv_plan(-1, 1)
+        hip.uncache_conv_filters(Wd)
+
+
 def test_conv2d_winograd_form_only_where_it_applies_and_with_kept_filters(hip, oracle):
     """Strides other than one and filters other than 3x3 keep the direct form under force_conv_plan(4, .) and set_conv_algo
     ("winograd"); registered filters keep their transformed copy, which follows writes to the filter tensor; the call that
