@@ -11,9 +11,10 @@ Every layer is checked on the DEVICE'S OWN input to that layer:
     output exactly; max-pool outputs equal the input gathered at the reported indices; the
     fused plan reproduces the layer-by-layer plan bit for bit - the network's outputs and every
     max-pool's values and both index tensors (in the fused plan the pools behind Winograd
-    convolutions are computed in the convolution's epilogue); the one exception: a searched plan
-    that holds the upsampled-input form of a 2x2 filter, which only the fused call can take, makes
-    the network's outputs agree to the tolerance instead (the pools, in front of it, stay exact).
+    convolutions are computed in the convolution's epilogue); the one exception: under the plan
+    search a 2x2 filter on an upsampled input (U-Net's decoder) is a geometry of its own, with a
+    form that only the fused call can take, and the network's outputs then agree to the tolerance
+    instead (the pools, in front of those layers, stay exact).
 The same checks run with every Winograd form forced wherever it applies and with the plan search
 switched on (the mode bench.py times): the searched K-split and Winograd plans are the ones checked.
 """
@@ -91,7 +92,7 @@ def check_fullsize(hip, ora, model, x, seed, only_convs=False):
     walked = {l.name: (model.output_of(l).numpy(), model.aux[id(l)]["indX"].numpy(), model.aux[id(l)]["indY"].numpy()) for l in pools}
     model.build(hip, fuse=True)
     out_fused = [o.numpy() for o in model.forward([x])]
-    assert_fused_equals_walk(hip, out_unfused, out_fused)  # (bit for bit, unless the search kept the upsampled-input form of a 2x2 filter)
+    assert_fused_equals_walk(hip, out_unfused, out_fused)  # (bit for bit, unless the search met a 2x2 filter on an upsampled input, a geometry of its own)
     for l in pools:  # pooled values and the coordinates of every maximum, bit for bit
         val, ix, iy = walked[l.name]
         assert np.array_equal(model.output_of(l).numpy(), val), "fused plan: values of " + l.name
