@@ -1820,21 +1820,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
     constexpr int RPI = 256 / MF, U_UNITS = U_FLOATS / 256, UPW = U_UNITS / 4;
     const int a_voff = ((lane / (MF / 4)) * p.Mp + m0 + 4 * (lane % (MF / 4))) * 4;
 
+    const bool whole_steps = p.Csplit == p.C || p.Csplit % CK == 0;
     auto load_step = [&](int step, lds_float *us, lds_float *rs, bool checked) {
 #pragma unroll
         for (int j = 0; j < UPW; j++) {
             const int u = wave + 4 * j;
             lds_dma_b128(dma_w, us + u * 256, a_voff, (step * (CK * 16) + u * RPI) * p.Mp * 4);
         }
-        // one input tensor and every channel of the step exists (nearly every step of every layer): nothing is selected
-        if (!checked && p.Csplit == p.C) {
+        // every channel of the step exists and lies in one tensor (nearly every step of every layer; a two-tensor input
+        // whose first tensor ends on a step boundary): nothing is selected per load, the step picks its tensor once
+        if (!checked && whole_steps) {
+            const bool second = step * CK >= p.Csplit;
+            const int32x4 dma = second ? dma_in2 : dma_in;
+            const int c0 = step * CK - (second ? p.Csplit : 0);
 #pragma unroll
             for (int jc = 0; jc < CK / 4; jc++) {
                 const int cl = wave + 4 * jc;
-                const int soff = (step * CK + cl) * HW4;
+                const int soff = (c0 + cl) * HW4;
 #pragma unroll
                 for (int k = 0; k < WLC; k++)
-                    if (k < nload) lds_dma_b32(dma_in, rs + cl * SLOTS + k * 64, voff[k], soff);
+                    if (k < nload) lds_dma_b32(dma, rs + cl * SLOTS + k * 64, voff[k], soff);
             }
             return;
         }
