@@ -456,7 +456,7 @@ UP2X2_FORM = 8      # force_conv_plan tiles 8 and 9: the upsampled-input form of
 
 def test_conv2d_upsampled_2x2_form_against_oracle(hip, oracle):
     """A 2x2 filter on an input upsampled twice, run as four convolutions of the stored image (one per parity of the output
-    row and column, weight sums as filters: force_conv_plan(8, .)): U-Net's decoder step (UpSampling2D, Pad of one row below
+    row and column, weight sums as filters: force_conv_plan(8, .) / (9, .)): U-Net's decoder step (UpSampling2D, Pad of one row below
     and one column right, Conv 2x2) in small, 'valid' and over-padded output sizes, odd stored sizes, ragged filter counts,
     channel counts that are whole K-steps of four, the fused epilogue with and without a residual - against the oracle's direct convolution of
     the upsampled, padded tensor; with registered filters (the nine matrices kept, following a write); with the 2x2 max-pool
@@ -464,7 +464,7 @@ def test_conv2d_upsampled_2x2_form_against_oracle(hip, oracle):
     rng = np.random.default_rng(88)
     # N, C, H, W (stored), Kf, output size or None (2H x 2W: one row / column of zeros), residual
     cases = [(2, 32, 6, 6, 16, None, False), (1, 44, 7, 5, 33, None, True), (3, 12, 5, 9, 70, (9, 17), False), (2, 64, 4, 4, 64, (9, 10), True),
-             (1, 96, 11, 3, 24, (21, 5), False), (5, 32, 8, 8, 128, None, False)]
+             (1, 96, 11, 3, 24, (21, 5), False), (5, 32, 8, 8, 128, None, False), (1, 8, 5, 5, 32, None, False), (2, 4, 6, 7, 16, None, True)]
     for (N, C, H, W, Kf, out, use_res) in cases:
         a = rng.standard_normal((N, C, H, W), dtype=np.float32)
         w = (rng.standard_normal((Kf, C, 2, 2)) * np.sqrt(2.0 / (C * 4))).astype(np.float32)
