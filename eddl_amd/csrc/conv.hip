@@ -601,9 +601,84 @@ __device__ __forceinline__ ChannelEpilogue channel_from_lds(const float *epi, in
     return e;
 }
 
+// NK (4 or 2) consecutive filter rows' outputs of one 2x2 block, x[k][a][b] = output (2 ty + a, 2 tx + b) of filter m + k -
+// the common case of wino_store_row NK times over: all NK filters exist, the block lies inside the output plane, and the
+// rows are aligned for 8-byte stores.  The arithmetic per value is wino_store_row's, step by step; which steps apply is
+// decided once for the 4 NK values (the flags are the same for every lane), the channel constants of the rows come from
+// LDS in one read each (`epi`: stage_channel_constants' layout, ml = the first row's place in the tile, a multiple of
+// NK), one 64-bit address serves all stores, and the residual's loads are in flight together.  (NK = 2 for a kernel with
+// no registers to spare.)
+template <int BM, int NK>
+__device__ __forceinline__ void wino_store_rows(const ConvParams &p, const float *epi, int ml, int m, int img, int ty, int tx, size_t plane,
+                                                float (&x)[NK][2][2]) {
+    static_assert(NK == 4 || NK == 2 || NK == 1, "the constants of the rows are one 16-byte, 8-byte or 4-byte read");
+    typedef float vec_t __attribute__((ext_vector_type(NK)));
+    const size_t o0 = ((size_t)img * p.Kf + (size_t)m) * plane + (size_t)(2 * ty) * p.wQ + 2 * tx;
+    float2 rr[NK][2];
+    if (p.residual) {
+#pragma unroll
+        for (int k = 0; k < NK; k++)
+#pragma unroll
+            for (int a = 0; a < 2; a++) rr[k][a] = *reinterpret_cast<const float2 *>(p.residual + o0 + (size_t)k * plane + (size_t)a * p.wQ);
+    }
+    if (p.bias) {
+        const vec_t bias = *reinterpret_cast<const vec_t *>(epi + ml);
+#pragma unroll
+        for (int k = 0; k < NK; k++)
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int b = 0; b < 2; b++) x[k][a][b] = __fadd_rn(x[k][a][b], bias[k]);
+    }
+    if (p.bn_mean) {
+        const vec_t mean = *reinterpret_cast<const vec_t *>(epi + BM + ml), sd = *reinterpret_cast<const vec_t *>(epi + 2 * BM + ml);
+#pragma unroll
+        for (int k = 0; k < NK; k++)
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int b = 0; b < 2; b++) x[k][a][b] = __fdiv_rn(__fsub_rn(x[k][a][b], mean[k]), sd[k]);
+        if (p.bn_g) {
+            const vec_t g = *reinterpret_cast<const vec_t *>(epi + 3 * BM + ml), bb = *reinterpret_cast<const vec_t *>(epi + 4 * BM + ml);
+#pragma unroll
+            for (int k = 0; k < NK; k++)
+#pragma unroll
+                for (int a = 0; a < 2; a++)
+#pragma unroll
+                    for (int b = 0; b < 2; b++) x[k][a][b] = __fadd_rn(__fmul_rn(x[k][a][b], g[k]), bb[k]);
+        }
+    }
+    if (p.residual) {
+#pragma unroll
+        for (int k = 0; k < NK; k++)
+#pragma unroll
+            for (int a = 0; a < 2; a++) x[k][a][0] = __fadd_rn(x[k][a][0], rr[k][a].x), x[k][a][1] = __fadd_rn(x[k][a][1], rr[k][a].y);
+    }
+    if (p.relu) {
+#pragma unroll
+        for (int k = 0; k < NK; k++)
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int b = 0; b < 2; b++) x[k][a][b] = x[k][a][b] > 0.0f ? x[k][a][b] : 0.0f;
+    }
+    if (p.O != nullptr) {
+#pragma unroll
+        for (int k = 0; k < NK; k++)
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+                *reinterpret_cast<float2 *>(p.O + o0 + (size_t)k * plane + (size_t)a * p.wQ) = make_float2(x[k][a][0], x[k][a][1]);
+    }
+    if (p.pool_O != nullptr) {
+#pragma unroll
+        for (int k = 0; k < NK; k++)
+            pool_block(p, (((size_t)img * p.Kf + (size_t)(m + k)) * p.wth + ty) * p.wtw + tx, ty, tx, x[k][0][0], x[k][0][1], x[k][1][0], x[k][1][1]);
+    }
+}
+
 // A wavefront's 32 filters x 32 blocks: lane = block (column) lane % 32, filter rows 8 * (v / 4) + 4 * (lane / 32) + v % 4.
 // `epi`: the tile's channel constants (stage_channel_constants); m_local: the wavefront's first row in the tile.
-template <int BM>
+template <int BM, int NK = 4>
 __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&y)[2][2], const float *epi, int m0, int m_local, int n_base,
                                                 int lane) {
     const int n = n_base + (lane & 31);
@@ -612,10 +687,35 @@ __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&
     const int img = n / per_img, r = n - img * per_img, ty = r / p.wtw, tx = r - ty * p.wtw;
     const size_t plane = (size_t)p.wP * p.wQ;
     const bool pair = (p.wQ % 2 == 0) && (((size_t)p.O | (size_t)(p.residual ? p.residual : p.O)) % 8 == 0);
+    if constexpr (NK == 1) {  // row by row (a caller with no registers to spare)
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
-        const int ml = m_local + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-        wino_store_row(p, channel_from_lds<BM>(epi, ml), m0 + ml, img, ty, tx, plane, pair, y[0][0][v], y[0][1][v], y[1][0][v], y[1][1][v]);
+        for (int v = 0; v < 16; v++) {
+            const int ml = m_local + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+            wino_store_row(p, channel_from_lds<BM>(epi, ml), m0 + ml, img, ty, tx, plane, pair, y[0][0][v], y[0][1][v], y[1][0][v], y[1][1][v]);
+        }
+        return;
+    }
+    const bool inside = pair && 2 * ty + 1 < p.wP && 2 * tx + 1 < p.wQ;
+#pragma unroll
+    for (int q = 0; q < 16 / NK; q++) {  // rows 8 (v / 4) + 4 (lane / 32) + v % 4 for v = NK q .. NK q + NK - 1
+        const int v0 = NK * q;
+        const int ml = m_local + 8 * (v0 / 4) + 4 * (lane >> 5) + (v0 % 4);
+        if (inside && m0 + ml + NK - 1 < p.Kf) {
+            float x[NK][2][2];
+#pragma unroll
+            for (int k = 0; k < NK; k++)
+#pragma unroll
+                for (int a = 0; a < 2; a++)
+#pragma unroll
+                    for (int b = 0; b < 2; b++) x[k][a][b] = y[a][b][v0 + k];
+            wino_store_rows<BM, NK>(p, epi, ml, m0 + ml, img, ty, tx, plane, x);
+        } else {
+#pragma unroll
+            for (int k = 0; k < NK; k++) {
+                const int v = v0 + k;
+                wino_store_row(p, channel_from_lds<BM>(epi, ml + k), m0 + ml + k, img, ty, tx, plane, pair, y[0][0][v], y[0][1][v], y[1][0][v], y[1][1][v]);
+            }
+        }
     }
 }
 
@@ -625,11 +725,12 @@ __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&
 // the step's channels; each of its loads is one (channel, tap) row segment of 64 floats.
 // MODE: 0 = a convolution; 1 = the 16 (9) products of a Winograd convolution with the output transform folded in
 // (wino_fold); 2 = a 2x2 convolution of an image upsampled twice, as four convolutions of the stored image, one per
-// parity of the output row and column, on four accumulators (see up2x2_filter_kernel).
+// parity of the output row and column, on four accumulators (see up2x2_filter_kernel); 3 = the same, built with registers
+// to spare for the epilogue that finishes four filter rows at a time.
 template <int WM, int WN, int TM, int TN, int R, int S, int CPB, bool DIRECT, int MODE>
 __device__ __forceinline__ void conv_tap_body(const ConvParams &p) {
     constexpr bool WINO = MODE == 1;  // the K range is a sequence of runs whose products end in the four outputs of a 2x2 block
-    constexpr bool UP2 = MODE == 2;
+    constexpr bool UP2 = MODE >= 2;  // (3: with registers to spare for the epilogue's four-row path)
     static_assert(WM * WN == 4, "four wavefronts per workgroup");
     static_assert(!WINO || (TM == 1 && TN == 1 && R == 1 && S == 1), "the Winograd products run on one 32x32 block per wavefront");
     static_assert(!UP2 || (DIRECT && R == 2 && S == 2 && TN == 1 && CPB % 2 == 0), "the upsampled form: 2x2 taps of the stored image, LDS-direct loads");
@@ -1006,8 +1107,13 @@ __device__ __forceinline__ void conv_tap_body(const ConvParams &p) {
         float *epi = &As[0][0];
         stage_channel_constants<BM>(p, epi, m0, tid);
         __syncthreads();
-#pragma unroll
-        for (int tm = 0; tm < TM; tm++) wino_store_tile<BM>(p, uy[tm], epi, m0, wm * TM * 32 + tm * 32, (int)n0 + wn * 32, lane);
+        // (written out: the optimizer does not unroll a loop around this much code, and a runtime index would put the
+        // accumulators in memory)
+        // (row by row under the 168-register budget: 128 accumulator registers leave no room for the values and constants
+        // of four rows at a time)
+        constexpr int NK = MODE == 3 ? 4 : 1;
+        wino_store_tile<BM, NK>(p, uy[0], epi, m0, wm * TM * 32, (int)n0 + wn * 32, lane);
+        if constexpr (UP2) wino_store_tile<BM, NK>(p, uy[UP2 ? 1 : 0], epi, m0, wm * TM * 32 + 32, (int)n0 + wn * 32, lane);
     } else if (split) {
         store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
     } else {
@@ -1034,7 +1140,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
 // to the last when the tile count is a whole number of generations that way and not the other.
 template <int WGS>
 __global__ __launch_bounds__(256, WGS) void conv_up2x2_kernel(const ConvParams p) {
-    conv_tap_body<1, 4, 2, 1, 2, 2, 4, true, 2>(p);
+    conv_tap_body<1, 4, 2, 1, 2, 2, 4, true, (WGS >= 3 ? 2 : 3)>(p);
 }
 
 // ---------------------------------------------------------------- MFMA kernel, any filter shape
@@ -1755,7 +1861,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
     constexpr int XCH_FLOATS = 4 * 2 * 16 * 64;  // the exchange of one 32x32 block: [position row][b][v][lane]
     constexpr int LDS_FLOATS = 2 * BUF_FLOATS > XCH_FLOATS ? 2 * BUF_FLOATS : XCH_FLOATS;
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
-    __shared__ float epi[5 * MF];
+    __shared__ __attribute__((aligned(16))) float epi[5 * MF];
 
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, half = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1980,29 +2086,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
             const int n = n0 + fn * 32 + l32;
             const int nc = n < p.wT ? n : 0;
             const int img = nc / per_img, r = nc - img * per_img, ty = r / p.wtw, tx = r - ty * p.wtw;
+            float yk[4][2][2];  // [k][a][b]: output (2 ty + a, 2 tx + b) of filter row 8 wave + 4 half + k of the block
 #pragma unroll
-            for (int k = 0; k < 4; k++) {
-                float y[2][2];
+            for (int k = 0; k < 4; k++)
 #pragma unroll
                 for (int b = 0; b < 2; b++) {
                     float t[4];
 #pragma unroll
                     for (int i = 0; i < 4; i++) t[i] = xch[((i * 2 + b) * 16 + 4 * wave + k) * 64 + lane];
-                    y[0][b] = __fadd_rn(__fadd_rn(t[0], t[1]), t[2]);
-                    y[1][b] = __fsub_rn(__fsub_rn(t[1], t[2]), t[3]);
+                    yk[k][0][b] = __fadd_rn(__fadd_rn(t[0], t[1]), t[2]);
+                    yk[k][1][b] = __fsub_rn(__fsub_rn(t[1], t[2]), t[3]);
                 }
-                if (split) {
-                    // this slice's share of the four outputs, raw: wino_fused_reduce_kernel adds the slices and finishes
-                    // (layout [slice][tile][32x32 block][wavefront][k][lane] of four floats: a store writes 1 KB)
-                    const size_t tiles = (gridDim.x - (unsigned)p.main_tiles) / p.nslices;
+            const int ml0 = fm * 32 + 8 * wave + 4 * half;
+            if (split) {
+                // this slice's share of the four outputs, raw: wino_fused_reduce_kernel adds the slices and finishes
+                // (layout [slice][tile][32x32 block][wavefront][k][lane] of four floats: a store writes 1 KB)
+                const size_t tiles = (gridDim.x - (unsigned)p.main_tiles) / p.nslices;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
                     floatx4 *dst = reinterpret_cast<floatx4 *>(p.partial) +
                                    (((((size_t)slice * tiles + local_tile) * (FM * FN) + fm * FN + fn) * 4 + wave) * 4 + k) * 64 + lane;
                     floatx4 yv;
-                    yv.x = y[0][0], yv.y = y[0][1], yv.z = y[1][0], yv.w = y[1][1];
+                    yv.x = yk[k][0][0], yv.y = yk[k][0][1], yv.z = yk[k][1][0], yv.w = yk[k][1][1];
                     *dst = yv;
-                } else if (n < p.wT) {
-                    const int ml = fm * 32 + 8 * wave + 4 * half + k;
-                    wino_store_row(p, channel_from_lds<MF>(epi, ml), m0 + ml, img, ty, tx, plane, pair, y[0][0], y[0][1], y[1][0], y[1][1]);
+                }
+            } else if (n < p.wT) {
+                if (pair && 2 * ty + 1 < p.wP && 2 * tx + 1 < p.wQ && m0 + ml0 + 3 < p.Kf) {
+                    wino_store_rows<MF, 4>(p, epi, ml0, m0 + ml0, img, ty, tx, plane, yk);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; k++)
+                        wino_store_row(p, channel_from_lds<MF>(epi, ml0 + k), m0 + ml0 + k, img, ty, tx, plane, pair, yk[k][0][0], yk[k][0][1], yk[k][1][0],
+                                       yk[k][1][1]);
                 }
             }
         }
