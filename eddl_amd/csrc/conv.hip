@@ -1873,7 +1873,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
     // a tile the launch plan divides along the channels: this workgroup sums steps step_lo .. step_hi - 1 only
     const int step_lo = split ? slice * p.slice_steps : 0;
     const int step_hi = split ? min(step_lo + p.slice_steps, p.nsteps) : p.nsteps;
-    if (!split) put_channel_constants<MF>(epi, fetch_channel_constants<MF>(p, m0, tid), tid);  // (published by the loop's first barrier)
+    // Requested first, used last: the step's filter slice needs nothing but the tile's place, so it is on its way while
+    // the lanes work out where the pixels go (below); so are the channel constants, which reach LDS after that.
+    ChannelEpilogue chan = {0.0f, 0.0f, 1.0f, 1.0f, 0.0f};
+
+    // filter slice: a wavefront instruction moves 256 consecutive floats of the slice, i.e. RPI whole rows of MF
+    constexpr int RPI = 256 / MF, U_UNITS = U_FLOATS / 256, UPW = U_UNITS / 4;
+    const int32x4 dma_w = make_rsrc_words(p.Wp, p.wp_bytes);
+    const int a_voff = ((lane / (MF / 4)) * p.Mp + m0 + 4 * (lane % (MF / 4))) * 4;
+    auto load_filters = [&](int step, lds_float *us) {
+#pragma unroll
+        for (int j = 0; j < UPW; j++) {
+            const int u = wave + 4 * j;
+            lds_dma_b128(dma_w, us + u * 256, a_voff, (step * (CK * 16) + u * RPI) * p.Mp * 4);
+        }
+    };
+    load_filters(step_lo, (lds_float *)&lds[0]);
+    if (!split) chan = fetch_channel_constants<MF>(p, m0, tid);
 
     // ---- where the tile's pixels go in LDS, and where this lane's patches lie there.  The tile's blocks are a run of
     // consecutive blocks, i.e. a few SEGMENTS of block rows (a segment: cnt neighbouring blocks of one row of blocks of one
@@ -1894,20 +1910,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
         const int n_end = min(n0 + NB, p.wT);
         const unsigned Hu = (unsigned)(p.H * p.uh), Wu = (unsigned)(p.W * p.uw);
         const int img_elems = p.Cimg * p.H * p.W;
+        const bool whole = p.uh == 1 && p.uw == 1;  // (the stored image itself: no division per slot)
         int base = 0;
         for (int seg_n = n0; seg_n < n_end;) {  // (uniform)
             const int row = seg_n / p.wtw, tx0 = seg_n - row * p.wtw;
             const int cnt = min(p.wtw - tx0, n_end - seg_n), width = 2 * cnt + 2;
             const int img = row / p.wth, ty = row - img * p.wth;
             const int y0 = 2 * ty - p.pt, x0 = 2 * tx0 - p.pl, gbase = img * img_elems;
+            // (only the loads that carry slots of this segment; selects instead of branches: this runs once per workgroup,
+            // in front of everything else, on a SIMD that other workgroups keep busy)
+            const int k_lo = base >> 6, k_hi = (base + 4 * width - 1) >> 6;
 #pragma unroll
             for (int k = 0; k < WLC; k++) {
+                if (k < k_lo || k > k_hi) continue;  // (uniform)
                 const int local = k * 64 + lane - base;
-                if (local >= 0 && local < 4 * width) {
-                    const int r = (local >= width ? 1 : 0) + (local >= 2 * width ? 1 : 0) + (local >= 3 * width ? 1 : 0);
-                    const unsigned y = (unsigned)(y0 + r), x = (unsigned)(x0 + local - r * width);
-                    if (y < Hu && x < Wu) voff[k] = (gbase + (int)(y / (unsigned)p.uh) * p.W + (int)(x / (unsigned)p.uw)) * 4;
-                }
+                const int r = (local >= width ? 1 : 0) + (local >= 2 * width ? 1 : 0) + (local >= 3 * width ? 1 : 0);
+                const unsigned y = (unsigned)(y0 + r), x = (unsigned)(x0 + local - r * width);
+                const bool ok = (unsigned)local < (unsigned)(4 * width) && y < Hu && x < Wu;
+                int off;
+                if (whole) off = (gbase + (int)y * p.W + (int)x) * 4;
+                else off = (gbase + (int)(y / (unsigned)p.uh) * p.W + (int)(x / (unsigned)p.uw)) * 4;
+                voff[k] = ok ? off : voff[k];
             }
 #pragma unroll
             for (int fn = 0; fn < FN; fn++) {
@@ -1920,19 +1943,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
         nload = (base + 63) >> 6;  // loads per channel that carry slots in use
     }
     const int HW4 = p.H * p.W * 4;
-    const int32x4 dma_w = make_rsrc_words(p.Wp, p.wp_bytes), dma_in = make_rsrc_words(p.I, p.in_bytes);
-    const int32x4 dma_in2 = make_rsrc_words(p.I2, p.in_bytes);
-    // filter slice: a wavefront instruction moves 256 consecutive floats of the slice, i.e. RPI whole rows of MF
-    constexpr int RPI = 256 / MF, U_UNITS = U_FLOATS / 256, UPW = U_UNITS / 4;
-    const int a_voff = ((lane / (MF / 4)) * p.Mp + m0 + 4 * (lane % (MF / 4))) * 4;
+    const int32x4 dma_in = make_rsrc_words(p.I, p.in_bytes), dma_in2 = make_rsrc_words(p.I2, p.in_bytes);
 
     const bool whole_steps = p.Csplit == p.C || p.Csplit % CK == 0;
-    auto load_step = [&](int step, lds_float *us, lds_float *rs, bool checked) {
-#pragma unroll
-        for (int j = 0; j < UPW; j++) {
-            const int u = wave + 4 * j;
-            lds_dma_b128(dma_w, us + u * 256, a_voff, (step * (CK * 16) + u * RPI) * p.Mp * 4);
-        }
+    auto load_step = [&](int step, lds_float *us, lds_float *rs, bool checked, bool filters = true) {
+        if (filters) load_filters(step, us);
         // every channel of the step exists and lies in one tensor (nearly every step of every layer; a two-tensor input
         // whose first tensor ends on a step boundary): nothing is selected per load, the step picks its tensor once
         if (!checked && whole_steps) {
@@ -2033,7 +2048,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
     auto rs_of = [&](int buf) { return (lds_float *)&lds[buf * BUF_FLOATS + U_FLOATS]; };
     const int full_steps = p.C / CK;
     constexpr int WAIT_ALL = 0x0F70;  // vmcnt(0): this wavefront's LDS-direct loads have landed
-    load_step(step_lo, us_of(0), rs_of(0), step_lo >= full_steps);
+    load_step(step_lo, us_of(0), rs_of(0), step_lo >= full_steps, false);  // (its filters were requested at the start)
+    if (!split) put_channel_constants<MF>(epi, chan, tid);  // (published by the barrier below)
     __builtin_amdgcn_s_waitcnt(WAIT_ALL);
     __syncthreads();
     trace_mark(p, 1);
