@@ -606,12 +606,11 @@ __device__ __forceinline__ ChannelEpilogue channel_from_lds(const float *epi, in
 // rows are aligned for 8-byte stores.  The arithmetic per value is wino_store_row's, step by step; which steps apply is
 // decided once for the 4 NK values (the flags are the same for every lane), the channel constants of the rows come from
 // LDS in one read each (`epi`: stage_channel_constants' layout, ml = the first row's place in the tile, a multiple of
-// NK), one 64-bit address serves all stores, and the residual's loads are in flight together.  (NK = 2 for a kernel with
-// no registers to spare.)
+// NK), one 64-bit address serves all stores, and the residual's loads are in flight together.
 template <int BM, int NK>
 __device__ __forceinline__ void wino_store_rows(const ConvParams &p, const float *epi, int ml, int m, int img, int ty, int tx, size_t plane,
                                                 float (&x)[NK][2][2]) {
-    static_assert(NK == 4 || NK == 2 || NK == 1, "the constants of the rows are one 16-byte, 8-byte or 4-byte read");
+    static_assert(NK == 4 || NK == 2, "the constants of the rows are one 16-byte or one 8-byte read");
     typedef float vec_t __attribute__((ext_vector_type(NK)));
     const size_t o0 = ((size_t)img * p.Kf + (size_t)m) * plane + (size_t)(2 * ty) * p.wQ + 2 * tx;
     float2 rr[NK][2];
@@ -678,6 +677,7 @@ __device__ __forceinline__ void wino_store_rows(const ConvParams &p, const float
 
 // A wavefront's 32 filters x 32 blocks: lane = block (column) lane % 32, filter rows 8 * (v / 4) + 4 * (lane / 32) + v % 4.
 // `epi`: the tile's channel constants (stage_channel_constants); m_local: the wavefront's first row in the tile.
+// NK: filter rows finished at a time (wino_store_rows), or 1 for a caller that has no registers for that.
 template <int BM, int NK = 4>
 __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&y)[2][2], const float *epi, int m0, int m_local, int n_base,
                                                 int lane) {
@@ -693,27 +693,28 @@ __device__ __forceinline__ void wino_store_tile(const ConvParams &p, floatx16 (&
             const int ml = m_local + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
             wino_store_row(p, channel_from_lds<BM>(epi, ml), m0 + ml, img, ty, tx, plane, pair, y[0][0][v], y[0][1][v], y[1][0][v], y[1][1][v]);
         }
-        return;
-    }
-    const bool inside = pair && 2 * ty + 1 < p.wP && 2 * tx + 1 < p.wQ;
+    } else {
+        const bool inside = pair && 2 * ty + 1 < p.wP && 2 * tx + 1 < p.wQ;
 #pragma unroll
-    for (int q = 0; q < 16 / NK; q++) {  // rows 8 (v / 4) + 4 (lane / 32) + v % 4 for v = NK q .. NK q + NK - 1
-        const int v0 = NK * q;
-        const int ml = m_local + 8 * (v0 / 4) + 4 * (lane >> 5) + (v0 % 4);
-        if (inside && m0 + ml + NK - 1 < p.Kf) {
-            float x[NK][2][2];
+        for (int q = 0; q < 16 / NK; q++) {  // rows 8 (v / 4) + 4 (lane / 32) + v % 4 for v = NK q .. NK q + NK - 1
+            const int v0 = NK * q;
+            const int ml = m_local + 8 * (v0 / 4) + 4 * (lane >> 5) + (v0 % 4);
+            if (inside && m0 + ml + NK - 1 < p.Kf) {
+                float x[NK][2][2];
 #pragma unroll
-            for (int k = 0; k < NK; k++)
+                for (int k = 0; k < NK; k++)
 #pragma unroll
-                for (int a = 0; a < 2; a++)
+                    for (int a = 0; a < 2; a++)
 #pragma unroll
-                    for (int b = 0; b < 2; b++) x[k][a][b] = y[a][b][v0 + k];
-            wino_store_rows<BM, NK>(p, epi, ml, m0 + ml, img, ty, tx, plane, x);
-        } else {
+                        for (int b = 0; b < 2; b++) x[k][a][b] = y[a][b][v0 + k];
+                wino_store_rows<BM, NK>(p, epi, ml, m0 + ml, img, ty, tx, plane, x);
+            } else {
 #pragma unroll
-            for (int k = 0; k < NK; k++) {
-                const int v = v0 + k;
-                wino_store_row(p, channel_from_lds<BM>(epi, ml + k), m0 + ml + k, img, ty, tx, plane, pair, y[0][0][v], y[0][1][v], y[1][0][v], y[1][1][v]);
+                for (int k = 0; k < NK; k++) {
+                    const int v = v0 + k;
+                    wino_store_row(p, channel_from_lds<BM>(epi, ml + k), m0 + ml + k, img, ty, tx, plane, pair, y[0][0][v], y[0][1][v], y[1][0][v],
+                                   y[1][1][v]);
+                }
             }
         }
     }
@@ -1107,13 +1108,12 @@ __device__ __forceinline__ void conv_tap_body(const ConvParams &p) {
         float *epi = &As[0][0];
         stage_channel_constants<BM>(p, epi, m0, tid);
         __syncthreads();
-        // (written out: the optimizer does not unroll a loop around this much code, and a runtime index would put the
-        // accumulators in memory)
-        // (row by row under the 168-register budget: 128 accumulator registers leave no room for the values and constants
-        // of four rows at a time)
+        // (the two blocks written out: the optimizer does not unroll a loop around this much code, and a runtime index
+        // would put the accumulators in memory; four rows at a time only in the build whose register budget has room for
+        // their values and constants beside the 128 accumulator registers)
         constexpr int NK = MODE == 3 ? 4 : 1;
         wino_store_tile<BM, NK>(p, uy[0], epi, m0, wm * TM * 32, (int)n0 + wn * 32, lane);
-        if constexpr (UP2) wino_store_tile<BM, NK>(p, uy[UP2 ? 1 : 0], epi, m0, wm * TM * 32 + 32, (int)n0 + wn * 32, lane);
+        wino_store_tile<BM, NK>(p, uy[TM - 1], epi, m0, wm * TM * 32 + 32, (int)n0 + wn * 32, lane);
     } else if (split) {
         store_partial<TM, TN>(p, acc, local_tile, slice, wave, lane);
     } else {
@@ -1135,7 +1135,7 @@ __global__ __launch_bounds__(256, (TM * TN >= 4 ? 3 : 4)) void conv_tap_kernel(c
 }
 
 // A 2x2 stride-1 convolution of an image upsampled twice (nearest neighbour), zero padding below and to the right only:
-// 64 filters x 128 stored pixels per workgroup, four channels per K-step (conv_tap_body, MODE 2).  WGS: workgroups per CU
+// 64 filters x 128 stored pixels per workgroup, four channels per K-step (conv_tap_body, MODE 2 / 3).  WGS: workgroups per CU
 // the register budget is set for - three hide more of a short K loop's loads and stores; two run alike from the first
 // to the last when the tile count is a whole number of generations that way and not the other.
 template <int WGS>
@@ -2224,9 +2224,11 @@ long long g_trace_wgs = 0;
 // eddlhip_conv2d_autotune: launch plans found by measurement, by device and geometry.  Neither the epilogue nor the form of
 // the input is part of the key (image size and paddings - a folded Pad layer changes both -, one tensor or two, stored or
 // upsampled image): what a plan fixes, tile shape and K slices, meets the same channels, filter and output pixels either
-// way, and a convolution sums in the same order in a fused plan and in a layer-by-layer one.
+// way, and a convolution sums in the same order in a fused plan and in a layer-by-layer one.  One exception: a 2x2 filter
+// on an input upsampled twice has a form that only that call can take (conv_up2x2_kernel), so it is a geometry of its own
+// (kind + 2).
 struct TunedPlan {
-    int key[10];       // N C Kf R S sr sc P Q direct
+    int key[10];       // N C Kf R S sr sc P Q kind (0 / 1: register-staged / LDS-direct gather; + 2: see above)
     int tile, slices;  // tile -1: the planner's own choice was the fastest; tile 4: the Winograd form
 };
 bool g_autotune = false;
@@ -2409,7 +2411,7 @@ struct CachedFilters {
     int wino_rows;
     float *Wfused;  // 3x3 filters: the transformed filters of the one-launch Winograd form [fused_rows][16][Mp], made on first use
     int fused_rows;
-    float *Wup;  // 2x2 filters: the nine matrices of the upsampled-input form [9][C][Mp] (up2x2_filter_kernel), made on first use
+    float *Wup;  // 2x2 filters: the nine weight-sum rows per channel of the upsampled-input form [C][9][Mp] (up2x2_filter_kernel), made on first use
     bool stale;  // K was written through this library since the last repack
 };
 std::mutex g_cache_mutex;
