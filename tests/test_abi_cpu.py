@@ -67,6 +67,17 @@ def test_tuned_plan_table_round_trips_through_a_file(tmp_path):
     assert b"not a plan" in lib.eddlhip_last_error()
     assert lib.eddlhip_conv2d_tuned_load(0, str(tmp_path / "missing.txt").encode()) < 0
     assert lib.eddlhip_conv2d_tuned_plans(0) == 2
+    # every plan number the library knows is accepted - 0..3 direct tiles, 4 / 5 / 6 / 7 the Winograd forms, 8 / 9 the
+    # upsampled-input form of a 2x2 filter, whose geometries carry kind 2 / 3 - and the first unknown one is refused
+    forms = tmp_path / "forms.txt"
+    forms.write_text("".join("4 %d 64 2 2 1 1 128 128 3 | %d 1\n" % (128 + t, t) for t in range(0, 10)))
+    assert lib.eddlhip_conv2d_tuned_load(0, str(forms).encode()) == 0
+    assert lib.eddlhip_conv2d_tuned_plans(0) == 12
+    bad.write_text("4 128 64 2 2 1 1 128 128 3 | 10 1\n")
+    assert lib.eddlhip_conv2d_tuned_load(0, str(bad).encode()) < 0
+    bad.write_text("4 128 64 2 2 1 1 128 128 3 | 8 17\n")      # (no search tries more than 16 slices)
+    assert lib.eddlhip_conv2d_tuned_load(0, str(bad).encode()) < 0
+    assert lib.eddlhip_conv2d_tuned_plans(0) == 12
     lib.eddlhip_conv2d_autotune(-1)
     assert lib.eddlhip_conv2d_tuned_plans(0) == 0
 
