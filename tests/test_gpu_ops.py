@@ -494,6 +494,23 @@ def test_conv2d_upsampled_2x2_form_against_oracle(hip, oracle):
         assert name.startswith("upsampled2x2[conv_up2x2_kernel<%d>," % (3 if form == UP2X2_FORM else 2)), name
         assert_conv_close(ref, O.numpy(), "upsampled 2x2 %s" % ((N, C, H, W, Kf, out, use_res),))
 
+    # the two builds of the kernel (three and two workgroups per CU; row-by-row and four-row epilogue) sum in one order
+    for (N, C, H, W, Kf) in ((3, 40, 9, 7, 70), (2, 128, 16, 16, 64)):
+        a = rng.standard_normal((N, C, H, W), dtype=np.float32)
+        w = (rng.standard_normal((Kf, C, 2, 2)) * 0.1).astype(np.float32)
+        bn = _bn_params(rng, Kf)
+        dbn = (hip.array(bn[0]), hip.array(bn[1]), hip.array(bn[2]), hip.array(bn[3]), bn[4])
+        outs = []
+        for form in (UP2X2_FORM, UP2X2_FORM + 1):
+            O = hip.full((N, Kf, 2 * H, 2 * W), float(form))
+            hip.force_conv_plan(form, 1)
+            try:
+                hip.conv2D(hip.array(a), hip.array(w), None, O, 1, 1, 0, 0, bn=dbn, relu=True, upsample=(2, 2))
+            finally:
+                hip.force_conv_plan(-1, 1)
+            outs.append(O.numpy())
+        assert np.array_equal(outs[0], outs[1]), (N, C, H, W, Kf)
+
     # registered filters: the nine matrices are kept and follow a write; the pool in the epilogue
     N, C, H, W, Kf = 2, 32, 6, 8, 40
     x = rng.standard_normal((N, C, H, W), dtype=np.float32)
