@@ -82,6 +82,28 @@ def test_tuned_plan_table_round_trips_through_a_file(tmp_path):
     assert lib.eddlhip_conv2d_tuned_plans(0) == 0
 
 
+def test_committed_plans_files_load():
+    """The plans files the profiled commands name (profiles/plans_<workload>.txt) are in the loader's format, and what the
+    loader keeps of each is what the file says, line for line."""
+    import glob
+    import tempfile
+    from eddl_amd import _lib
+    lib = _lib.load()
+    files = sorted(glob.glob(os.path.join(ROOT, "profiles", "plans_*.txt")))
+    assert len(files) >= 4, files
+    for path in files:
+        lib.eddlhip_conv2d_autotune(-1)
+        assert lib.eddlhip_conv2d_tuned_load(0, path.encode()) == 0, (path, lib.eddlhip_last_error())
+        want = sorted(l.strip() for l in open(path).read().splitlines() if l.strip() and not l.startswith("#"))
+        assert lib.eddlhip_conv2d_tuned_plans(0) == len(want) > 0, path
+        with tempfile.TemporaryDirectory() as tmp:
+            out = os.path.join(tmp, "saved.txt")
+            assert lib.eddlhip_conv2d_tuned_save(0, out.encode()) == 0
+            got = sorted(l.strip() for l in open(out).read().splitlines() if l.strip() and not l.startswith("#"))
+        assert got == want, path
+    lib.eddlhip_conv2d_autotune(-1)
+
+
 def test_descriptor_mirrors_match_the_oracle_geometry(oracle, golden):
     from eddl_amd.descriptors import ConvolDescriptor, PoolDescriptor
     t = golden["output_sizes"]
