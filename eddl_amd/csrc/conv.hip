@@ -1851,7 +1851,9 @@ __device__ __forceinline__ void wino_sched_pair() {
 // block: y[a][b] = s[0][b] + s[1][b] + s[2][b] (a = 0), s[1][b] - s[2][b] - s[3][b] (a = 1), then the convolution's
 // epilogue (wino_store_row).  Sums: channels in increasing order, two per matrix instruction, one accumulator per
 // position from the first channel to the last; the output transform in the order just given.  Whole tiles only.
-template <int FM, int FN, int CK, int WPE>  // WPE: wavefronts per SIMD the register budget is set for
+// WPE: wavefronts per SIMD the register budget is set for.  WIDE: the pixels come in 16 bytes per lane (two load instructions
+// per channel where the 4-byte gather issues five), for launches whose image rows are a multiple of four pixels long.
+template <int FM, int FN, int CK, int WPE, bool WIDE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void wino_fused_kernel(const ConvParams p) {
     static_assert(CK % 4 == 0 && FN <= 2 && FM <= 2, "a wavefront stages whole channels; a lane gathers one block");
     constexpr int MF = 32 * FM, NB = 32 * FN;
@@ -1898,7 +1900,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
     // 2 tx_first - pad_left + x).  The slots of a channel are consecutive LDS floats, slot k * 64 + lane is written by lane
     // `lane` of load k: its byte offset in a channel plane (or out of range: padding, a block past the end) is worked out
     // here once.  16 NB slots always suffice (a segment of one block takes 16).
-    constexpr int SLOTS = 16 * NB, WLC = SLOTS / 64;
+    constexpr int SLOTS = 16 * NB, WLC = WIDE ? SLOTS / 256 : SLOTS / 64;
     const int per_img = p.wth * p.wtw;
     int voff[WLC], my_base[FN], my_stride[FN];
 #pragma unroll
@@ -1917,30 +1919,54 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
             const int cnt = min(p.wtw - tx0, n_end - seg_n), width = 2 * cnt + 2;
             const int img = row / p.wth, ty = row - img * p.wth;
             const int y0 = 2 * ty - p.pt, x0 = 2 * tx0 - p.pl, gbase = img * img_elems;
-            // (only the loads that carry slots of this segment; selects instead of branches: this runs once per workgroup,
-            // in front of everything else, on a SIMD that other workgroups keep busy)
-            const int k_lo = base >> 6, k_hi = (base + 4 * width - 1) >> 6;
+            if constexpr (WIDE) {
+                // 16 bytes per lane: a segment's pixel rows start at the multiple of four columns at or below x0 and are
+                // a whole number of GROUPS of four columns long.  The launch has image rows of a multiple of four pixels
+                // and 16-byte aligned tensors, so a group lies inside the image or outside it as a whole (out of range:
+                // four zeros), every load is aligned, and a patch starts `shift` slots into its row (odd with one column
+                // of padding: the patches are read with 4-byte alignment).  Group g of a channel is written by lane
+                // g % 64 of load g / 64.  (The host launches this build only where 16 NB slots hold the widened rows.)
+                const int xs = ((x0 + 4) & ~3) - 4, shift = x0 - xs, gpr = (shift + width + 3) >> 2, gb = base >> 2;
 #pragma unroll
-            for (int k = 0; k < WLC; k++) {
-                if (k < k_lo || k > k_hi) continue;  // (uniform)
-                const int local = k * 64 + lane - base;
-                const int r = (local >= width ? 1 : 0) + (local >= 2 * width ? 1 : 0) + (local >= 3 * width ? 1 : 0);
-                const unsigned y = (unsigned)(y0 + r), x = (unsigned)(x0 + local - r * width);
-                const bool ok = (unsigned)local < (unsigned)(4 * width) && y < Hu && x < Wu;
-                int off;
-                if (whole) off = (gbase + (int)y * p.W + (int)x) * 4;
-                else off = (gbase + (int)(y / (unsigned)p.uh) * p.W + (int)(x / (unsigned)p.uw)) * 4;
-                voff[k] = ok ? off : voff[k];
-            }
+                for (int k = 0; k < WLC; k++) {
+                    const int local = k * 64 + lane - gb;
+                    const int r = (local >= gpr ? 1 : 0) + (local >= 2 * gpr ? 1 : 0) + (local >= 3 * gpr ? 1 : 0);
+                    const unsigned y = (unsigned)(y0 + r), x = (unsigned)(xs + 4 * (local - r * gpr));
+                    const bool ok = (unsigned)local < (unsigned)(4 * gpr) && y < Hu && x < Wu;
+                    voff[k] = ok ? (gbase + (int)y * p.W + (int)x) * 4 : voff[k];
+                }
 #pragma unroll
-            for (int fn = 0; fn < FN; fn++) {
-                const int n = n0 + fn * 32 + l32;
-                if (n >= seg_n && n < seg_n + cnt) my_base[fn] = base + 2 * (n - seg_n), my_stride[fn] = width;
+                for (int fn = 0; fn < FN; fn++) {
+                    const int n = n0 + fn * 32 + l32;
+                    if (n >= seg_n && n < seg_n + cnt) my_base[fn] = base + shift + 2 * (n - seg_n), my_stride[fn] = 4 * gpr;
+                }
+                base += 16 * gpr;
+            } else {
+                // (only the loads that carry slots of this segment; selects instead of branches: this runs once per
+                // workgroup, in front of everything else, on a SIMD that other workgroups keep busy)
+                const int k_lo = base >> 6, k_hi = (base + 4 * width - 1) >> 6;
+#pragma unroll
+                for (int k = 0; k < WLC; k++) {
+                    if (k < k_lo || k > k_hi) continue;  // (uniform)
+                    const int local = k * 64 + lane - base;
+                    const int r = (local >= width ? 1 : 0) + (local >= 2 * width ? 1 : 0) + (local >= 3 * width ? 1 : 0);
+                    const unsigned y = (unsigned)(y0 + r), x = (unsigned)(x0 + local - r * width);
+                    const bool ok = (unsigned)local < (unsigned)(4 * width) && y < Hu && x < Wu;
+                    int off;
+                    if (whole) off = (gbase + (int)y * p.W + (int)x) * 4;
+                    else off = (gbase + (int)(y / (unsigned)p.uh) * p.W + (int)(x / (unsigned)p.uw)) * 4;
+                    voff[k] = ok ? off : voff[k];
+                }
+#pragma unroll
+                for (int fn = 0; fn < FN; fn++) {
+                    const int n = n0 + fn * 32 + l32;
+                    if (n >= seg_n && n < seg_n + cnt) my_base[fn] = base + 2 * (n - seg_n), my_stride[fn] = width;
+                }
+                base += 4 * width;
             }
-            base += 4 * width;
             seg_n += cnt;
         }
-        nload = (base + 63) >> 6;  // loads per channel that carry slots in use
+        nload = WIDE ? (base + 255) >> 8 : (base + 63) >> 6;  // loads per channel that carry slots in use
     }
     const int HW4 = p.H * p.W * 4;
     const int32x4 dma_in = make_rsrc_words(p.I, p.in_bytes), dma_in2 = make_rsrc_words(p.I2, p.in_bytes);
@@ -1960,7 +1986,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
                 const int soff = (c0 + cl) * HW4;
 #pragma unroll
                 for (int k = 0; k < WLC; k++)
-                    if (k < nload) lds_dma_b32(dma, rs + cl * SLOTS + k * 64, voff[k], soff);
+                    if (k < nload) {
+                        if constexpr (WIDE) lds_dma_b128(dma, rs + cl * SLOTS + k * 256, voff[k], soff);
+                        else lds_dma_b32(dma, rs + cl * SLOTS + k * 64, voff[k], soff);
+                    }
             }
             return;
         }
@@ -1972,7 +2001,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
             const int soff = (cok ? (second ? c - p.Csplit : c) : 0) * HW4;
 #pragma unroll
             for (int k = 0; k < WLC; k++)
-                if (k < nload) lds_dma_b32(second ? dma_in2 : dma_in, rs + cl * SLOTS + k * 64, cok ? voff[k] : OOB, soff);
+                if (k < nload) {
+                    if constexpr (WIDE) lds_dma_b128(second ? dma_in2 : dma_in, rs + cl * SLOTS + k * 256, cok ? voff[k] : OOB, soff);
+                    else lds_dma_b32(second ? dma_in2 : dma_in, rs + cl * SLOTS + k * 64, cok ? voff[k] : OOB, soff);
+                }
         }
     };
 
@@ -2011,13 +2043,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 #pragma unroll
             for (int fm = 0; fm < FM; fm++) a[into][j][fm] = us[a_off + cp * (32 * MF) + j * MF + fm * 32];
 #pragma unroll
-        for (int fn = 0; fn < FN; fn++) {  // (a patch starts at an even slot: 8-byte reads)
-            typedef float floatx2 __attribute__((ext_vector_type(2)));
-            typedef const __attribute__((address_space(3))) floatx2 *lds_f2;
-            const floatx2 a0 = *(lds_f2)(rs + ra_off[fn] + cp * (2 * SLOTS)), a1 = *(lds_f2)(rs + ra_off[fn] + cp * (2 * SLOTS) + 2);
-            const floatx2 b0 = *(lds_f2)(rs + rb_off[fn] + cp * (2 * SLOTS)), b1 = *(lds_f2)(rs + rb_off[fn] + cp * (2 * SLOTS) + 2);
-            d[0][0][fn] = a0.x, d[0][1][fn] = a0.y, d[0][2][fn] = a1.x, d[0][3][fn] = a1.y;
-            d[1][0][fn] = b0.x, d[1][1][fn] = b0.y, d[1][2][fn] = b1.x, d[1][3][fn] = b1.y;
+        for (int fn = 0; fn < FN; fn++) {
+            if constexpr (WIDE) {  // (a patch may start at an odd slot: pairs of 4-byte reads)
+                const lds_float *pa = rs + ra_off[fn] + cp * (2 * SLOTS), *pb = rs + rb_off[fn] + cp * (2 * SLOTS);
+                d[0][0][fn] = pa[0], d[0][1][fn] = pa[1], d[0][2][fn] = pa[2], d[0][3][fn] = pa[3];
+                d[1][0][fn] = pb[0], d[1][1][fn] = pb[1], d[1][2][fn] = pb[2], d[1][3][fn] = pb[3];
+            } else {  // (a patch starts at an even slot: 8-byte reads)
+                typedef float floatx2 __attribute__((ext_vector_type(2)));
+                typedef const __attribute__((address_space(3))) floatx2 *lds_f2;
+                const floatx2 a0 = *(lds_f2)(rs + ra_off[fn] + cp * (2 * SLOTS)), a1 = *(lds_f2)(rs + ra_off[fn] + cp * (2 * SLOTS) + 2);
+                const floatx2 b0 = *(lds_f2)(rs + rb_off[fn] + cp * (2 * SLOTS)), b1 = *(lds_f2)(rs + rb_off[fn] + cp * (2 * SLOTS) + 2);
+                d[0][0][fn] = a0.x, d[0][1][fn] = a0.y, d[0][2][fn] = a1.x, d[0][3][fn] = a1.y;
+                d[1][0][fn] = b0.x, d[1][1][fn] = b0.y, d[1][2][fn] = b1.x, d[1][3][fn] = b1.y;
+            }
         }
     };
     auto transform = [&](int into) __attribute__((always_inline)) {
@@ -2269,13 +2307,15 @@ const Variant kgen[2][4] = {{GEN(2, 2, 2, 2, false), GEN(1, 4, 2, 1, false), GEN
 
 // The one-launch Winograd form's tile shapes: 32 FM filters x 32 FN blocks, CK channels per K-step.
 struct FusedVariant {
-    const char *name;
+    const char *name, *name_wide;
     int fm, fn, ck;
     void (*kernel)(const ConvParams);
+    void (*kernel_wide)(const ConvParams);  // the build that loads the pixels 16 bytes per lane (fused_wide_loads)
     void (*reduce)(const ConvParams);
 };
-#define FUSED(FM, FN, CK, WPE) \
-    {"wino_fused_kernel<" #FM "," #FN "," #CK "," #WPE ">", FM, FN, CK, wino_fused_kernel<FM, FN, CK, WPE>, wino_fused_reduce_kernel<FM, FN>}
+#define FUSED(FM, FN, CK, WPE)                                                                                                       \
+    {"wino_fused_kernel<" #FM "," #FN "," #CK "," #WPE ">", "wino_fused_kernel<" #FM "," #FN "," #CK "," #WPE ",true>", FM, FN, CK,  \
+     wino_fused_kernel<FM, FN, CK, WPE, false>,         wino_fused_kernel<FM, FN, CK, WPE, true>, wino_fused_reduce_kernel<FM, FN>}
 const FusedVariant kfused[] = {FUSED(1, 1, 4, 4), FUSED(2, 1, 4, 3)};
 constexpr int NUM_FUSED = (int)(sizeof(kfused) / sizeof(kfused[0]));
 constexpr int FUSED_TILE0 = 6;      // plan "tile" numbers 6 .. 6 + NUM_FUSED - 1 name these shapes (0..3: direct tiles, 4 / 5: the other Winograd forms)
@@ -3502,6 +3542,11 @@ int conv2d_winograd_fused(int variant, int slices, int dev, const float *I, cons
     int slice_steps = 0;
     const int nslices = fused_slices(fv, slices, chunk_imgs * per_img, C, Kf, state(dev).num_cu, &leftover, &slice_steps);
     const size_t tile_floats = (size_t)32 * fv.fm * 32 * fv.fn * 4;  // four outputs per filter and block
+    // The pixels come in 16 bytes per lane where a group of four columns that starts at a multiple of four lies inside the
+    // image or outside it as a whole and is aligned in memory (image rows of a multiple of four pixels, stored as they are
+    // read, 16-byte aligned tensors), and where rows of blocks are long enough that the widened pixel rows of a tile's
+    // segments fit its 16 slots per block (at most 2 + 30 / tw segments of at most 6 slots more than they need each).
+    const bool wide = uh == 1 && uw == 1 && W % 4 == 0 && tw >= 6 && pad_left <= 4 && (uintptr_t)I % 16 == 0 && (I2 == nullptr || (uintptr_t)I2 % 16 == 0);
     const size_t partial_bytes = (size_t)nslices * leftover * tile_floats * sizeof(float);
 
     const float *U = nullptr;
@@ -3574,7 +3619,7 @@ int conv2d_winograd_fused(int variant, int slices, int dev, const float *I, cons
         const long long wgs = q.main_tiles + split_tiles * q.nslices;
         q.trace = (g_trace != nullptr && wgs <= g_trace_wgs) ? g_trace : nullptr;
         EH_TRY(prof_begin(st));
-        hipLaunchKernelGGL(fv.kernel, dim3((unsigned)wgs), dim3(256), 0, st, q);
+        hipLaunchKernelGGL(wide ? fv.kernel_wide : fv.kernel, dim3((unsigned)wgs), dim3(256), 0, st, q);
         EH_CHECK_LAUNCH();
         EH_TRY(prof_end(st));
         if (split_tiles > 0) {
@@ -3582,8 +3627,9 @@ int conv2d_winograd_fused(int variant, int slices, int dev, const float *I, cons
             EH_CHECK_LAUNCH();
         }
     }
-    if (leftover > 0) snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%s +ksplit(%lld tiles x %d), %lld blocks]", fv.name, leftover, nslices, (long long)N * per_img);
-    else snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%s, %lld blocks]", fv.name, (long long)N * per_img);
+    const char *name = wide ? fv.name_wide : fv.name;
+    if (leftover > 0) snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%s +ksplit(%lld tiles x %d), %lld blocks]", name, leftover, nslices, (long long)N * per_img);
+    else snprintf(g_last_kernel, sizeof(g_last_kernel), "winograd[%s, %lld blocks]", name, (long long)N * per_img);
     return 0;
 }
 

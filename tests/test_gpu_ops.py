@@ -358,6 +358,8 @@ WINOGRAD_CASES = [
     (2, 16, 6, 5, 24, (1, 1), None, True, False, False, False, False, (2, 2)),       # a folded UpSampling2D
     (1, 16, 6, 6, 24, (0, 0), (11, 11), False, False, False, False, False, (2, 3)),
     (4, 256, 28, 28, 256, (1, 1), None, False, True, False, True, False, None),      # a long channel sum
+    (2, 24, 11, 20, 40, (0, 0), None, True, False, False, False, False, None),       # rows of a multiple of four pixels: 16-byte pixel loads, no padding
+    (2, 16, 12, 24, 24, (1, 2), None, False, False, False, True, False, None),       # the same with two columns of padding
 ]
 
 
@@ -549,6 +551,48 @@ def test_conv2d_upsampled_2x2_form_against_oracle(hip, oracle):
     finally:
         hip.force_conv_plan(-1, 1)
         hip.uncache_conv_filters(Wd)
+
+
+def _misaligned_copy(hip, host):
+    """A device copy of `host` that starts four bytes into its allocation, i.e. not at a multiple of 16 bytes."""
+    from eddl_amd.backend import _View
+    base = hip.empty((host.size + 1,))
+    full = np.zeros(host.size + 1, np.float32)
+    full[1:] = host.ravel()
+    base.copy_from(full)
+    view = object.__new__(_View)
+    view.backend, view.ptr, view.size, view.nbytes, view.shape, view._base = hip, base.ptr + 4, host.size, host.size * 4, host.shape, base
+    return view
+
+
+@pytest.mark.parametrize("form", [(6, 1), (7, 1), (7, 3)], ids=["32x32", "64x32", "64x32-3-slices"])
+def test_conv2d_one_launch_pixel_loads_of_16_and_of_4_bytes_give_the_same_bits(hip, form):
+    """The one-launch Winograd kernel loads the pixels 16 bytes per lane where image rows are a multiple of four pixels
+    and the tensors are 16-byte aligned, 4 bytes per lane otherwise: the same input at an address that is not a multiple
+    of 16 takes the other build and gives the same output bit for bit (one and two input tensors, with and without
+    padding, rows of blocks that end inside a tile)."""
+    rng = np.random.default_rng(91)
+    for N, C, H, W, Kf, (pt, pl), two in [(3, 24, 16, 24, 40, (1, 1), False), (2, 32, 11, 20, 70, (0, 0), False), (2, 32, 12, 12, 48, (1, 1), True),
+                                          (2, 16, 12, 24, 24, (1, 2), False), (5, 64, 28, 28, 64, (1, 1), False)]:
+        Ci = C // 2 if two else C
+        a = rng.standard_normal((N, Ci, H, W), dtype=np.float32)
+        b = rng.standard_normal((N, Ci, H, W), dtype=np.float32) if two else None
+        w = hip.array((rng.standard_normal((Kf, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32))
+        P, Q = H + 2 * pt - 2, W + 2 * pl - 2
+        outs = []
+        for misaligned in (False, True):
+            da = _misaligned_copy(hip, a) if misaligned else hip.array(a)
+            db = None if not two else (_misaligned_copy(hip, b) if misaligned else hip.array(b))
+            assert (da.ptr % 16 != 0) == misaligned
+            O = hip.full((N, Kf, P, Q), 3.0)
+            hip.force_conv_plan(*form)
+            try:
+                hip.conv2D(da, w, None, O, 1, 1, pt, pl, relu=True, second=db)
+                assert "wino_fused_kernel" in hip.last_conv_kernel()
+            finally:
+                hip.force_conv_plan(-1, 1)
+            outs.append(O.numpy())
+        assert np.array_equal(outs[0], outs[1]), (N, C, H, W, Kf, pt, pl, two)
 
 
 def test_conv2d_winograd_form_only_where_it_applies_and_with_kept_filters(hip, oracle):
