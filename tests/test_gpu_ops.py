@@ -572,8 +572,13 @@ def test_conv2d_one_launch_pixel_loads_of_16_and_of_4_bytes_give_the_same_bits(h
     of 16 takes the other build and gives the same output bit for bit (one and two input tensors, with and without
     padding, rows of blocks that end inside a tile)."""
     rng = np.random.default_rng(91)
-    for N, C, H, W, Kf, (pt, pl), two in [(3, 24, 16, 24, 40, (1, 1), False), (2, 32, 11, 20, 70, (0, 0), False), (2, 32, 12, 12, 48, (1, 1), True),
-                                          (2, 16, 12, 24, 24, (1, 2), False), (5, 64, 28, 28, 64, (1, 1), False)]:
+    cases = [(3, 24, 16, 24, 40, (1, 1), False), (2, 32, 11, 20, 70, (0, 0), False), (2, 32, 12, 12, 48, (1, 1), True),
+             (2, 16, 12, 24, 24, (1, 2), False), (5, 64, 28, 28, 64, (1, 1), False)]
+    for _ in range(12):  # and random ones: rows of 12 ... 64 pixels, any height, ragged channel and filter counts
+        two = bool(rng.integers(0, 2))
+        cases.append((int(rng.integers(1, 5)), int(rng.integers(2, 36)) * (2 if two else 1), int(rng.integers(5, 40)), 4 * int(rng.integers(3, 17)),
+                      int(rng.integers(8, 140)), (int(rng.integers(0, 3)), int(rng.integers(0, 3))), two))
+    for N, C, H, W, Kf, (pt, pl), two in cases:
         Ci = C // 2 if two else C
         a = rng.standard_normal((N, Ci, H, W), dtype=np.float32)
         b = rng.standard_normal((N, Ci, H, W), dtype=np.float32) if two else None
@@ -588,7 +593,9 @@ def test_conv2d_one_launch_pixel_loads_of_16_and_of_4_bytes_give_the_same_bits(h
             hip.force_conv_plan(*form)
             try:
                 hip.conv2D(da, w, None, O, 1, 1, pt, pl, relu=True, second=db)
-                assert "wino_fused_kernel" in hip.last_conv_kernel()
+                name = hip.last_conv_kernel()
+                # (the 16-byte build where it applies - rows of at least six blocks - and only at an aligned address)
+                assert "wino_fused_kernel" in name and (",true>" in name) == (not misaligned and (Q + 1) // 2 >= 6), name
             finally:
                 hip.force_conv_plan(-1, 1)
             outs.append(O.numpy())
