@@ -233,7 +233,10 @@ int eddlhip_conv2d_fwd_noalloc(int dev, const float *I, const float *K, const fl
  * itself - raw pixels and transformed filters are staged through LDS, a lane derives its transformed operands from LDS
  * reads and additions, a workgroup keeps all 16 positions' products of its tile (32 or 64 filters x 32 blocks) in
  * registers and transforms them at the end - so no transformed input or product is ever in memory and the only
- * workspace is the transformed filters (unless registered) and the partial output tiles of a K-split plan.  Non-finite inputs: the
+ * workspace is the transformed filters (unless registered) and the partial output tiles of a K-split plan.  Where the
+ * stored image has rows of a multiple of four pixels and the input tensors are 16-byte aligned the kernel loads its pixels
+ * 16 bytes per lane (its name in eddlhip_conv2d_last_kernel then ends in ",true>"), 4 bytes per lane otherwise: same sums,
+ * same bits.  Non-finite inputs: the
  * transforms take differences of neighbouring pixels, so an infinity in the input can turn into NaN in outputs where the
  * direct form yields an infinity (all finite inputs give finite outputs as in the direct form); a caller that relies on
  * the propagation of infinities keeps the plan search off or calls eddlhip_conv2d_set_algo(9).
