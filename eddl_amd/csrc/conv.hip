@@ -2310,7 +2310,7 @@ struct FusedVariant {
     const char *name, *name_wide;
     int fm, fn, ck;
     void (*kernel)(const ConvParams);
-    void (*kernel_wide)(const ConvParams);  // the build that loads the pixels 16 bytes per lane (fused_wide_loads)
+    void (*kernel_wide)(const ConvParams);  // the build that loads the pixels 16 bytes per lane (conv2d_winograd_fused decides)
     void (*reduce)(const ConvParams);
 };
 #define FUSED(FM, FN, CK, WPE)                                                                                                       \
@@ -3545,7 +3545,7 @@ int conv2d_winograd_fused(int variant, int slices, int dev, const float *I, cons
     // The pixels come in 16 bytes per lane where a group of four columns that starts at a multiple of four lies inside the
     // image or outside it as a whole and is aligned in memory (image rows of a multiple of four pixels, stored as they are
     // read, 16-byte aligned tensors), and where rows of blocks are long enough that the widened pixel rows of a tile's
-    // segments fit its 16 slots per block (at most 2 + 30 / tw segments of at most 6 slots more than they need each).
+    // segments fit its 16 slots per block (at most 2 + 30 / tw segments, each pixel row at most 6 slots longer than it needs to be).
     const bool wide = uh == 1 && uw == 1 && W % 4 == 0 && tw >= 6 && pad_left <= 4 && (uintptr_t)I % 16 == 0 && (I2 == nullptr || (uintptr_t)I2 % 16 == 0);
     const size_t partial_bytes = (size_t)nslices * leftover * tile_floats * sizeof(float);
 
